@@ -1,0 +1,265 @@
+"""Tensor-level front end of libboxconv_hip.so (C ABI in include/boxconv.h).
+
+The four functions mirror the reference's pybind11 module ``box_convolution_cpp_cuda``
+(reference src/bind.cpp:29-34) in names, argument order, argument meaning and error messages
+(reference src/box_convolution_interface.cpp:19-34,153-170, src/integral_image_interface.cpp:9).
+PyTorch is used only for device memory and the current stream; all arithmetic happens in the HIP
+kernels. There is no CPU implementation here: tensors that are not on a HIP device, or a missing
+library, raise ``RuntimeError``.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_NAME = "libboxconv_hip.so"
+LIB_PATH = os.path.join(_HERE, LIB_NAME)
+
+ABI_VERSION = 1
+
+_lib = None
+
+_vp, _i, _i64, _sz, _f, _d = (ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_size_t,
+                              ctypes.c_float, ctypes.c_double)
+
+# name -> (restype, argtypes); kept in step with include/boxconv.h
+_SIGNATURES = {
+    "boxconv_abi_version": (_i, []),
+    "boxconv_last_error": (ctypes.c_char_p, []),
+    "boxconv_integral_image_workspace_bytes": (_sz, [_i64, _i, _i]),
+    "boxconv_backward_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i, _i, _i]),
+}
+for _s in ("f32", "f64"):
+    _SIGNATURES["boxconv_integral_image_" + _s] = (_i, [_vp, _vp, _i64, _i, _i, _vp, _sz, _vp])
+    _SIGNATURES["boxconv_forward_" + _s] = (_i, [_vp] * 6 + [_i] * 7 + [_vp])
+    _SIGNATURES["boxconv_backward_" + _s] = (
+        _i, [_vp] * 7 + [_f, _f, _i, _i] + [_vp] * 5 + [_i] * 5 + [_vp, _sz, _vp])
+    _SIGNATURES["boxconv_clip_parameters_" + _s] = (_i, [_vp] * 4 + [_i] + [_d] * 4 + [_i, _vp])
+
+EXPORTED_SYMBOLS = tuple(sorted(_SIGNATURES))
+
+_SUFFIX = {torch.float32: "f32", torch.float64: "f64"}
+
+
+def load():
+    """Load libboxconv_hip.so once. Raises RuntimeError if it was never built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.isfile(LIB_PATH):
+        raise RuntimeError(
+            "box_convolution: %s is missing; build it with "
+            "`python box-convolutions_amd/build.py` (needs hipcc). There is no CPU fallback."
+            % LIB_PATH)
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in _SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    if lib.boxconv_abi_version() != ABI_VERSION:
+        raise RuntimeError("box_convolution: %s has ABI version %d, expected %d"
+                           % (LIB_PATH, lib.boxconv_abi_version(), ABI_VERSION))
+    _lib = lib
+    return lib
+
+
+def _check(rc, what):
+    if rc != 0:
+        msg = load().boxconv_last_error().decode("utf-8", "replace")
+        raise RuntimeError("box_convolution: %s failed (code %d): %s" % (what, rc, msg))
+
+
+def _suffix(t, what):
+    try:
+        return _SUFFIX[t.dtype]
+    except KeyError:
+        raise RuntimeError("box_convolution: %s must be float32 or float64, got %s"
+                           % (what, t.dtype)) from None
+
+
+def _require_device(t, what):
+    if not t.is_cuda:
+        raise RuntimeError(
+            "box_convolution: %s is on '%s'; this build runs on AMD GPUs only (no CPU path)"
+            % (what, t.device))
+
+
+def _stream(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _workspace(nbytes, device):
+    if nbytes == 0:
+        return None
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
+def integral_image(input):
+    """``integral_image(Tensor) -> Tensor`` (reference src/integral_image_interface.cpp:8-27)."""
+    if input.dim() < 2:
+        raise RuntimeError("integral image input must have >=2 dimensions")
+    _require_device(input, "integral image input")
+    sfx = _suffix(input, "integral image input")
+    lib = load()
+    input = input.contiguous()
+    h, w = input.shape[-2:]
+    out_shape = tuple(input.shape[:-2]) + (h + 1, w + 1)
+    output = torch.empty(out_shape, dtype=input.dtype, device=input.device)
+    if h == 0 or w == 0:
+        return output.zero_()
+    planes = input.numel() // (h * w)
+    with torch.cuda.device(input.device):
+        nbytes = lib.boxconv_integral_image_workspace_bytes(planes, h, w)
+        ws = _workspace(nbytes, input.device)
+        rc = getattr(lib, "boxconv_integral_image_" + sfx)(
+            _ptr(input), _ptr(output), planes, h, w, _ptr(ws), nbytes, _stream(input.device))
+    _check(rc, "integral_image")
+    return output
+
+
+def _check_params(x_min, x_max, y_min, y_max, in_planes, prefix):
+    if not (x_min.dim() == 2 and x_max.dim() == 2 and y_min.dim() == 2 and y_max.dim() == 2):
+        raise RuntimeError(prefix + "all parameters must have 2 dimensions")
+    if not (x_min.size(0) == x_max.size(0) == y_min.size(0) == y_max.size(0) == in_planes):
+        raise RuntimeError(
+            prefix + "all parameters must have as many rows as there are input channels")
+    if not (x_min.size(1) == x_max.size(1) == y_min.size(1) == y_max.size(1)):
+        raise RuntimeError(prefix + "all parameters must have equal number of columns")
+
+
+def _same_kind(params, like, what):
+    out = []
+    for p in params:
+        if p.device != like.device:
+            raise RuntimeError("BoxConv2d: input and parameters are on different devices")
+        if p.dtype != like.dtype:
+            raise RuntimeError("box_convolution: %s and parameters have different dtypes (%s, %s)"
+                               % (what, like.dtype, p.dtype))
+        out.append(p.detach().contiguous())
+    return out
+
+
+def box_convolution_forward(input_integrated, x_min, x_max, y_min, y_max, normalize, exact):
+    """Reference src/box_convolution_interface.cpp:13-139. Parameters are in real pixel units.
+
+    Returns ``[B, C*F, h, w]``."""
+    if input_integrated.device != x_min.device:
+        raise RuntimeError("BoxConv2d: input and parameters are on different devices")
+    _require_device(input_integrated, "input")
+    if input_integrated.dim() != 4:
+        raise RuntimeError("BoxConv2d: input must have 4 dimensions")
+    sfx = _suffix(input_integrated, "input")
+    _check_params(x_min, x_max, y_min, y_max, input_integrated.size(1), "BoxConv2d: ")
+    lib = load()
+    input_integrated = input_integrated.contiguous()
+    x_min, x_max, y_min, y_max = _same_kind((x_min, x_max, y_min, y_max), input_integrated, "input")
+    B, C, h1, w1 = input_integrated.shape
+    F = x_min.size(1)
+    h, w = h1 - 1, w1 - 1
+    if h < 1 or w < 1:
+        raise RuntimeError("BoxConv2d: integral image must be at least 2x2")
+    output = torch.empty((B, C * F, h, w), dtype=input_integrated.dtype,
+                         device=input_integrated.device)
+    if output.numel() == 0:
+        return output
+    with torch.cuda.device(input_integrated.device):
+        rc = getattr(lib, "boxconv_forward_" + sfx)(
+            _ptr(input_integrated), _ptr(x_min), _ptr(x_max), _ptr(y_min), _ptr(y_max),
+            _ptr(output), B, C, F, h, w, int(bool(normalize)), int(bool(exact)),
+            _stream(output.device))
+    _check(rc, "box_convolution_forward")
+    return output
+
+
+def box_convolution_backward(input_integrated, x_min, x_max, y_min, y_max, grad_output, output,
+                             reparametrization_h, reparametrization_w, normalize, exact,
+                             input_needs_grad, x_min_needs_grad, x_max_needs_grad,
+                             y_min_needs_grad, y_max_needs_grad):
+    """Reference src/box_convolution_interface.cpp:141-395.
+
+    Returns ``[grad_input, grad_x_min, grad_x_max, grad_y_min, grad_y_max]`` with ``None`` for a
+    gradient that was not requested. ``output`` (the saved forward result) may be ``None``."""
+    _require_device(grad_output, "grad_output")
+    if grad_output.dim() != 4:
+        raise RuntimeError("grad_output for box_convolution must have 4 dimensions")
+    if input_integrated.dim() != 4:
+        raise RuntimeError("BoxConv2d: input must have 4 dimensions")
+    B, C, h1, w1 = input_integrated.shape
+    h, w = h1 - 1, w1 - 1
+    _check_params(x_min, x_max, y_min, y_max, C, "all box conv parameters: ")
+    F = x_min.size(1)
+    if tuple(grad_output.shape) != (B, C * F, h, w):
+        raise RuntimeError("box_convolution: sizes of grad_output and input_integrated don't match")
+    sfx = _suffix(grad_output, "grad_output")
+    if input_integrated.device != grad_output.device or input_integrated.dtype != grad_output.dtype:
+        raise RuntimeError("box_convolution: grad_output and input_integrated differ in device or dtype")
+    lib = load()
+    grad_output = grad_output.contiguous()
+    input_integrated = input_integrated.contiguous()
+    x_min, x_max, y_min, y_max = _same_kind((x_min, x_max, y_min, y_max), grad_output, "grad_output")
+    dev, dt = grad_output.device, grad_output.dtype
+    needs_p = (x_min_needs_grad, x_max_needs_grad, y_min_needs_grad, y_max_needs_grad)
+
+    grad_input = None
+    if input_needs_grad:
+        grad_input = (torch.empty if F > 0 else torch.zeros)((B, C, h, w), dtype=dt, device=dev)
+    grads = [torch.empty((C, F), dtype=dt, device=dev) if n else None for n in needs_p]
+    want_input = input_needs_grad and grad_input.numel() > 0 and F > 0
+    want_params = any(needs_p) and C * F > 0
+    if want_input or want_params:
+        with torch.cuda.device(dev):
+            nbytes = lib.boxconv_backward_workspace_bytes(
+                B, C, F, h, w, grad_output.element_size(), int(want_input), int(want_params))
+            ws = _workspace(nbytes, dev)
+            rc = getattr(lib, "boxconv_backward_" + sfx)(
+                _ptr(input_integrated), _ptr(x_min), _ptr(x_max), _ptr(y_min), _ptr(y_max),
+                _ptr(grad_output), _ptr(output) if output is not None and output.numel() else None,
+                float(reparametrization_h), float(reparametrization_w), int(bool(normalize)),
+                int(bool(exact)), _ptr(grad_input) if want_input else None,
+                *[_ptr(g) if want_params else None for g in grads],
+                B, C, F, h, w, _ptr(ws), nbytes, _stream(dev))
+        _check(rc, "box_convolution_backward")
+    return [grad_input] + grads
+
+
+def clip_parameters(x_min, x_max, y_min, y_max, reparametrization_h, reparametrization_w,
+                    max_input_h, max_input_w, exact):
+    """In place on the stored parameters (reference src/box_convolution_interface.cpp:397-415).
+
+    Parameters that live in host memory are clipped by the same HIP kernel through a device copy,
+    so that ``BoxConv2d(...).eval()`` works before the module is moved to the GPU."""
+    if not x_min.is_contiguous():
+        raise RuntimeError("x_min must be contiguous")
+    params = (x_min, x_max, y_min, y_max)
+    for p in params[1:]:
+        if (p.shape != x_min.shape or p.dtype != x_min.dtype or p.device != x_min.device
+                or not p.is_contiguous()):
+            raise RuntimeError("box_convolution: clip_parameters needs four contiguous tensors of "
+                               "one shape, dtype and device")
+    sfx = _suffix(x_min, "parameters")
+    n = x_min.numel()
+    if n == 0:
+        return
+    lib = load()
+    if not x_min.is_cuda:
+        if not torch.cuda.is_available():
+            raise RuntimeError("box_convolution: parameters are on '%s' and no AMD GPU is "
+                               "available; there is no CPU path" % x_min.device)
+        with torch.no_grad():
+            staged = [p.detach().to("cuda") for p in params]
+            clip_parameters(*staged, reparametrization_h, reparametrization_w, max_input_h,
+                            max_input_w, exact)
+            for p, s in zip(params, staged):
+                p.detach().copy_(s)
+        return
+    with torch.cuda.device(x_min.device):
+        rc = getattr(lib, "boxconv_clip_parameters_" + sfx)(
+            _ptr(x_min), _ptr(x_max), _ptr(y_min), _ptr(y_max), n,
+            float(reparametrization_h), float(reparametrization_w), float(max_input_h),
+            float(max_input_w), int(bool(exact)), _stream(x_min.device))
+    _check(rc, "clip_parameters")

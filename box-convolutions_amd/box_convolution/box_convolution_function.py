@@ -1,0 +1,69 @@
+"""Autograd glue: ``reparametrize`` and ``BoxConvolutionFunction``.
+
+Same public surface as the reference's box_convolution/box_convolution_function.py:5-65; the
+native calls go to the HIP library instead of ``box_convolution_cpp_cuda``.
+"""
+import torch
+
+from . import _native
+
+
+def reparametrize(
+        x_min, x_max, y_min, y_max, reparametrization_h, reparametrization_w,
+        inplace=False, inverse=False):
+    """Convert box bounds between stored units (about [-1, 1], friendly to SGD step sizes) and
+    real pixel units. ``inverse=False``: real -> stored (divide); ``inverse=True``: stored -> real.
+
+    With ``inplace`` the four tensors are modified and nothing is returned; otherwise four new
+    tensors are returned. Never recorded by autograd.
+    (reference box_convolution_function.py:5-27)
+    """
+    scale_h = reparametrization_h if inverse else (1 / reparametrization_h)
+    scale_w = reparametrization_w if inverse else (1 / reparametrization_w)
+
+    with torch.no_grad():
+        if inplace:
+            x_min *= scale_h
+            x_max *= scale_h
+            y_min *= scale_w
+            y_max *= scale_w
+            return None
+        return x_min * scale_h, x_max * scale_h, y_min * scale_w, y_max * scale_w
+
+
+class BoxConvolutionFunction(torch.autograd.Function):
+    """``apply(input, x_min, x_max, y_min, y_max, reparametrization_h, reparametrization_w,
+    normalize, exact) -> output [B, C*F, h, w]``; parameters in stored units.
+    (reference box_convolution_function.py:30-65)
+    """
+
+    @staticmethod
+    def forward(ctx, input, x_min, x_max, y_min, y_max,
+                reparametrization_h, reparametrization_w, normalize, exact):
+        ctx.normalize = normalize
+        ctx.reparametrization_h = reparametrization_h
+        ctx.reparametrization_w = reparametrization_w
+        ctx.exact = exact
+
+        x_min, x_max, y_min, y_max = reparametrize(
+            x_min, x_max, y_min, y_max, reparametrization_h, reparametrization_w, inverse=True)
+
+        input_integrated = _native.integral_image(input)
+        output = _native.box_convolution_forward(
+            input_integrated, x_min, x_max, y_min, y_max, normalize, exact)
+
+        # The saved forward output of the reference is not kept: the backward kernels rebuild the
+        # one sum that needs it from the integral image.
+        ctx.save_for_backward(input_integrated, x_min, x_max, y_min, y_max)
+        return output
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, grad_output):
+        input_integrated, x_min, x_max, y_min, y_max = ctx.saved_tensors
+        grads = _native.box_convolution_backward(
+            input_integrated, x_min, x_max, y_min, y_max, grad_output, None,
+            ctx.reparametrization_h, ctx.reparametrization_w,
+            ctx.normalize, ctx.exact, *ctx.needs_input_grad[:5])
+        # no gradients for reparametrization_h, reparametrization_w, normalize, exact
+        return tuple(grads) + (None,) * 4

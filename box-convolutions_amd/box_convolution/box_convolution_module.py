@@ -1,0 +1,107 @@
+"""``BoxConv2d``: depthwise convolution with learnable box (rectangular averaging) kernels.
+
+Drop-in for the reference's box_convolution/box_convolution_module.py:6-222: same constructor,
+attributes, parameter names/shapes (so ``state_dict``s interchange) and methods.
+"""
+import random
+
+import torch
+
+from . import _native
+from .box_convolution_function import BoxConvolutionFunction, reparametrize
+
+
+class BoxConv2d(torch.nn.Module):
+    """Convolves every input channel with ``num_filters`` box filters whose four bounds are
+    learnable real numbers.
+
+    Input ``[B, in_planes, h, w]`` -> output ``[B, in_planes*num_filters, h, w]`` (output channel
+    ``c*num_filters + f``). ``x_*`` bounds run along the height axis, ``y_*`` along the width.
+
+    Arguments:
+        in_planes, num_filters: channels in, filters per channel.
+        max_input_h, max_input_w: expected largest input size; only used to initialise the boxes
+            and to clip boxes that grew or drifted too far (``_clip_parameters``).
+        reparametrization_factor: parameters are stored divided by
+            ``max_input_{h,w} * reparametrization_factor`` so that plain SGD step sizes work.
+        stride_h, stride_w: must be 1.
+        normalize: ``True`` -> box averages, ``False`` -> box sums.
+
+    Attribute ``exact`` (default ``True``): ``False`` rounds the bounds towards the smaller box
+    before filtering (cheaper, no fractional borders).
+    """
+
+    def __init__(self, in_planes, num_filters, max_input_h, max_input_w,
+                 reparametrization_factor=8, stride_h=1, stride_w=1, normalize=True):
+        super().__init__()
+        self.in_planes = in_planes
+        self.num_filters = num_filters
+        self.max_input_h, self.max_input_w = max_input_h, max_input_w
+        self.reparametrization_h = max_input_h * reparametrization_factor
+        self.reparametrization_w = max_input_w * reparametrization_factor
+        self.stride_h, self.stride_w = stride_h, stride_w
+        assert stride_h == 1 and stride_w == 1, 'Sorry, strides are NYI'
+        self.normalize = normalize
+        self.exact = True
+
+        self.x_min, self.x_max, self.y_min, self.y_max = \
+            (torch.nn.Parameter(torch.empty(in_planes, num_filters)) for _ in range(4))
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        """Random boxes centred inside the middle of the image, drawn from Python's global
+        ``random`` in the reference's order (per box: centre_h, centre_w, height, width;
+        reference box_convolution_module.py:69-97), then stored in reparametrized units."""
+        max_h, max_w = self.max_input_h, self.max_input_w
+        min_h, min_w = 2, 2
+        lim_h, lim_w = max_h * 2 / 4.8, max_w * 2 / 4.8
+        rows = [[], [], [], []]
+        for _ in range(self.in_planes * self.num_filters):
+            center_h = random.uniform(-lim_h + 1 + min_h / 2, lim_h - 1 - min_h / 2)
+            center_w = random.uniform(-lim_w + 1 + min_w / 2, lim_w - 1 - min_w / 2)
+            height = 2 * random.uniform(
+                min_h / 2, min((lim_h - 1) - center_h, center_h - (-lim_h + 1)))
+            width = 2 * random.uniform(
+                min_w / 2, min((lim_w - 1) - center_w, center_w - (-lim_w + 1)))
+            rows[0].append((center_h - height / 2) * 1.5)
+            rows[1].append((center_h + height / 2) * 1.5)
+            rows[2].append((center_w - width / 2) * 1.5)
+            rows[3].append((center_w + width / 2) * 1.5)
+
+        with torch.no_grad():
+            for param, values in zip((self.x_min, self.x_max, self.y_min, self.y_max), rows):
+                host = torch.tensor(values, dtype=torch.float64).to(param.dtype)
+                param.copy_(host.view(self.in_planes, self.num_filters))
+
+        reparametrize(
+            self.x_min, self.x_max, self.y_min, self.y_max,
+            self.reparametrization_h, self.reparametrization_w, inplace=True)
+
+    def get_actual_parameters(self):
+        """The four bounds in real pixel units (new tensors)."""
+        return reparametrize(
+            self.x_min, self.x_max, self.y_min, self.y_max,
+            self.reparametrization_h, self.reparametrization_w, inplace=False, inverse=True)
+
+    def _clip_parameters(self):
+        """Projection step after an optimizer update: keep every box within
+        ``[-(max_input+1), max_input-1]`` pixels and at least ~1 pixel (2 when ``not exact``)
+        thick. In place, outside autograd. (reference box_convolution_module.py:195-206)"""
+        _native.clip_parameters(
+            self.x_min, self.x_max, self.y_min, self.y_max,
+            self.reparametrization_h, self.reparametrization_w,
+            self.max_input_h, self.max_input_w, self.exact)
+
+    def train(self, mode=True):
+        self.training = mode
+        if mode is False:
+            self._clip_parameters()
+        return self
+
+    def forward(self, input):
+        if self.training:
+            self._clip_parameters()
+
+        return BoxConvolutionFunction.apply(
+            input, self.x_min, self.x_max, self.y_min, self.y_max,
+            self.reparametrization_h, self.reparametrization_w, self.normalize, self.exact)

@@ -1,0 +1,255 @@
+// extern "C" entry points of libboxconv_hip.so (declared in include/boxconv.h): argument checks on
+// the host, workspace carving, kernel launches. No torch types, no allocation, no synchronisation.
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "../../include/boxconv.h"
+#include "boxconv_host.hpp"
+
+namespace {
+
+thread_local char g_error[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    std::vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int hip_result(hipError_t e, const char* what) {
+    if (e == hipSuccess) return 0;
+    return fail(static_cast<int>(e), "%s: %s", what, hipGetErrorString(e));
+}
+
+constexpr int64_t kMaxElems = (int64_t(1) << 31) - 1;
+
+size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+int check_dims(int batch, int in_planes, int num_filters, int h, int w) {
+    if (batch < 0 || in_planes < 0 || num_filters < 0 || h < 1 || w < 1)
+        return fail(BOXCONV_E_INVALID_ARGUMENT,
+                    "invalid sizes: batch=%d in_planes=%d num_filters=%d h=%d w=%d", batch,
+                    in_planes, num_filters, h, w);
+    const int64_t big = static_cast<int64_t>(batch) * in_planes * std::max(num_filters, 1) *
+                        static_cast<int64_t>(h + 1) * (w + 1);
+    if (big > kMaxElems)
+        return fail(BOXCONV_E_TOO_LARGE, "tensor of %lld elements exceeds 2^31-1",
+                    static_cast<long long>(big));
+    return 0;
+}
+
+struct BackwardLayout {
+    size_t gint_off, aux_off, acc_off, total;
+};
+
+BackwardLayout backward_layout(int batch, int in_planes, int num_filters, int h, int w,
+                               int elem_size, bool need_input, bool need_params) {
+    BackwardLayout L{};
+    size_t off = 0;
+    L.gint_off = off;
+    if (need_input) {
+        const int64_t planes = static_cast<int64_t>(batch) * in_planes * num_filters;
+        off += align_up(static_cast<size_t>(planes) * (h + 1) * (w + 1) * elem_size, 256);
+        L.aux_off = off;
+        off += align_up(static_cast<size_t>(boxconv::plan_integral(planes, h, w).aux_doubles) * 8, 256);
+    } else {
+        L.aux_off = off;
+    }
+    L.acc_off = off;
+    if (need_params) off += align_up(static_cast<size_t>(in_planes) * num_filters * 5 * 8, 256);
+    L.total = off;
+    return L;
+}
+
+template <class T>
+int integral_image_impl(const T* in, T* out, int64_t planes, int h, int w, void* workspace,
+                        size_t workspace_bytes, void* stream) {
+    if (planes < 0 || h < 1 || w < 1)
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "integral image: invalid sizes planes=%lld h=%d w=%d",
+                    static_cast<long long>(planes), h, w);
+    if (planes == 0) return 0;
+    if (in == nullptr || out == nullptr)
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "integral image: null tensor pointer");
+    if (planes * static_cast<int64_t>(h + 1) * (w + 1) > kMaxElems)
+        return fail(BOXCONV_E_TOO_LARGE, "integral image: output exceeds 2^31-1 elements");
+    const size_t need = boxconv_integral_image_workspace_bytes(planes, h, w);
+    if (need > 0 && (workspace == nullptr || workspace_bytes < need ||
+                     reinterpret_cast<uintptr_t>(workspace) % 8 != 0))
+        return fail(BOXCONV_E_WORKSPACE, "integral image: workspace of %zu bytes (8-byte aligned) required, got %zu",
+                    need, workspace_bytes);
+    return hip_result(boxconv::integral_image_launch<T>(in, out, planes, h, w,
+                                                        static_cast<double*>(workspace),
+                                                        static_cast<hipStream_t>(stream)),
+                      "integral image launch");
+}
+
+template <class T>
+int forward_impl(const T* integ, const T* x_min, const T* x_max, const T* y_min, const T* y_max,
+                 T* output, int batch, int in_planes, int num_filters, int h, int w,
+                 int normalize, int exact, void* stream) {
+    if (int rc = check_dims(batch, in_planes, num_filters, h, w)) return rc;
+    if (static_cast<int64_t>(batch) * in_planes * num_filters == 0) return 0;
+    if (!integ || !x_min || !x_max || !y_min || !y_max || !output)
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "forward: null tensor pointer");
+    boxconv::Dims d{batch, in_planes, num_filters, h, w};
+    boxconv::BoxParams<T> prm{x_min, x_max, y_min, y_max};
+    return hip_result(boxconv::forward_launch<T>(integ, prm, output, d, normalize != 0, exact != 0,
+                                                 static_cast<hipStream_t>(stream)),
+                      "forward launch");
+}
+
+template <class T>
+int backward_impl(const T* integ, const T* x_min, const T* x_max, const T* y_min, const T* y_max,
+                  const T* grad_output, const T* /*output*/, float reparam_h, float reparam_w,
+                  int normalize, int exact, T* grad_input, T* gx_min, T* gx_max, T* gy_min,
+                  T* gy_max, int batch, int in_planes, int num_filters, int h, int w,
+                  void* workspace, size_t workspace_bytes, void* stream) {
+    if (int rc = check_dims(batch, in_planes, num_filters, h, w)) return rc;
+    const bool need_input = grad_input != nullptr;
+    const bool need_params = gx_min || gx_max || gy_min || gy_max;
+    if (!need_input && !need_params) return 0;
+    if (!x_min || !x_max || !y_min || !y_max)
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "backward: null parameter pointer");
+    const int64_t nout = static_cast<int64_t>(batch) * in_planes * num_filters;
+    if (nout > 0 && (!grad_output || (need_params && !integ)))
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "backward: null tensor pointer");
+    const BackwardLayout L = backward_layout(batch, in_planes, num_filters, h, w, sizeof(T),
+                                             need_input, need_params);
+    if (L.total > 0 && (workspace == nullptr || workspace_bytes < L.total ||
+                        reinterpret_cast<uintptr_t>(workspace) % 256 != 0))
+        return fail(BOXCONV_E_WORKSPACE, "backward: workspace of %zu bytes (256-byte aligned) required, got %zu",
+                    L.total, workspace_bytes);
+
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    unsigned char* ws = static_cast<unsigned char*>(workspace);
+    boxconv::Dims d{batch, in_planes, num_filters, h, w};
+    boxconv::BoxParams<T> prm{x_min, x_max, y_min, y_max};
+
+    if (need_params) {
+        if (int rc = hip_result(boxconv::grad_params_launch<T>(
+                integ, grad_output, prm, reinterpret_cast<double*>(ws + L.acc_off), gx_min, gx_max,
+                gy_min, gy_max, d, reparam_h, reparam_w, normalize != 0, exact != 0, s),
+                "parameter-gradient launch"))
+            return rc;
+    }
+    if (need_input) {
+        if (nout == 0) {
+            // no filters: the sum over an empty set of filters is zero
+            return fail(BOXCONV_E_INVALID_ARGUMENT, "backward: grad_input requested with zero filters");
+        }
+        T* gint = reinterpret_cast<T*>(ws + L.gint_off);
+        if (int rc = hip_result(boxconv::integral_image_launch<T>(
+                grad_output, gint, nout, h, w, reinterpret_cast<double*>(ws + L.aux_off), s),
+                "grad_output integral image launch"))
+            return rc;
+        if (int rc = hip_result(boxconv::grad_input_launch<T>(gint, prm, grad_input, d,
+                                                              normalize != 0, exact != 0, s),
+                                "input-gradient launch"))
+            return rc;
+    }
+    return 0;
+}
+
+template <class T>
+int clip_impl(T* x_min, T* x_max, T* y_min, T* y_max, int n, double reparam_h, double reparam_w,
+              double max_h, double max_w, int exact, void* stream) {
+    if (n < 0) return fail(BOXCONV_E_INVALID_ARGUMENT, "clip: negative element count");
+    if (n == 0) return 0;
+    if (!x_min || !x_max || !y_min || !y_max)
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "clip: null parameter pointer");
+    if (!(reparam_h != 0.0) || !(reparam_w != 0.0))
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "clip: reparametrization factor is zero");
+    return hip_result(boxconv::clip_launch<T>(x_min, x_max, y_min, y_max, n, reparam_h, reparam_w,
+                                              max_h, max_w, exact != 0,
+                                              static_cast<hipStream_t>(stream)),
+                      "clip launch");
+}
+
+}  // namespace
+
+extern "C" {
+
+int boxconv_abi_version(void) { return BOXCONV_ABI_VERSION; }
+
+const char* boxconv_last_error(void) { return g_error; }
+
+size_t boxconv_integral_image_workspace_bytes(int64_t planes, int h, int w) {
+    if (planes <= 0 || h < 1 || w < 1) return 0;
+    return static_cast<size_t>(boxconv::plan_integral(planes, h, w).aux_doubles) * 8;
+}
+
+int boxconv_integral_image_f32(const float* in, float* out, int64_t planes, int h, int w,
+                               void* workspace, size_t workspace_bytes, void* stream) {
+    return integral_image_impl<float>(in, out, planes, h, w, workspace, workspace_bytes, stream);
+}
+int boxconv_integral_image_f64(const double* in, double* out, int64_t planes, int h, int w,
+                               void* workspace, size_t workspace_bytes, void* stream) {
+    return integral_image_impl<double>(in, out, planes, h, w, workspace, workspace_bytes, stream);
+}
+
+int boxconv_forward_f32(const float* input_integrated, const float* x_min, const float* x_max,
+                        const float* y_min, const float* y_max, float* output, int batch,
+                        int in_planes, int num_filters, int h, int w, int normalize, int exact,
+                        void* stream) {
+    return forward_impl<float>(input_integrated, x_min, x_max, y_min, y_max, output, batch,
+                               in_planes, num_filters, h, w, normalize, exact, stream);
+}
+int boxconv_forward_f64(const double* input_integrated, const double* x_min, const double* x_max,
+                        const double* y_min, const double* y_max, double* output, int batch,
+                        int in_planes, int num_filters, int h, int w, int normalize, int exact,
+                        void* stream) {
+    return forward_impl<double>(input_integrated, x_min, x_max, y_min, y_max, output, batch,
+                                in_planes, num_filters, h, w, normalize, exact, stream);
+}
+
+size_t boxconv_backward_workspace_bytes(int batch, int in_planes, int num_filters, int h, int w,
+                                        int elem_size, int input_needs_grad,
+                                        int params_need_grad) {
+    if (batch < 0 || in_planes < 0 || num_filters < 0 || h < 1 || w < 1) return 0;
+    if (elem_size != 4 && elem_size != 8) return 0;
+    return backward_layout(batch, in_planes, num_filters, h, w, elem_size, input_needs_grad != 0,
+                           params_need_grad != 0).total;
+}
+
+int boxconv_backward_f32(const float* input_integrated, const float* x_min, const float* x_max,
+                         const float* y_min, const float* y_max, const float* grad_output,
+                         const float* output, float reparametrization_h,
+                         float reparametrization_w, int normalize, int exact, float* grad_input,
+                         float* grad_x_min, float* grad_x_max, float* grad_y_min,
+                         float* grad_y_max, int batch, int in_planes, int num_filters, int h,
+                         int w, void* workspace, size_t workspace_bytes, void* stream) {
+    return backward_impl<float>(input_integrated, x_min, x_max, y_min, y_max, grad_output, output,
+                                reparametrization_h, reparametrization_w, normalize, exact,
+                                grad_input, grad_x_min, grad_x_max, grad_y_min, grad_y_max, batch,
+                                in_planes, num_filters, h, w, workspace, workspace_bytes, stream);
+}
+int boxconv_backward_f64(const double* input_integrated, const double* x_min, const double* x_max,
+                         const double* y_min, const double* y_max, const double* grad_output,
+                         const double* output, float reparametrization_h,
+                         float reparametrization_w, int normalize, int exact, double* grad_input,
+                         double* grad_x_min, double* grad_x_max, double* grad_y_min,
+                         double* grad_y_max, int batch, int in_planes, int num_filters, int h,
+                         int w, void* workspace, size_t workspace_bytes, void* stream) {
+    return backward_impl<double>(input_integrated, x_min, x_max, y_min, y_max, grad_output, output,
+                                 reparametrization_h, reparametrization_w, normalize, exact,
+                                 grad_input, grad_x_min, grad_x_max, grad_y_min, grad_y_max, batch,
+                                 in_planes, num_filters, h, w, workspace, workspace_bytes, stream);
+}
+
+int boxconv_clip_parameters_f32(float* x_min, float* x_max, float* y_min, float* y_max, int n,
+                                double reparametrization_h, double reparametrization_w,
+                                double max_input_h, double max_input_w, int exact, void* stream) {
+    return clip_impl<float>(x_min, x_max, y_min, y_max, n, reparametrization_h,
+                            reparametrization_w, max_input_h, max_input_w, exact, stream);
+}
+int boxconv_clip_parameters_f64(double* x_min, double* x_max, double* y_min, double* y_max, int n,
+                                double reparametrization_h, double reparametrization_w,
+                                double max_input_h, double max_input_w, int exact, void* stream) {
+    return clip_impl<double>(x_min, x_max, y_min, y_max, n, reparametrization_h,
+                             reparametrization_w, max_input_h, max_input_w, exact, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,286 @@
+// Integral image (2-D inclusive prefix sum with a zero first row and column) for gfx950.
+//
+// Replaces reference src/integral_image.cpp:8-39 (CPU) / src/integral_image_cuda.cu:67-173.
+// out[p][r+1][c+1] = sum_{i<=r, j<=c} in[p][i][j], out[p][0][*] = out[p][*][0] = 0.
+//
+// Decomposition. A plane is cut into horizontal bands of R rows; one workgroup owns one band at
+// full width, so the only dependency between workgroups is "everything above my band", a vector
+// of w column sums. That dependency is resolved without any inter-workgroup waiting by three
+// stream-ordered launches:
+//   1. band_colsum_kernel  : column sums of every band but the last  -> aux[p][band][c]
+//   2. band_prefix_kernel  : running sum of aux over bands (in place) -> sum of all bands above
+//   3. band_scan_kernel    : per band, rows top to bottom: column accumulators (registers) +=
+//                            input row, then a row-direction prefix of the accumulators.
+// With a single band (tall enough grid without cutting) only launch 3 runs.
+//
+// Arithmetic. All sums are carried in double and rounded once on store, so every stored value
+// is the correctly rounded exact sum (the CPU reference carries row sums in double as well but
+// rounds the column carry every row; this is at least as accurate).
+//
+// Memory. Loads are 4 consecutive elements per lane (16 B for float, coalesced across the wave).
+// The output pitch w+1 is odd, so results are staged through LDS and written as consecutive
+// dwords per lane (256 B contiguous per wave instruction).
+
+#include "boxconv_device.hpp"
+#include "boxconv_host.hpp"
+
+namespace boxconv {
+
+namespace {
+
+template <class T>
+struct alignas(4 * sizeof(T)) Vec4 { T v[4]; };
+
+// ---- pass 1 -----------------------------------------------------------------------------------
+template <class T>
+__global__ void __launch_bounds__(256)
+band_colsum_kernel(const T* __restrict__ in, double* __restrict__ aux, int h, int w, int nb,
+                   int R) {
+    const int64_t blk = blockIdx.x;                 // p * (nb-1) + band, band < nb-1
+    const int band = static_cast<int>(blk % (nb - 1));
+    const int64_t p = blk / (nb - 1);
+    const int r0 = band * R;
+    const int r1 = min(h, r0 + R);
+    const T* src = in + p * static_cast<int64_t>(h) * w;
+    double* dst = aux + blk * static_cast<int64_t>(w);
+    for (int c = threadIdx.x; c < w; c += blockDim.x) {
+        double a0 = 0, a1 = 0, a2 = 0, a3 = 0;
+        int r = r0;
+        for (; r + 3 < r1; r += 4) {
+            const T x0 = src[static_cast<int64_t>(r) * w + c];
+            const T x1 = src[static_cast<int64_t>(r + 1) * w + c];
+            const T x2 = src[static_cast<int64_t>(r + 2) * w + c];
+            const T x3 = src[static_cast<int64_t>(r + 3) * w + c];
+            a0 += x0; a1 += x1; a2 += x2; a3 += x3;
+        }
+        for (; r < r1; ++r) a0 += src[static_cast<int64_t>(r) * w + c];
+        dst[c] = (a0 + a1) + (a2 + a3);
+    }
+}
+
+// ---- pass 2 -----------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+band_prefix_kernel(double* __restrict__ aux, int64_t planes, int w, int nb) {
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= planes * w) return;
+    const int64_t p = idx / w;
+    const int c = static_cast<int>(idx % w);
+    double* col = aux + p * static_cast<int64_t>(nb - 1) * w + c;
+    double run = col[0];
+    for (int k = 1; k < nb - 1; ++k) {
+        run += col[static_cast<int64_t>(k) * w];
+        col[static_cast<int64_t>(k) * w] = run;
+    }
+}
+
+// ---- pass 3 -----------------------------------------------------------------------------------
+// WAVES*64 threads; a "chunk" is WAVES*256 consecutive columns (4 per lane); M chunks cover the
+// tile of columns this launch handles per row; RB rows are in flight together.
+template <class T, int WAVES, int M, int RB, bool VEC>
+__global__ void __launch_bounds__(WAVES * 64)
+band_scan_kernel(const T* __restrict__ in, T* __restrict__ out, const double* __restrict__ aux,
+                 int h, int w, int nb, int R) {
+    constexpr int NT = WAVES * 64;
+    constexpr int CW = NT * 4;          // columns per chunk
+    constexpr int TW = CW * M;          // columns per tile
+
+    __shared__ double wave_tot[RB][M][WAVES];
+    __shared__ __align__(32) T stage[RB][TW];
+    __shared__ double row_carry[256];   // prefix of each band row up to the current tile; R <= 256
+
+    const int64_t blk = blockIdx.x;     // p * nb + band
+    const int band = static_cast<int>(blk % nb);
+    const int64_t p = blk / nb;
+    const int r0 = band * R;
+    const int r1 = min(h, r0 + R);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int64_t W1 = static_cast<int64_t>(w) + 1;
+
+    const T* src = in + p * static_cast<int64_t>(h) * w;
+    T* dst = out + p * static_cast<int64_t>(h + 1) * W1;
+    const double* above = (band > 0)
+        ? aux + (p * static_cast<int64_t>(nb - 1) + (band - 1)) * static_cast<int64_t>(w)
+        : nullptr;
+
+    if (band == 0)
+        for (int c = tid; c <= w; c += NT) dst[c] = T(0);
+    for (int r = tid; r < r1 - r0; r += NT) row_carry[r] = 0.0;
+    __syncthreads();
+
+    for (int c0 = 0; c0 < w; c0 += TW) {
+        // column accumulators for this tile start at the sum of all bands above
+        double colacc[M][4];
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int c = c0 + m * CW + 4 * tid + v;
+                colacc[m][v] = (above != nullptr && c < w) ? above[c] : 0.0;
+            }
+
+        for (int rbase = r0; rbase < r1; rbase += RB) {
+            // -- issue all loads of the batch
+            T x[RB][M][4];
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+                const int row = rbase + rb;
+#pragma unroll
+                for (int m = 0; m < M; ++m) {
+                    const int c = c0 + m * CW + 4 * tid;
+                    if (VEC) {
+                        Vec4<T> q = {{T(0), T(0), T(0), T(0)}};
+                        if (row < r1 && c < w)
+                            q = *reinterpret_cast<const Vec4<T>*>(src + static_cast<int64_t>(row) * w + c);
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) x[rb][m][v] = q.v[v];
+                    } else {
+#pragma unroll
+                        for (int v = 0; v < 4; ++v)
+                            x[rb][m][v] = (row < r1 && c + v < w)
+                                ? src[static_cast<int64_t>(row) * w + c + v] : T(0);
+                    }
+                }
+            }
+
+            // -- accumulate down the rows, prefix inside the lane, scan across the wave
+            double pre[RB][M][4];
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+                for (int m = 0; m < M; ++m) {
+                    double run = 0.0;
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        colacc[m][v] += static_cast<double>(x[rb][m][v]);
+                        run += colacc[m][v];
+                        pre[rb][m][v] = run;            // inclusive within the lane
+                    }
+                    const double incl = wave_inclusive_scan(run);
+                    const double excl = incl - run;     // lanes to the left, this wave
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) pre[rb][m][v] += excl;
+                    if (lane == 63) wave_tot[rb][m][wave] = incl;
+                }
+            __syncthreads();
+
+            // -- add waves/chunks to the left and the tiles to the left; stage as T
+            double tile_end[RB];
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+                const int row = rbase + rb;
+                double left = (row < r1) ? row_carry[row - r0] : 0.0;
+#pragma unroll
+                for (int m = 0; m < M; ++m) {
+                    double mine = left;
+#pragma unroll
+                    for (int wv = 0; wv < WAVES; ++wv) {
+                        const double t = wave_tot[rb][m][wv];
+                        if (wv < wave) mine += t;
+                        left += t;
+                    }
+                    Vec4<T> q;
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) q.v[v] = static_cast<T>(mine + pre[rb][m][v]);
+                    *reinterpret_cast<Vec4<T>*>(&stage[rb][m * CW + 4 * tid]) = q;
+                }
+                tile_end[rb] = left;        // row prefix through the end of this tile
+            }
+            __syncthreads();
+            if (tid == 0 && c0 + TW < w) {
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb)
+                    if (rbase + rb < r1) row_carry[rbase + rb - r0] = tile_end[rb];
+            }
+
+            // -- coalesced stores: lane-consecutive dwords into the (w+1)-pitched output
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+                const int row = rbase + rb;
+                if (row < r1) {
+                    T* orow = dst + static_cast<int64_t>(row + 1) * W1;
+                    const int lim = min(TW, w - c0);
+                    for (int i = tid; i < lim; i += NT) orow[c0 + i + 1] = stage[rb][i];
+                    if (c0 == 0 && tid == 0) orow[0] = T(0);
+                }
+            }
+            __syncthreads();
+        }
+    }
+}
+
+template <class T>
+bool aligned_for_vec4(const T* p, int w) {
+    return (w % 4 == 0) && (reinterpret_cast<uintptr_t>(p) % (4 * sizeof(T)) == 0);
+}
+
+template <class T, int WAVES, int M, int RB>
+hipError_t launch_scan(const T* in, T* out, const double* aux, int64_t planes, int h, int w,
+                       int nb, int R, hipStream_t stream) {
+    const dim3 grid(static_cast<unsigned>(planes * nb));
+    const dim3 block(WAVES * 64);
+    if (aligned_for_vec4(in, w))
+        hipLaunchKernelGGL((band_scan_kernel<T, WAVES, M, RB, true>), grid, block, 0, stream,
+                           in, out, aux, h, w, nb, R);
+    else
+        hipLaunchKernelGGL((band_scan_kernel<T, WAVES, M, RB, false>), grid, block, 0, stream,
+                           in, out, aux, h, w, nb, R);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+IntegralPlan plan_integral(int64_t planes, int h, int w) {
+    IntegralPlan pl;
+    // Enough workgroups to cover 256 CUs several times over, but bands no shorter than 32 rows
+    // (the per-band column-sum vector is 8 B per column, i.e. 2/R of the input bytes) and no
+    // taller than 256 (size of the per-row carry array in LDS).
+    const int64_t want = 1024;
+    int nb = static_cast<int>(std::min<int64_t>((want + planes - 1) / std::max<int64_t>(planes, 1),
+                                                std::max(1, h / 32)));
+    nb = std::max(nb, (h + 255) / 256);
+    nb = std::max(nb, 1);
+    int R = (h + nb - 1) / nb;
+    R = ((R + 3) / 4) * 4;                 // whole row batches
+    R = std::min(R, 256);
+    nb = (h + R - 1) / R;
+    pl.nb = nb;
+    pl.R = R;
+    pl.aux_doubles = (nb > 1) ? planes * static_cast<int64_t>(nb - 1) * w : 0;
+    return pl;
+}
+
+template <class T>
+hipError_t integral_image_launch(const T* in, T* out, int64_t planes, int h, int w,
+                                 double* aux, hipStream_t stream) {
+    if (planes == 0) return hipSuccess;
+    const IntegralPlan pl = plan_integral(planes, h, w);
+    const int nb = pl.nb, R = pl.R;
+    if (nb > 1) {
+        hipLaunchKernelGGL((band_colsum_kernel<T>), dim3(static_cast<unsigned>(planes * (nb - 1))),
+                           dim3(256), 0, stream, in, aux, h, w, nb, R);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        if (nb > 2) {
+            const int64_t n = planes * w;
+            hipLaunchKernelGGL(band_prefix_kernel, dim3(static_cast<unsigned>((n + 255) / 256)),
+                               dim3(256), 0, stream, aux, planes, w, nb);
+            e = hipGetLastError();
+            if (e != hipSuccess) return e;
+        }
+    }
+    // Tile width: one wave covers 256 columns per chunk, four waves 1024.
+    if (w <= 256)        return launch_scan<T, 1, 1, 4>(in, out, aux, planes, h, w, nb, R, stream);
+    else if (w <= 512)   return launch_scan<T, 2, 1, 4>(in, out, aux, planes, h, w, nb, R, stream);
+    else if (w <= 1024)  return launch_scan<T, 4, 1, 4>(in, out, aux, planes, h, w, nb, R, stream);
+    else if (w <= 2048)  return launch_scan<T, 4, 2, 2>(in, out, aux, planes, h, w, nb, R, stream);
+    else                 return launch_scan<T, 4, 4, 1>(in, out, aux, planes, h, w, nb, R, stream);
+}
+
+template hipError_t integral_image_launch<float>(const float*, float*, int64_t, int, int,
+                                                 double*, hipStream_t);
+template hipError_t integral_image_launch<double>(const double*, double*, int64_t, int, int,
+                                                  double*, hipStream_t);
+
+}  // namespace boxconv

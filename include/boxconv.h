@@ -1,0 +1,119 @@
+/* libboxconv_hip.so -- box convolution (integral-image box filters) for AMD gfx950 (MI355X).
+ *
+ * C ABI: plain pointers and sizes, no torch types. Every pointer is DEVICE memory on the current
+ * HIP device unless stated otherwise; the caller owns every buffer, including scratch. `stream`
+ * is a hipStream_t passed as void* (NULL = the null stream). All work is enqueued on that stream
+ * and the call returns without synchronising. Nothing here allocates device memory.
+ *
+ * Return value: 0 on success; a positive value is a hipError_t from a launch; negative values are
+ * BOXCONV_E_* argument errors detected before anything was launched. boxconv_last_error() gives
+ * the message of the last failure on the calling thread.
+ *
+ * The four entry-point families replace the four functions of the reference's native module
+ * `box_convolution_cpp_cuda` (reference src/bind.cpp:29-34); _f32 / _f64 select the element type
+ * (the reference dispatches on the tensor dtype).
+ *
+ * Layouts (all contiguous, row-major):
+ *   input            [batch, in_planes, h, w]
+ *   input_integrated [batch, in_planes, h+1, w+1]     row 0 and column 0 are zero
+ *   x_min .. y_max   [in_planes, num_filters]         REAL pixel units (already multiplied by the
+ *                                                     module's reparametrization factors);
+ *                                                     x_* are ROW bounds, y_* COLUMN bounds
+ *   output, grad_output [batch, in_planes*num_filters, h, w]   channel index = plane*num_filters + filter
+ */
+#ifndef BOXCONV_H_
+#define BOXCONV_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BOXCONV_ABI_VERSION 1
+
+#define BOXCONV_E_INVALID_ARGUMENT (-1) /* null pointer, non-positive size, ... */
+#define BOXCONV_E_WORKSPACE        (-2) /* workspace missing or smaller than *_workspace_bytes() */
+#define BOXCONV_E_TOO_LARGE        (-3) /* a tensor has 2^31 or more elements */
+
+int boxconv_abi_version(void);
+
+/* Message of the last error on this thread ("" if none). Never NULL; valid until the next call
+ * on this thread. */
+const char* boxconv_last_error(void);
+
+/* ---- integral image ------------------------------------------------------------------------
+ * Replaces `integral_image(Tensor) -> Tensor`, reference src/integral_image_interface.cpp:8-27
+ * (kernels: src/integral_image.cpp:8-39). `planes` is the product of all leading dimensions.
+ * out[p][r+1][c+1] = sum_{i<=r, j<=c} in[p][i][j]; out[p][0][*] = out[p][*][0] = 0.
+ * workspace: boxconv_integral_image_workspace_bytes(planes, h, w) bytes, 8-byte aligned (may be
+ * NULL when that size is 0). */
+size_t boxconv_integral_image_workspace_bytes(int64_t planes, int h, int w);
+int boxconv_integral_image_f32(const float* in, float* out, int64_t planes, int h, int w,
+                               void* workspace, size_t workspace_bytes, void* stream);
+int boxconv_integral_image_f64(const double* in, double* out, int64_t planes, int h, int w,
+                               void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- forward ----------------------------------------------------------------------------------
+ * Replaces `box_convolution_forward(input_integrated, x_min, x_max, y_min, y_max, normalize,
+ * exact) -> Tensor[B, C*F, h, w]`, reference src/box_convolution_interface.cpp:13-139 (kernels:
+ * src/box_convolution.cpp:14-40, 100-261, 765-793). normalize: divide by the box area;
+ * exact = 0: bounds are rounded towards the smaller box first. */
+int boxconv_forward_f32(const float* input_integrated, const float* x_min, const float* x_max,
+                        const float* y_min, const float* y_max, float* output, int batch,
+                        int in_planes, int num_filters, int h, int w, int normalize, int exact,
+                        void* stream);
+int boxconv_forward_f64(const double* input_integrated, const double* x_min, const double* x_max,
+                        const double* y_min, const double* y_max, double* output, int batch,
+                        int in_planes, int num_filters, int h, int w, int normalize, int exact,
+                        void* stream);
+
+/* ---- backward ---------------------------------------------------------------------------------
+ * Replaces `box_convolution_backward(input_integrated, x_min, x_max, y_min, y_max, grad_output,
+ * output, reparametrization_h, reparametrization_w, normalize, exact, input_needs_grad,
+ * x_min_needs_grad, x_max_needs_grad, y_min_needs_grad, y_max_needs_grad) -> 5 Tensors`,
+ * reference src/box_convolution_interface.cpp:141-395 (kernels: src/box_convolution.cpp:43-98,
+ * 286-715). A gradient is wanted iff its output pointer is non-NULL:
+ *   grad_input [batch, in_planes, h, w];  grad_x_min .. grad_y_max [in_planes, num_filters],
+ * the latter already multiplied by reparametrization_h (x) / reparametrization_w (y).
+ * `output` (the saved forward result) is accepted for signature parity and may be NULL: the
+ * normalisation term sum(grad_output*output) is recomputed from input_integrated instead of
+ * re-reading it.
+ * workspace: boxconv_backward_workspace_bytes(...) bytes, 256-byte aligned. It receives the
+ * integral image of grad_output (the bulk), band sums and the per-box accumulators. */
+size_t boxconv_backward_workspace_bytes(int batch, int in_planes, int num_filters, int h, int w,
+                                        int elem_size, int input_needs_grad,
+                                        int params_need_grad);
+int boxconv_backward_f32(const float* input_integrated, const float* x_min, const float* x_max,
+                         const float* y_min, const float* y_max, const float* grad_output,
+                         const float* output, float reparametrization_h,
+                         float reparametrization_w, int normalize, int exact, float* grad_input,
+                         float* grad_x_min, float* grad_x_max, float* grad_y_min,
+                         float* grad_y_max, int batch, int in_planes, int num_filters, int h,
+                         int w, void* workspace, size_t workspace_bytes, void* stream);
+int boxconv_backward_f64(const double* input_integrated, const double* x_min, const double* x_max,
+                         const double* y_min, const double* y_max, const double* grad_output,
+                         const double* output, float reparametrization_h,
+                         float reparametrization_w, int normalize, int exact, double* grad_input,
+                         double* grad_x_min, double* grad_x_max, double* grad_y_min,
+                         double* grad_y_max, int batch, int in_planes, int num_filters, int h,
+                         int w, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- clip parameters --------------------------------------------------------------------------
+ * Replaces `clip_parameters(x_min, x_max, y_min, y_max, reparametrization_h, reparametrization_w,
+ * max_input_h, max_input_w, exact) -> None`, reference src/box_convolution_interface.cpp:397-415
+ * (kernel: src/box_convolution.cpp:729-763). In place on the STORED (reparametrized) parameters,
+ * n = in_planes*num_filters elements each. */
+int boxconv_clip_parameters_f32(float* x_min, float* x_max, float* y_min, float* y_max, int n,
+                                double reparametrization_h, double reparametrization_w,
+                                double max_input_h, double max_input_w, int exact, void* stream);
+int boxconv_clip_parameters_f64(double* x_min, double* x_max, double* y_min, double* y_max, int n,
+                                double reparametrization_h, double reparametrization_w,
+                                double max_input_h, double max_input_w, int exact, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* BOXCONV_H_ */

@@ -1,0 +1,191 @@
+"""HIP kernels vs the CPU oracle on identical seeded inputs, through the C ABI (ctypes).
+
+Tolerances: forward and grad_input max|gpu-cpu|/max|cpu| <= 1e-4, box-parameter gradients <= 1e-3
+for float32 (the targets the build is held to); 1e-9 for float64.
+"""
+import numpy as np
+import pytest
+import torch
+
+from helpers import make_boxes, param_grad_floor, rel_err
+
+pytestmark = pytest.mark.gpu
+
+TOL = {np.float32: (1e-4, 1e-3), np.float64: (1e-9, 1e-9)}
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    return t.detach().cpu().numpy()
+
+
+# planes, h, w: chosen to hit one band / several bands, one wave / four waves, vector / scalar
+# loads, several column tiles.
+INTEGRAL_SHAPES = [
+    (1, 2, 2), (3, 5, 7), (2, 10, 10), (6, 28, 28), (1, 33, 257), (2, 64, 128), (1, 200, 36),
+    (1, 300, 1023), (2, 130, 1024), (1, 70, 2048), (1, 40, 2500), (1, 36, 4100), (1, 9, 9000),
+    (5, 1, 1), (2, 1, 300), (2, 300, 1),
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("planes,h,w", INTEGRAL_SHAPES)
+def test_integral_image(hip, oracle, planes, h, w, dtype):
+    rng = np.random.default_rng(planes * 1000003 + h * 1009 + w)
+    x = (rng.random((planes, h, w)) * 2 - 0.5).astype(dtype)
+    got = host(hip.integral_image(dev(x)))
+    want = oracle.integral_image(x)
+    assert got.shape == want.shape
+    # closed form: float64 cumulative sums (the reference's own test oracle, test.py:12-35)
+    exact = np.zeros((planes, h + 1, w + 1))
+    exact[:, 1:, 1:] = x.astype(np.float64).cumsum(1).cumsum(2)
+    assert np.all(got[:, 0, :] == 0) and np.all(got[:, :, 0] == 0)
+    tol = 1e-6 if dtype == np.float32 else 1e-13
+    assert rel_err(got, exact) <= tol
+    assert rel_err(got, want) <= 10 * tol
+    if dtype == np.float32:
+        # sums are carried in double and rounded once: (almost) every entry is the correctly
+        # rounded exact sum, and none is off by more than one unit in the last place
+        ideal = exact.astype(np.float32)
+        assert np.mean(got != ideal) < 1e-4
+        assert np.all(np.abs(got - ideal) <= np.spacing(np.abs(ideal)))
+
+
+def test_integral_image_leading_dims(hip, oracle):
+    x = np.random.default_rng(5).random((2, 3, 2, 17, 19)).astype(np.float32)
+    got = host(hip.integral_image(dev(x)))
+    assert got.shape == (2, 3, 2, 18, 20)
+    assert rel_err(got, oracle.integral_image(x)) <= 1e-6
+    x2 = np.random.default_rng(6).random((17, 19)).astype(np.float32)
+    assert rel_err(host(hip.integral_image(dev(x2))), oracle.integral_image(x2)) <= 1e-6
+
+
+def run_both(hip, oracle, x, boxes, reparam_h, reparam_w, normalize, exact, grad_out,
+             needs=(True,) * 5):
+    """Forward + backward of the native functions on both sides, parameters in real units."""
+    integ_cpu = oracle.integral_image(x)
+    out_cpu = oracle.box_forward(integ_cpu, *boxes, normalize, exact)
+    back_cpu = oracle.box_backward(integ_cpu, *boxes, grad_out, out_cpu, reparam_h, reparam_w,
+                                   normalize, exact, needs)
+    integ = hip.integral_image(dev(x))
+    b = [dev(p) for p in boxes]
+    out = hip.box_convolution_forward(integ, *b, normalize, exact)
+    back = hip.box_convolution_backward(integ, *b, dev(grad_out), out, reparam_h, reparam_w,
+                                        normalize, exact, *needs)
+    torch.cuda.synchronize()
+    scales = dict(i_max=float(np.abs(integ_cpu).max()),
+                  gi_max=float(np.abs(oracle.integral_image(grad_out)).max()))
+    return (out_cpu, back_cpu), (host(out), [None if g is None else host(g) for g in back]), scales
+
+
+def assert_parity(cpu, gpu, dtype, what="", i_max=0.0, gi_max=0.0):
+    """max|gpu-cpu| <= tol * max|cpu| + 8 eps * (largest integral-image entry).
+
+    The additive term is the rounding noise both implementations carry: every output is a
+    difference of integral-image entries, each known to half a unit in its last place. It only
+    matters for tensors that are (nearly) zero, e.g. a box that misses the image entirely.
+    i_max / gi_max: largest |entry| of the integral image of the input / of grad_output."""
+    tol_f, tol_p = TOL[dtype]
+    eps = float(np.finfo(dtype).eps)
+    (out_c, back_c), (out_g, back_g) = cpu, gpu
+
+    def close(got, want, tol, atol):
+        want = np.asarray(want, dtype=np.float64)
+        diff = np.abs(np.asarray(got, dtype=np.float64) - want).max() if want.size else 0.0
+        return diff <= tol * (np.abs(want).max() if want.size else 0.0) + atol
+
+    assert close(out_g, out_c, tol_f, 8 * eps * i_max), what + " forward"
+    if back_c[0] is not None:
+        assert close(back_g[0], back_c[0], tol_f, 8 * eps * gi_max), what + " grad_input"
+    floor = param_grad_floor(back_c[1:])
+    for k, name in enumerate(("x_min", "x_max", "y_min", "y_max")):
+        if back_c[1 + k] is not None:
+            assert rel_err(back_g[1 + k], back_c[1 + k], floor) <= tol_p, what + " grad_" + name
+
+
+SMALL_CASES = [
+    # B, C, F, h, w
+    (1, 1, 1, 2, 2), (1, 1, 1, 5, 9), (2, 3, 2, 7, 6), (1, 2, 3, 10, 10), (2, 1, 5, 28, 28),
+    (1, 2, 2, 17, 65), (1, 1, 3, 40, 130), (1, 2, 2, 33, 300), (1, 1, 2, 20, 600),
+    (1, 1, 2, 12, 1100), (1, 1, 1, 9, 2100), (1, 1, 2, 1, 1), (1, 1, 2, 1, 70), (1, 1, 2, 70, 1),
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("kind", ["inside", "hanging", "integer"])
+@pytest.mark.parametrize("B,C,F,h,w", SMALL_CASES)
+def test_forward_backward_small(hip, oracle, B, C, F, h, w, kind, dtype):
+    seed = (B * 7 + C * 11 + F * 13 + h * 17 + w * 19) * 3 + len(kind)
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((B, C, h, w)).astype(dtype)
+    g = rng.standard_normal((B, C * F, h, w)).astype(dtype)
+    boxes = make_boxes(rng, C, F, max(h, 4), max(w, 4), kind, dtype)
+    for normalize in (True, False):
+        for exact in (True, False):
+            if not exact:
+                # rounded mode needs boxes at least one whole pixel thick to have a finite area
+                bx = list(boxes)
+                bx[1] = (np.maximum(bx[1], np.ceil(bx[0]) + 1)).astype(dtype)
+                bx[3] = (np.maximum(bx[3], np.ceil(bx[2]) + 1)).astype(dtype)
+                use = tuple(bx)
+            else:
+                use = boxes
+            cpu, gpu, sc = run_both(hip, oracle, x, use, 3.5 * h, 2.25 * w, normalize, exact, g)
+            assert_parity(cpu, gpu, dtype, "%s normalize=%s exact=%s" % (kind, normalize, exact), **sc)
+
+
+def test_unit_box_is_identity(hip):
+    x = torch.randn(2, 3, 13, 31, device="cuda")
+    z = torch.zeros(3, 2, device="cuda")
+    out = hip.box_convolution_forward(hip.integral_image(x), z, z, z, z, True, True)
+    want = x.repeat_interleave(2, dim=1)
+    assert torch.allclose(out, want, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("needs", [(True, False, False, False, False), (False, True, True, True, True),
+                                   (False, False, True, False, False), (True, True, False, False, True)])
+def test_selective_gradients(hip, oracle, needs):
+    rng = np.random.default_rng(77)
+    B, C, F, h, w = 2, 2, 3, 19, 23
+    x = rng.standard_normal((B, C, h, w)).astype(np.float32)
+    g = rng.standard_normal((B, C * F, h, w)).astype(np.float32)
+    boxes = make_boxes(rng, C, F, h, w, "hanging")
+    cpu, gpu, sc = run_both(hip, oracle, x, boxes, 40.0, 50.0, True, True, g, needs)
+    for k in range(5):
+        assert (gpu[1][k] is None) == (not needs[k])
+    assert_parity(cpu, gpu, np.float32, **sc)
+
+
+def test_gather_kernels_match_row_streaming(hip, oracle, monkeypatch):
+    """The per-pixel gather kernels (used for very wide images) against the oracle."""
+    rng = np.random.default_rng(123)
+    B, C, F, h, w = 2, 2, 3, 31, 77
+    x = rng.standard_normal((B, C, h, w)).astype(np.float32)
+    g = rng.standard_normal((B, C * F, h, w)).astype(np.float32)
+    boxes = make_boxes(rng, C, F, h, w, "hanging")
+    monkeypatch.setenv("BOXCONV_FORCE_GATHER", "1")
+    for normalize in (True, False):
+        for exact in (True, False):
+            if not exact:
+                boxes = make_boxes(rng, C, F, h, w, "inside")
+            cpu, gpu, sc = run_both(hip, oracle, x, boxes, 40.0, 50.0, normalize, exact, g)
+            assert_parity(cpu, gpu, np.float32, "gather normalize=%s exact=%s" % (normalize, exact), **sc)
+
+
+def test_clip_parameters_matches_oracle(hip, oracle):
+    rng = np.random.default_rng(9)
+    for dtype in (np.float32, np.float64):
+        for exact in (True, False):
+            n = 257
+            rh, rw, mh, mw = 8.0 * 28, 3.3 * 40, 28.0, 40.0
+            p = [(rng.uniform(-1.5, 1.5, n) * s).astype(dtype) for s in (mh / rh, mh / rh, mw / rw, mw / rw)]
+            p[1][:40] = p[0][:40] + rng.uniform(-0.5, 0.5, 40).astype(dtype) / rh   # thin / inverted boxes
+            want = [a.copy() for a in p]
+            oracle.clip_parameters(*want, rh, rw, mh, mw, exact)
+            t = [dev(a) for a in p]
+            hip.clip_parameters(*t, rh, rw, mh, mw, exact)
+            for a, b in zip(t, want):
+                assert np.array_equal(host(a), b)

@@ -1,0 +1,221 @@
+#!/usr/bin/env python3
+"""Benchmark of the box-convolution hot path on one MI355X.
+
+One step = BoxConv2d forward + backward (training mode: parameter clip, stored->real scaling,
+integral image, box sampling; backward to the input and to all four box parameters) on the
+headline workload: BoxConv2d(16, 8, 512, 1024), input float32 [2,16,512,1024], synthetic N(0,1)
+data with seeded boxes, normalize=True, exact=True. Inputs are resident in HBM before timing.
+
+Prints ONE JSON line. `value` is the effective bandwidth on the ALGORITHMIC byte count of one
+step, 4*(2*N_in + 3*N_int + 2*N_out + 2*N_gint) bytes (each tensor of the integral-image data
+flow moved once), divided by the measured time per step. `roofline` prices the dominant kernel
+alone: its algorithmic bytes per launch over its average duration, taken with HIP events placed
+around that kernel's launches on its stream during the timed steps. `cpu_baseline` is the
+reference's CPU path timed on this host on a bounded sample of the same workload.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 1..5] [--no-cpu]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "box-convolutions_amd"))
+
+HBM_PEAK_GBS = 8000.0   # MI355X HBM3E
+METRIC = "BoxConv2d fwd+bwd ms/iter + effective HBM GB/s (% peak) at 2x16ch 512x1024 fp32"
+
+
+def kernel_algorithmic_bytes(ab, elem=4):
+    """Algorithmic bytes moved by ONE launch of each kernel at a given workload: the share of the
+    step's data flow that the kernel is responsible for. band_scan is launched twice per step (input,
+    then grad_output); the figure is the grad_output launch, the larger one."""
+    return {
+        "band_scan": elem * (ab["n_out"] + ab["n_gint"]),        # read grad_output, write its integral
+        "band_colsum": elem * ab["n_out"],                       # pre-pass over grad_output
+        "forward_rows": elem * (ab["n_int"] + ab["n_out"]),      # read integral, write output
+        "grad_input_rows": elem * (ab["n_gint"] + ab["n_in"]),   # read integral of grad_output, write grad_input
+        "grad_params_rows": elem * (ab["n_out"] + ab["n_int"]),  # read grad_output and integral
+    }
+
+
+def load_measured_traffic(kernel, workload_name):
+    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), if a summary
+    for this kernel and workload has been recorded under profiles/."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    try:
+        with open(path) as fh:
+            table = json.load(fh)
+        return table[workload_name][kernel]["bytes_per_launch"]
+    except (OSError, KeyError, ValueError):
+        return None
+
+
+def cpu_baseline(k, ab_full):
+    """The reference's CPU kernels (oracle/_ref, built from the reference's own sources) or, where
+    that library does not exist, the C++ restatement, on a bounded sample of the workload."""
+    import numpy as np  # noqa: F401
+    from baseline_workloads import algorithmic_bytes, make_workload
+    from oracle import cpu_checker
+    chk = cpu_checker.reference() or cpu_checker.oracle()
+    name, B, C, F, h, w = __import__("baseline_workloads").SHAPES[k]
+    # about 10-30 s of single-threaded work: output pixels per second is roughly constant
+    full_px = B * C * F * h * w
+    budget_px = 70e6
+    c = C
+    while c > 1 and B * c * F * h * w > budget_px:
+        c //= 2
+    wl = make_workload(k, in_planes=c)
+    args = [t.numpy() for t in (wl.x, wl.x_min, wl.x_max, wl.y_min, wl.y_max)]
+    t0 = time.perf_counter()
+    out, saved = chk.module_forward(*args, wl.reparametrization_h, wl.reparametrization_w, True, True)
+    chk.module_backward(saved, wl.grad_output.numpy(), wl.reparametrization_h,
+                        wl.reparametrization_w, True, True)
+    dt = time.perf_counter() - t0
+    ab = algorithmic_bytes(wl.B, wl.C, wl.F, wl.h, wl.w)
+    frac = (wl.B * wl.C * wl.F * wl.h * wl.w) / full_px
+    return {
+        "value": ab["alg"] / dt / 1e9,
+        "unit": "GB/s",
+        "cores": 1,
+        "kind": chk.kind,
+        "sample": "%s restricted to its first %d of %d input planes (%.0f%% of the step, %.1f s; "
+                  "planes are independent and the reference's loops are single-threaded, so the "
+                  "full step would take %.1f s)" % (name, wl.C, C, 100 * frac, dt, dt / frac),
+        "ms_per_step_extrapolated": 1e3 * dt / frac,
+        "host_cpus": os.cpu_count(),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", type=int, default=3, choices=[1, 2, 3, 4, 5])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--phases", action="store_true", help="also print per-kernel times to stderr")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU; --gpus %d is not supported (box convolution "
+                 "shards over batch and input planes with no exchange but a %d-float all-reduce, "
+                 "which is outside this benchmark)" % (args.gpus, 4))
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    from baseline_workloads import algorithmic_bytes, make_workload
+    from box_convolution import BoxConv2d, _native
+    _native.load()
+
+    dev = torch.device("cuda:0")
+    wl = make_workload(args.workload)
+    ab = algorithmic_bytes(wl.B, wl.C, wl.F, wl.h, wl.w)
+
+    module = BoxConv2d(wl.C, wl.F, wl.h, wl.w, wl.reparametrization_factor).to(dev)
+    with torch.no_grad():
+        for p, v in zip((module.x_min, module.x_max, module.y_min, module.y_max),
+                        (wl.x_min, wl.x_max, wl.y_min, wl.y_max)):
+            p.copy_(v)
+    module.train()
+    x = wl.x.to(dev).requires_grad_(True)
+    g = wl.grad_output.to(dev)
+    params = list(module.parameters())
+
+    def step():
+        x.grad = None
+        for p in params:
+            p.grad = None
+        out = module(x)
+        out.backward(g)
+
+    before = [p.detach().clone() for p in params]
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    for p, b in zip(params, before):
+        assert torch.equal(p.detach(), b), "workload boxes must be invariant under clipping"
+
+    # which kernel takes the most time per step (one untimed step per candidate)
+    per_kernel = {}
+    for name in ("band_scan", "band_colsum", "forward_rows", "grad_input_rows", "grad_params_rows"):
+        _native.profile_arm(name)
+        step()
+        ms, launches = _native.profile_collect()
+        per_kernel[name] = (ms, launches)
+    dominant = max(per_kernel, key=lambda n: per_kernel[n][0])
+    if args.phases:
+        print("per-kernel ms per step:", {k: round(v[0], 4) for k, v in per_kernel.items()},
+              file=sys.stderr)
+
+    # ---- timed region ---------------------------------------------------------------------------
+    _native.profile_arm(dominant)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    dom_ms, dom_launches = _native.profile_collect()
+
+    ms_per_step = 1e3 * elapsed / args.steps
+    value = ab["alg"] / (elapsed / args.steps) / 1e9
+
+    kbytes = kernel_algorithmic_bytes(ab)
+    if dominant == "band_scan":
+        # two launches per step (input planes, then grad_output planes): price the pair
+        launches_per_step = dom_launches / args.steps
+        bytes_per_launch = (kbytes["band_scan"] + 4 * (ab["n_in"] + ab["n_int"])) / launches_per_step
+    else:
+        bytes_per_launch = kbytes[dominant]
+    avg_launch_s = dom_ms / 1e3 / max(dom_launches, 1)
+    achieved = bytes_per_launch / avg_launch_s / 1e9
+
+    result = {
+        "metric": METRIC,
+        "value": round(value, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "%s: BoxConv2d(%d,%d,%d,%d) fwd+bwd, input [%d,%d,%d,%d], normalize, exact, "
+                        "grads to input and 4 box parameters" % (
+                            wl.name, wl.C, wl.F, wl.h, wl.w, wl.B, wl.C, wl.h, wl.w),
+            "algorithmic_bytes_per_step": ab["alg"],
+            "io_bytes_per_step": ab["io"],
+            "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+            "io_GBps": round(ab["io"] / (elapsed / args.steps) / 1e9, 2),
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": dominant,
+            "achieved": round(achieved, 2),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": load_measured_traffic(dominant, wl.name),
+            "algorithmic_bytes_per_launch": int(bytes_per_launch),
+            "avg_launch_us": round(1e6 * avg_launch_s, 2),
+            "launches_timed": dom_launches,
+        },
+        "kernel_ms_per_step": {k: round(v[0], 4) for k, v in per_kernel.items()},
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(args.workload, ab)
+        result["cpu_baseline"]["speedup_vs_cpu"] = round(
+            result["cpu_baseline"]["ms_per_step_extrapolated"] / ms_per_step, 1)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

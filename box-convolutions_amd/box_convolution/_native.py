@@ -27,6 +27,8 @@ _vp, _i, _i64, _sz, _f, _d = (ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, cty
 _SIGNATURES = {
     "boxconv_abi_version": (_i, []),
     "boxconv_last_error": (ctypes.c_char_p, []),
+    "boxconv_profile_arm": (_i, [ctypes.c_char_p]),
+    "boxconv_profile_collect": (_i, [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int)]),
     "boxconv_integral_image_workspace_bytes": (_sz, [_i64, _i, _i]),
     "boxconv_backward_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i, _i, _i]),
 }
@@ -263,3 +265,22 @@ def clip_parameters(x_min, x_max, y_min, y_max, reparametrization_h, reparametri
             float(reparametrization_h), float(reparametrization_w), float(max_input_h),
             float(max_input_w), int(bool(exact)), _stream(x_min.device))
     _check(rc, "clip_parameters")
+
+
+KERNEL_NAMES = ("band_colsum", "band_prefix", "band_scan", "forward_rows", "grad_input_rows",
+                "grad_params_rows", "param_grad_finalize", "fill_zero", "clip", "forward_gather",
+                "grad_input_gather", "grad_params_gather")
+
+
+def profile_arm(kernel_name):
+    """Bracket every later launch of `kernel_name` with HIP events (None disarms)."""
+    _check(load().boxconv_profile_arm(kernel_name.encode() if kernel_name else None),
+           "profile_arm")
+
+
+def profile_collect():
+    """(summed kernel milliseconds, launches) since profile_arm; waits for the kernels."""
+    total, count = ctypes.c_double(0.0), ctypes.c_int(0)
+    _check(load().boxconv_profile_collect(ctypes.byref(total), ctypes.byref(count)),
+           "profile_collect")
+    return total.value, count.value

@@ -55,8 +55,8 @@ hipError_t clip_launch(T* xmin, T* xmax, T* ymin, T* ymax, int n, double reparam
     if (n == 0) return hipSuccess;
     // float literals widened to double (src/box_convolution_interface.cpp:405-406)
     const double min_size = static_cast<double>(exact ? 1.001f : 2.001f);
-    hipLaunchKernelGGL((clip_kernel<T>), dim3((n + 255) / 256), dim3(256), 0, stream, xmin, xmax,
-                       ymin, ymax, n, reparam_h, reparam_w, max_h, max_w, min_size);
+    BOXCONV_LAUNCH("clip", (clip_kernel<T>), dim3((n + 255) / 256), dim3(256), 0, stream, xmin, xmax,
+                   ymin, ymax, n, reparam_h, reparam_w, max_h, max_w, min_size);
     return hipGetLastError();
 }
 

@@ -20,10 +20,12 @@
 //
 // Row streaming. Column 0 of I is zero, so V(i) has w interesting entries. A workgroup owns a
 // band of output rows at full width: each lane keeps I[t(i-1)] and I[b(i)] of its columns in
-// registers, loads only the two new rows I[t(i)], I[b(i+1)] per output row (coalesced), writes
-// V(i) to LDS, and after one barrier every output pixel reads its four V entries from LDS.
-// That is 2 global loads per output pixel instead of 16 gathers. The row after next is
-// requested before the barrier so its latency overlaps the LDS phase.
+// registers and loads only the new rows I[t(i)], I[b(i+1)] per output row (coalesced). Two output
+// rows are handled per barrier, and the loads of the next two are issued before the barrier.
+//   forward / grad input: V(i) goes to LDS; every output pixel reads its four V entries.
+//   parameter gradients : the row of grad_output goes to LDS instead and every column q reads
+//       the four grad_output entries whose box edges fall on q (the transposed access), so V and
+//       the two row differences never leave registers: sum_j g[j]*H(X)[j] = sum_q X[q]*Ht(g)[q].
 //
 // Workgroup ids are remapped (xcd_contiguous_id) so all filters and bands of one input plane run
 // on one XCD and its integral plane stays in that XCD's L2.
@@ -48,25 +50,41 @@ template <class T>
 struct SampleArgs {
     const T* src;         // integral planes, (h+1) x (w+1) each, contiguous
     BoxParams<T> prm;
-    T* dst;               // forward: [B,C,F,h,w]; grad input: [B,C,h,w]
-    const T* grad_out;    // param grads only: [B,C,F,h,w]
+    T* dst;               // forward: [planes,F,h,w]; grad input: [planes,h,w]
+    const T* grad_out;    // param grads only: [planes,F,h,w]
     double* acc;          // param grads only: [C*F*5]
+    double* colsum;       // param grads only: per-band column sums of grad_out, or null
     int C, F, h, w;
     int nb, R;            // bands per plane and rows per band
+    int64_t plane0;       // global index of the first plane (selects the boxes)
     int64_t total;        // workgroups with work
     int64_t per_xcd;      // ceil(total / 8)
     int normalize;
 };
 
-template <class T, int K>
+// FULL: w == K * blockDim.x, so every (lane, k) slot is a valid column and no bounds checks are
+// compiled in.
+template <class T, int K, bool FULL>
 __device__ __forceinline__ void load_row(const T* __restrict__ plane, int64_t pitch, int row,
                                          int w, int q0, int nt, T (&dst)[K]) {
     const T* r = plane + static_cast<int64_t>(row) * pitch;
 #pragma unroll
     for (int k = 0; k < K; ++k) {
         const int q = q0 + nt * k;
-        dst[k] = (q <= w) ? r[q] : T(0);
+        dst[k] = (FULL || q <= w) ? r[q] : T(0);
     }
+}
+
+// The four rows that become new when the window moves from output rows (i-2, i-1) to (i, i+1):
+// I[t(i)], I[t(i+1)], I[b(i+1)], I[b(i+2)].
+template <class T, int K, bool FULL>
+__device__ __forceinline__ void load_pair(const T* __restrict__ plane, int64_t pitch, int i,
+                                          int xlo, int xhi, int h, int w, int q0, int nt,
+                                          T (&t0)[K], T (&t1)[K], T (&b1)[K], T (&b2)[K]) {
+    load_row<T, K, FULL>(plane, pitch, clampi(i + xlo, 0, h), w, q0, nt, t0);
+    load_row<T, K, FULL>(plane, pitch, clampi(i + 1 + xlo, 0, h), w, q0, nt, t1);
+    load_row<T, K, FULL>(plane, pitch, clampi(i + 1 + xhi, 0, h), w, q0, nt, b1);
+    load_row<T, K, FULL>(plane, pitch, clampi(i + 2 + xhi, 0, h), w, q0, nt, b2);
 }
 
 template <class T, bool EXACT>
@@ -78,31 +96,43 @@ __device__ __forceinline__ T blend(T lo_adv, T lo, T hi, T hi_adv, T flo, T fhi)
 
 // Row vector into LDS. Layout: V[q+1] for q = -1..w+1 with V(-1) = V(0) = 0 and V(w+1) = V(w), so
 // a clamped column pair is always two adjacent entries.
-template <class T, int K>
+template <class T, int K, bool FULL>
 __device__ __forceinline__ void publish_row(T* __restrict__ V, const T (&val)[K], int w, int q0,
                                             int nt) {
 #pragma unroll
     for (int k = 0; k < K; ++k) {
         const int q = q0 + nt * k;
-        if (q <= w) {
-            V[q + 1] = val[k];
-            if (q == w) V[w + 2] = val[k];
-        }
+        if (FULL || q <= w) V[q + 1] = val[k];
+        if (FULL ? (k == K - 1 && q0 == nt) : (q == w)) V[w + 2] = val[k];
     }
     if (q0 == 1) { V[0] = T(0); V[1] = T(0); }
 }
 
-struct ColumnTaps { int lo, hi; };   // LDS indices of (lAdv, l) = (lo, lo+1) and (r, rAdv) = (hi, hi+1)
-__device__ __forceinline__ ColumnTaps column_taps(int j, int ylo, int yhi, int w) {
-    ColumnTaps c;
-    c.lo = clampi(j + ylo, 0, w + 1);        // V index of lAdv; l is the next entry
-    c.hi = clampi(j + yhi, -1, w) + 1;       // V index of r; rAdv is the next entry
-    return c;
+// LDS indices of the column pairs (lAdv, l) = (lo, lo+1) and (r, rAdv) = (hi, hi+1) of pixel j.
+template <int K>
+__device__ __forceinline__ void column_taps(int (&lo)[K], int (&hi)[K], int ylo, int yhi, int w,
+                                            int nt) {
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const int j = static_cast<int>(threadIdx.x) + nt * k;
+        lo[k] = clampi(j + ylo, 0, w + 1);
+        hi[k] = clampi(j + yhi, -1, w) + 1;
+    }
+}
+
+template <class T>
+struct BoxOfWorkgroup {
+    T xmin, xmax, ymin, ymax;
+};
+template <class T>
+__device__ __forceinline__ BoxOfWorkgroup<T> load_box(const BoxParams<T>& prm, int k_par) {
+    return {prm.xmin[k_par], prm.xmax[k_par], prm.ymin[k_par], prm.ymax[k_par]};
 }
 
 // ---------------------------------------------------------------------------------------------
-// Forward. Work item = (plane p, filter f, band). blockDim = nt, K = ceil(w / nt) <= template K.
-template <class T, int K, bool EXACT>
+// Forward. Work item = (plane p, filter f, band). blockDim = nt, K >= ceil(w / nt).
+// LDS: [2 buffers][2 rows][w+3] T.
+template <class T, int K, bool EXACT, bool FULL>
 __global__ void __launch_bounds__(256) forward_rows_kernel(SampleArgs<T> a) {
     const int64_t vid = xcd_contiguous_id(a.per_xcd);
     if (vid >= a.total) return;
@@ -110,13 +140,13 @@ __global__ void __launch_bounds__(256) forward_rows_kernel(SampleArgs<T> a) {
     const int64_t pf = vid / a.nb;
     const int f = static_cast<int>(pf % a.F);
     const int64_t p = pf / a.F;
-    const int k_par = static_cast<int>(p % a.C) * a.F + f;
+    const int k_par = static_cast<int>((a.plane0 + p) % a.C) * a.F + f;
     const int h = a.h, w = a.w, nt = blockDim.x, q0 = 1 + threadIdx.x;
 
-    const T xmin = a.prm.xmin[k_par], xmax = a.prm.xmax[k_par];
-    const T ymin = a.prm.ymin[k_par], ymax = a.prm.ymax[k_par];
-    const BoxSplit<T> s = split_forward(xmin, xmax, ymin, ymax);
-    const T scale = a.normalize ? inverse_extent(xmin, xmax, ymin, ymax, EXACT, true, true) : T(1);
+    const BoxOfWorkgroup<T> bx = load_box(a.prm, k_par);
+    const BoxSplit<T> s = split_forward(bx.xmin, bx.xmax, bx.ymin, bx.ymax);
+    const T scale = a.normalize
+        ? inverse_extent(bx.xmin, bx.xmax, bx.ymin, bx.ymax, EXACT, true, true) : T(1);
 
     const int64_t pitch = w + 1;
     const T* plane = a.src + p * static_cast<int64_t>(h + 1) * pitch;
@@ -127,50 +157,69 @@ __global__ void __launch_bounds__(256) forward_rows_kernel(SampleArgs<T> a) {
     const int i0 = band * a.R;
     const int i1 = min(h, i0 + a.R);
 
-    T pT[K], pB[K], nT[K], nB[K];
-    load_row<T, K>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), w, q0, nt, pT);
-    load_row<T, K>(plane, pitch, clampi(i0 + s.xhi, 0, h), w, q0, nt, pB);
-    load_row<T, K>(plane, pitch, clampi(i0 + s.xlo, 0, h), w, q0, nt, nT);
-    load_row<T, K>(plane, pitch, clampi(i0 + s.xhi + 1, 0, h), w, q0, nt, nB);
+    int lo[K], hi[K];
+    column_taps<K>(lo, hi, s.ylo, s.yhi, w, nt);
 
-    for (int i = i0; i < i1; ++i) {
-        T* V = vbuf + ((i - i0) & 1) * vlen;
-        T fT[K] = {}, fB[K] = {};
-        if (i + 1 < i1) {
-            load_row<T, K>(plane, pitch, clampi(i + 1 + s.xlo, 0, h), w, q0, nt, fT);
-            load_row<T, K>(plane, pitch, clampi(i + 2 + s.xhi, 0, h), w, q0, nt, fB);
-        }
-        T val[K];
+    T ta[K], bc[K];                       // I[t(i-1)], I[b(i)]
+    T t0[K], t1[K], b1[K], b2[K];         // I[t(i)], I[t(i+1)], I[b(i+1)], I[b(i+2)]
+    load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), w, q0, nt, ta);
+    load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xhi, 0, h), w, q0, nt, bc);
+    load_pair<T, K, FULL>(plane, pitch, i0, s.xlo, s.xhi, h, w, q0, nt, t0, t1, b1, b2);
+
+    int flip = 0;
+    for (int i = i0; i < i1; i += 2) {
+        T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {};
+        if (i + 2 < i1)
+            load_pair<T, K, FULL>(plane, pitch, i + 2, s.xlo, s.xhi, h, w, q0, nt, n0, n1, n2, n3);
+
+        T* V0 = vbuf + flip * 2 * vlen;
+        T* V1 = V0 + vlen;
+        flip ^= 1;
+        T v0[K], v1[K];
 #pragma unroll
-        for (int k = 0; k < K; ++k) val[k] = blend<T, EXACT>(pT[k], nT[k], pB[k], nB[k], s.fxlo, s.fxhi);
-        publish_row<T, K>(V, val, w, q0, nt);
+        for (int k = 0; k < K; ++k) {
+            v0[k] = blend<T, EXACT>(ta[k], t0[k], bc[k], b1[k], s.fxlo, s.fxhi);
+            v1[k] = blend<T, EXACT>(t0[k], t1[k], b1[k], b2[k], s.fxlo, s.fxhi);
+        }
+        publish_row<T, K, FULL>(V0, v0, w, q0, nt);
+        publish_row<T, K, FULL>(V1, v1, w, q0, nt);
         __syncthreads();
 
         T* orow = out + static_cast<int64_t>(i) * w;
+        const bool second = i + 1 < i1;
 #pragma unroll
         for (int k = 0; k < K; ++k) {
             const int j = static_cast<int>(threadIdx.x) + nt * k;
-            if (j < w) {
-                const ColumnTaps c = column_taps(j, s.ylo, s.yhi, w);
-                const T o = blend<T, EXACT>(V[c.lo], V[c.lo + 1], V[c.hi], V[c.hi + 1], s.fylo, s.fyhi);
-                __builtin_nontemporal_store(o * scale, orow + j);
+            if (FULL || j < w) {
+                const T o0 = blend<T, EXACT>(V0[lo[k]], V0[lo[k] + 1], V0[hi[k]], V0[hi[k] + 1],
+                                             s.fylo, s.fyhi);
+                __builtin_nontemporal_store(o0 * scale, orow + j);
+                if (second) {
+                    const T o1 = blend<T, EXACT>(V1[lo[k]], V1[lo[k] + 1], V1[hi[k]],
+                                                 V1[hi[k] + 1], s.fylo, s.fyhi);
+                    __builtin_nontemporal_store(o1 * scale, orow + w + j);
+                }
             }
         }
 #pragma unroll
-        for (int k = 0; k < K; ++k) { pT[k] = nT[k]; pB[k] = nB[k]; nT[k] = fT[k]; nB[k] = fB[k]; }
+        for (int k = 0; k < K; ++k) {
+            ta[k] = t1[k]; bc[k] = b2[k];
+            t0[k] = n0[k]; t1[k] = n1[k]; b1[k] = n2[k]; b2[k] = n3[k];
+        }
     }
 }
 
 // ---------------------------------------------------------------------------------------------
 // Gradient w.r.t. the input. Work item = (plane p = (b,c), band of RB rows); the F mirrored boxes
 // are visited in order and summed in registers, so no [B,C,F,h,w] temporary exists.
-template <class T, int K, int RB, bool EXACT>
+template <class T, int K, int RB, bool EXACT, bool FULL>
 __global__ void __launch_bounds__(256) grad_input_rows_kernel(SampleArgs<T> a) {
+    static_assert(RB % 2 == 0, "rows are handled in pairs");
     const int64_t vid = xcd_contiguous_id(a.per_xcd);
     if (vid >= a.total) return;
     const int band = static_cast<int>(vid % a.nb);
     const int64_t p = vid / a.nb;
-    const int c_in = static_cast<int>(p % a.C);
+    const int c_in = static_cast<int>((a.plane0 + p) % a.C);
     const int h = a.h, w = a.w, nt = blockDim.x, q0 = 1 + threadIdx.x;
     const int64_t pitch = w + 1;
     const int64_t ipl = static_cast<int64_t>(h + 1) * pitch;
@@ -186,48 +235,54 @@ __global__ void __launch_bounds__(256) grad_input_rows_kernel(SampleArgs<T> a) {
 
     int flip = 0;
     for (int f = 0; f < a.F; ++f) {
-        const int k_par = c_in * a.F + f;
-        const T xmin = a.prm.xmin[k_par], xmax = a.prm.xmax[k_par];
-        const T ymin = a.prm.ymin[k_par], ymax = a.prm.ymax[k_par];
-        const BoxSplit<T> s = split_grad_input(xmin, xmax, ymin, ymax);
-        const T scale = a.normalize ? inverse_extent(xmin, xmax, ymin, ymax, EXACT, true, true) : T(1);
+        const BoxOfWorkgroup<T> bx = load_box(a.prm, c_in * a.F + f);
+        const BoxSplit<T> s = split_grad_input(bx.xmin, bx.xmax, bx.ymin, bx.ymax);
+        const T scale = a.normalize
+            ? inverse_extent(bx.xmin, bx.xmax, bx.ymin, bx.ymax, EXACT, true, true) : T(1);
         const T* plane = a.src + (p * a.F + f) * ipl;
 
-        T pT[K], pB[K], nT[K], nB[K];
-        load_row<T, K>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), w, q0, nt, pT);
-        load_row<T, K>(plane, pitch, clampi(i0 + s.xhi, 0, h), w, q0, nt, pB);
-        load_row<T, K>(plane, pitch, clampi(i0 + s.xlo, 0, h), w, q0, nt, nT);
-        load_row<T, K>(plane, pitch, clampi(i0 + s.xhi + 1, 0, h), w, q0, nt, nB);
+        int lo[K], hi[K];
+        column_taps<K>(lo, hi, s.ylo, s.yhi, w, nt);
+
+        T ta[K], bc[K], t0[K], t1[K], b1[K], b2[K];
+        load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), w, q0, nt, ta);
+        load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xhi, 0, h), w, q0, nt, bc);
+        load_pair<T, K, FULL>(plane, pitch, i0, s.xlo, s.xhi, h, w, q0, nt, t0, t1, b1, b2);
 
 #pragma unroll
-        for (int r = 0; r < RB; ++r) {
+        for (int r = 0; r < RB; r += 2) {
             const int i = i0 + r;
             if (i < h) {                                   // uniform across the workgroup
-                T* V = vbuf + flip * vlen;
+                T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {};
+                if (r + 2 < RB && i + 2 < h)
+                    load_pair<T, K, FULL>(plane, pitch, i + 2, s.xlo, s.xhi, h, w, q0, nt, n0, n1, n2, n3);
+                T* V0 = vbuf + flip * 2 * vlen;
+                T* V1 = V0 + vlen;
                 flip ^= 1;
-                T fT[K] = {}, fB[K] = {};
-                if (r + 1 < RB && i + 1 < h) {
-                    load_row<T, K>(plane, pitch, clampi(i + 1 + s.xlo, 0, h), w, q0, nt, fT);
-                    load_row<T, K>(plane, pitch, clampi(i + 2 + s.xhi, 0, h), w, q0, nt, fB);
-                }
-                T val[K];
+                T v0[K], v1[K];
 #pragma unroll
-                for (int k = 0; k < K; ++k)
-                    val[k] = blend<T, EXACT>(pT[k], nT[k], pB[k], nB[k], s.fxlo, s.fxhi);
-                publish_row<T, K>(V, val, w, q0, nt);
+                for (int k = 0; k < K; ++k) {
+                    v0[k] = blend<T, EXACT>(ta[k], t0[k], bc[k], b1[k], s.fxlo, s.fxhi);
+                    v1[k] = blend<T, EXACT>(t0[k], t1[k], b1[k], b2[k], s.fxlo, s.fxhi);
+                }
+                publish_row<T, K, FULL>(V0, v0, w, q0, nt);
+                publish_row<T, K, FULL>(V1, v1, w, q0, nt);
                 __syncthreads();
 #pragma unroll
                 for (int k = 0; k < K; ++k) {
                     const int j = static_cast<int>(threadIdx.x) + nt * k;
-                    if (j < w) {
-                        const ColumnTaps c = column_taps(j, s.ylo, s.yhi, w);
-                        const T o = blend<T, EXACT>(V[c.lo], V[c.lo + 1], V[c.hi], V[c.hi + 1],
-                                                    s.fylo, s.fyhi);
-                        acc[r][k] += o * scale;
+                    if (FULL || j < w) {
+                        acc[r][k] += scale * blend<T, EXACT>(V0[lo[k]], V0[lo[k] + 1], V0[hi[k]],
+                                                             V0[hi[k] + 1], s.fylo, s.fyhi);
+                        acc[r + 1][k] += scale * blend<T, EXACT>(V1[lo[k]], V1[lo[k] + 1], V1[hi[k]],
+                                                                 V1[hi[k] + 1], s.fylo, s.fyhi);
                     }
                 }
 #pragma unroll
-                for (int k = 0; k < K; ++k) { pT[k] = nT[k]; pB[k] = nB[k]; nT[k] = fT[k]; nB[k] = fB[k]; }
+                for (int k = 0; k < K; ++k) {
+                    ta[k] = t1[k]; bc[k] = b2[k];
+                    t0[k] = n0[k]; t1[k] = n1[k]; b1[k] = n2[k]; b2[k] = n3[k];
+                }
             }
         }
     }
@@ -240,7 +295,7 @@ __global__ void __launch_bounds__(256) grad_input_rows_kernel(SampleArgs<T> a) {
 #pragma unroll
             for (int k = 0; k < K; ++k) {
                 const int j = static_cast<int>(threadIdx.x) + nt * k;
-                if (j < w) out[static_cast<int64_t>(i) * w + j] = acc[r][k];
+                if (FULL || j < w) out[static_cast<int64_t>(i) * w + j] = acc[r][k];
             }
         }
     }
@@ -266,89 +321,188 @@ __device__ __forceinline__ void block_accumulate5(const double (&v)[5], double* 
 
 // Gradient w.r.t. the box bounds. Work item = (plane p, filter f, band). Accumulates, per (c,f):
 //   [0] sum g*dS/dxmin  [1] sum g*dS/dxmax  [2] sum g*dS/dymin  [3] sum g*dS/dymax  [4] sum g*S
-// Lanes accumulate in T over their pixels of the band, the workgroup sum is taken in double and
-// leaves through one atomic per value.
-template <class T, int K, bool EXACT>
+//
+// Transposed access: for X in {V, DT = I[t]-I[tAdv], DB = I[bAdv]-I[b]} (per-column values of the
+// current output row, held in registers by the lane that owns column q),
+//   sum_j g[j]*H(X)[j] = sum_{q=1..w} X[q]*W[q] + X[w]*tail,
+//   W[q] = (gr - gl) + fyhi*(grA - gr) + fylo*(gl - glA),
+//   gr = g[q-yhi], grA = g[q-yhi-1], gl = g[q-ylo], glA = g[q-ylo+1]   (0 outside [0,w)).
+// W[w] as written counts some pixels whose box edge is clamped onto column w with the wrong
+// weight; `tail` = sum_j g[j]*delta[j] fixes that with a per-column constant
+//   delta[j] = (1-fyhi)[j > w-yhi] + fyhi[j > w-yhi-1] - (1-fylo)[j > w-ylo] - fylo[j > w-ylo+1].
+// Likewise dS/dymax = sum_q V[q]*(grA - gr) + V[w]*g[w-yhi] and
+//          dS/dymin = -sum_q V[q]*(gl - glA) - V[w]*g[w-ylo+1].
+// Column 0 of the integral image is zero, so clamping at the left edge needs no correction.
+//
+// LDS: [2 buffers][2 rows] of { grad_output row with two zeros on either side (w+4), X[w] (3) }.
+// If a.colsum is set, the per-band column sums of grad_output are written too (first pass of
+// the integral image of grad_output, which therefore does not have to read it a second time).
+template <class T, int K, bool EXACT, bool FULL>
 __global__ void __launch_bounds__(256) grad_params_rows_kernel(SampleArgs<T> a) {
     const int64_t vid = xcd_contiguous_id(a.per_xcd);
-    const bool live = vid < a.total;
-    // No early return: every lane reaches the wave-wide sums below.
-    const int64_t wid = live ? vid : 0;
-    const int band = static_cast<int>(wid % a.nb);
-    const int64_t pf = wid / a.nb;
+    if (vid >= a.total) return;                      // whole workgroup leaves together
+    const int band = static_cast<int>(vid % a.nb);
+    const int64_t pf = vid / a.nb;
     const int f = static_cast<int>(pf % a.F);
     const int64_t p = pf / a.F;
-    const int k_par = static_cast<int>(p % a.C) * a.F + f;
-    const int h = a.h, w = a.w, nt = blockDim.x, q0 = 1 + threadIdx.x;
+    const int k_par = static_cast<int>((a.plane0 + p) % a.C) * a.F + f;
+    const int h = a.h, w = a.w, nt = blockDim.x, tid = threadIdx.x, q0 = 1 + tid;
 
-    const T xmin = a.prm.xmin[k_par], xmax = a.prm.xmax[k_par];
-    const T ymin = a.prm.ymin[k_par], ymax = a.prm.ymax[k_par];
-    const BoxSplit<T> s = split_grad_params(xmin, xmax, ymin, ymax);
+    const BoxOfWorkgroup<T> bx = load_box(a.prm, k_par);
+    const BoxSplit<T> s = split_grad_params(bx.xmin, bx.xmax, bx.ymin, bx.ymax);
 
     const int64_t pitch = w + 1;
     const T* plane = a.src + p * static_cast<int64_t>(h + 1) * pitch;
     const T* gout = a.grad_out + pf * static_cast<int64_t>(h) * w;
-    const int vlen = w + 3;
-    T* vbuf = reinterpret_cast<T*>(smem_raw);                       // [2][3][vlen]
-    double* red = reinterpret_cast<double*>(smem_raw + ((2 * 3 * vlen * sizeof(T) + 15) / 16) * 16);
+    const int glen = w + 8;                          // row (w), 2+2 zero pads, X[w] triple, spare
+    T* gbuf = reinterpret_cast<T*>(smem_raw);        // [2][2][glen]
+    double* red = reinterpret_cast<double*>(smem_raw + ((4 * glen * sizeof(T) + 15) / 16) * 16);
 
     const int i0 = band * a.R;
-    const int i1 = live ? min(h, i0 + a.R) : i0;
+    const int i1 = min(h, i0 + a.R);
+
+    // zero pads of all four rows (never overwritten)
+    if (tid < 16) {
+        T* row = gbuf + (tid >> 2) * glen;
+        const int e = tid & 3;
+        row[e < 2 ? e : w + e] = T(0);
+    }
+
+    // lane-constant LDS indices of the pairs (grA, gr) and (gl, glA), and the tail weights
+    int ir[K], il[K];
+    T delta[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const int j = tid + nt * k;
+        const int q = j + 1;
+        ir[k] = clampi(q - s.yhi - 1, -2, w) + 2;
+        il[k] = clampi(q - s.ylo, -2, w) + 2;
+        T d = T(0);
+        if (FULL || j < w) {
+            const T one = T(1);
+            d = (EXACT ? (one - s.fyhi) : one) * T(j > w - s.yhi)
+              + (EXACT ? s.fyhi : T(0)) * T(j > w - s.yhi - 1)
+              - (EXACT ? (one - s.fylo) : one) * T(j > w - s.ylo)
+              - (EXACT ? s.fylo : T(0)) * T(j > w - s.ylo + 1);
+        }
+        delta[k] = d;
+    }
+    const int j_ymax = w - s.yhi, j_ymin = w - s.ylo + 1;
+    const int idx_ymax = (j_ymax >= 0 && j_ymax < w) ? j_ymax + 2 : 0;     // index 0 holds a zero
+    const int idx_ymin = (j_ymin >= 0 && j_ymin < w) ? j_ymin + 2 : 0;
 
     T sum[5] = {T(0), T(0), T(0), T(0), T(0)};
+    double cs[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) cs[k] = 0.0;
 
-    T pT[K], pB[K], nT[K], nB[K];
-    load_row<T, K>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), w, q0, nt, pT);
-    load_row<T, K>(plane, pitch, clampi(i0 + s.xhi, 0, h), w, q0, nt, pB);
-    load_row<T, K>(plane, pitch, clampi(i0 + s.xlo, 0, h), w, q0, nt, nT);
-    load_row<T, K>(plane, pitch, clampi(i0 + s.xhi + 1, 0, h), w, q0, nt, nB);
-
-    for (int i = i0; i < i1; ++i) {
-        T* V = vbuf + ((i - i0) & 1) * 3 * vlen;
-        T* DT = V + vlen;
-        T* DB = DT + vlen;
-        T fT[K] = {}, fB[K] = {}, g[K];
-        if (i + 1 < i1) {
-            load_row<T, K>(plane, pitch, clampi(i + 1 + s.xlo, 0, h), w, q0, nt, fT);
-            load_row<T, K>(plane, pitch, clampi(i + 2 + s.xhi, 0, h), w, q0, nt, fB);
-        }
-        const T* grow = gout + static_cast<int64_t>(i) * w;
+    T ta[K], bc[K], t0[K], t1[K], b1[K], b2[K], g0[K], g1[K];
+    load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), w, q0, nt, ta);
+    load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xhi, 0, h), w, q0, nt, bc);
+    load_pair<T, K, FULL>(plane, pitch, i0, s.xlo, s.xhi, h, w, q0, nt, t0, t1, b1, b2);
+    auto load_g = [&](int i, T (&dst)[K]) {
+        const T* grow = gout + static_cast<int64_t>(min(i, h - 1)) * w;
+        const bool valid = i < i1;
 #pragma unroll
         for (int k = 0; k < K; ++k) {
-            const int j = static_cast<int>(threadIdx.x) + nt * k;
-            g[k] = (j < w) ? grow[j] : T(0);
+            const int j = tid + nt * k;
+            dst[k] = (valid && (FULL || j < w)) ? grow[j] : T(0);
         }
-        T val[K], dt[K], db[K];
+    };
+    load_g(i0, g0);
+    load_g(i0 + 1, g1);
+
+    int flip = 0;
+    for (int i = i0; i < i1; i += 2) {
+        T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {}, m0[K] = {}, m1[K] = {};
+        if (i + 2 < i1) {
+            load_pair<T, K, FULL>(plane, pitch, i + 2, s.xlo, s.xhi, h, w, q0, nt, n0, n1, n2, n3);
+            load_g(i + 2, m0);
+            load_g(i + 3, m1);
+        }
+
+        T* G0 = gbuf + flip * 2 * glen;
+        T* G1 = G0 + glen;
+        flip ^= 1;
+
+        T v0[K], dt0[K], db0[K], v1[K], dt1[K], db1[K];
 #pragma unroll
         for (int k = 0; k < K; ++k) {
-            val[k] = blend<T, EXACT>(pT[k], nT[k], pB[k], nB[k], s.fxlo, s.fxhi);
-            dt[k] = nT[k] - pT[k];
-            db[k] = nB[k] - pB[k];
+            dt0[k] = t0[k] - ta[k];  db0[k] = b1[k] - bc[k];
+            dt1[k] = t1[k] - t0[k];  db1[k] = b2[k] - b1[k];
+            v0[k] = bc[k] - t0[k];
+            v1[k] = b1[k] - t1[k];
+            if (EXACT) {
+                v0[k] += s.fxhi * db0[k] + s.fxlo * dt0[k];
+                v1[k] += s.fxhi * db1[k] + s.fxlo * dt1[k];
+            }
+            const int j = tid + nt * k;
+            if (FULL || j < w) {
+                G0[j + 2] = g0[k];
+                G1[j + 2] = g1[k];
+                cs[k] += static_cast<double>(g0[k]) + static_cast<double>(g1[k]);
+            }
+            if (FULL ? (k == K - 1 && tid == nt - 1) : (j == w - 1)) {      // owner of column q = w
+                G0[w + 4] = v0[k]; G0[w + 5] = dt0[k]; G0[w + 6] = db0[k];
+                G1[w + 4] = v1[k]; G1[w + 5] = dt1[k]; G1[w + 6] = db1[k];
+            }
         }
-        publish_row<T, K>(V, val, w, q0, nt);
-        publish_row<T, K>(DT, dt, w, q0, nt);
-        publish_row<T, K>(DB, db, w, q0, nt);
         __syncthreads();
+
+        T tail0 = T(0), tail1 = T(0);
 #pragma unroll
         for (int k = 0; k < K; ++k) {
-            const int j = static_cast<int>(threadIdx.x) + nt * k;
-            if (j < w) {
-                const ColumnTaps c = column_taps(j, s.ylo, s.yhi, w);
-                const T vla = V[c.lo], vl = V[c.lo + 1], vr = V[c.hi], vra = V[c.hi + 1];
-                const T S = blend<T, EXACT>(vla, vl, vr, vra, s.fylo, s.fyhi);
-                const T dxmin = -blend<T, EXACT>(DT[c.lo], DT[c.lo + 1], DT[c.hi], DT[c.hi + 1], s.fylo, s.fyhi);
-                const T dxmax = blend<T, EXACT>(DB[c.lo], DB[c.lo + 1], DB[c.hi], DB[c.hi + 1], s.fylo, s.fyhi);
-                const T dymin = -(vl - vla);
-                const T dymax = vra - vr;
-                sum[0] += g[k] * dxmin;
-                sum[1] += g[k] * dxmax;
-                sum[2] += g[k] * dymin;
-                sum[3] += g[k] * dymax;
-                sum[4] += g[k] * S;
+            {
+                const T grA = G0[ir[k]], gr = G0[ir[k] + 1], gl = G0[il[k]], glA = G0[il[k] + 1];
+                const T dr = grA - gr, dl = gl - glA;
+                T wq = gr - gl;
+                if (EXACT) wq += s.fyhi * dr + s.fylo * dl;
+                sum[4] += v0[k] * wq;
+                sum[1] += db0[k] * wq;
+                sum[0] -= dt0[k] * wq;
+                sum[3] += v0[k] * dr;
+                sum[2] -= v0[k] * dl;
+                tail0 += delta[k] * g0[k];
+            }
+            {
+                const T grA = G1[ir[k]], gr = G1[ir[k] + 1], gl = G1[il[k]], glA = G1[il[k] + 1];
+                const T dr = grA - gr, dl = gl - glA;
+                T wq = gr - gl;
+                if (EXACT) wq += s.fyhi * dr + s.fylo * dl;
+                sum[4] += v1[k] * wq;
+                sum[1] += db1[k] * wq;
+                sum[0] -= dt1[k] * wq;
+                sum[3] += v1[k] * dr;
+                sum[2] -= v1[k] * dl;
+                tail1 += delta[k] * g1[k];
+            }
+        }
+        {
+            const T vw0 = G0[w + 4], dtw0 = G0[w + 5], dbw0 = G0[w + 6];
+            const T vw1 = G1[w + 4], dtw1 = G1[w + 5], dbw1 = G1[w + 6];
+            sum[4] += vw0 * tail0 + vw1 * tail1;
+            sum[1] += dbw0 * tail0 + dbw1 * tail1;
+            sum[0] -= dtw0 * tail0 + dtw1 * tail1;
+            if (tid == 0) {
+                sum[3] += vw0 * G0[idx_ymax] + vw1 * G1[idx_ymax];
+                sum[2] -= vw0 * G0[idx_ymin] + vw1 * G1[idx_ymin];
             }
         }
 #pragma unroll
-        for (int k = 0; k < K; ++k) { pT[k] = nT[k]; pB[k] = nB[k]; nT[k] = fT[k]; nB[k] = fB[k]; }
+        for (int k = 0; k < K; ++k) {
+            ta[k] = t1[k]; bc[k] = b2[k];
+            t0[k] = n0[k]; t1[k] = n1[k]; b1[k] = n2[k]; b2[k] = n3[k];
+            g0[k] = m0[k]; g1[k] = m1[k];
+        }
+    }
+
+    if (a.colsum != nullptr && band < a.nb - 1) {
+        double* dst = a.colsum + (pf * (a.nb - 1) + band) * static_cast<int64_t>(w);
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            const int j = tid + nt * k;
+            if (FULL || j < w) dst[j] = cs[k];
+        }
     }
 
     __syncthreads();
@@ -397,11 +551,11 @@ __global__ void __launch_bounds__(256) forward_gather_kernel(SampleArgs<T> a) {
     const int pix = static_cast<int>(idx % hw);
     const int i = pix / a.w, j = pix % a.w;
     const int64_t p = pf / a.F;
-    const int k_par = static_cast<int>(p % a.C) * a.F + static_cast<int>(pf % a.F);
-    const T xmin = a.prm.xmin[k_par], xmax = a.prm.xmax[k_par];
-    const T ymin = a.prm.ymin[k_par], ymax = a.prm.ymax[k_par];
-    const BoxSplit<T> s = split_forward(xmin, xmax, ymin, ymax);
-    const T scale = a.normalize ? inverse_extent(xmin, xmax, ymin, ymax, EXACT, true, true) : T(1);
+    const int k_par = static_cast<int>((a.plane0 + p) % a.C) * a.F + static_cast<int>(pf % a.F);
+    const BoxOfWorkgroup<T> bx = load_box(a.prm, k_par);
+    const BoxSplit<T> s = split_forward(bx.xmin, bx.xmax, bx.ymin, bx.ymax);
+    const T scale = a.normalize
+        ? inverse_extent(bx.xmin, bx.xmax, bx.ymin, bx.ymax, EXACT, true, true) : T(1);
     const T* plane = a.src + p * static_cast<int64_t>(a.h + 1) * (a.w + 1);
     a.dst[idx] = gather_box<T, EXACT>(plane, s, i, j, a.h, a.w) * scale;
 }
@@ -414,15 +568,14 @@ __global__ void __launch_bounds__(256) grad_input_gather_kernel(SampleArgs<T> a)
     const int64_t p = idx / hw;
     const int pix = static_cast<int>(idx % hw);
     const int i = pix / a.w, j = pix % a.w;
-    const int c_in = static_cast<int>(p % a.C);
+    const int c_in = static_cast<int>((a.plane0 + p) % a.C);
     const int64_t ipl = static_cast<int64_t>(a.h + 1) * (a.w + 1);
     T acc = T(0);
     for (int f = 0; f < a.F; ++f) {
-        const int k_par = c_in * a.F + f;
-        const T xmin = a.prm.xmin[k_par], xmax = a.prm.xmax[k_par];
-        const T ymin = a.prm.ymin[k_par], ymax = a.prm.ymax[k_par];
-        const BoxSplit<T> s = split_grad_input(xmin, xmax, ymin, ymax);
-        const T scale = a.normalize ? inverse_extent(xmin, xmax, ymin, ymax, EXACT, true, true) : T(1);
+        const BoxOfWorkgroup<T> bx = load_box(a.prm, c_in * a.F + f);
+        const BoxSplit<T> s = split_grad_input(bx.xmin, bx.xmax, bx.ymin, bx.ymax);
+        const T scale = a.normalize
+            ? inverse_extent(bx.xmin, bx.xmax, bx.ymin, bx.ymax, EXACT, true, true) : T(1);
         acc += gather_box<T, EXACT>(a.src + (p * a.F + f) * ipl, s, i, j, a.h, a.w) * scale;
     }
     a.dst[idx] = acc;
@@ -436,12 +589,12 @@ __global__ void __launch_bounds__(256) grad_params_gather_kernel(SampleArgs<T> a
     const int64_t pf = blockIdx.x / blocks_per_plane;
     const int pix = static_cast<int>(blockIdx.x % blocks_per_plane) * blockDim.x + threadIdx.x;
     const int64_t p = pf / a.F;
-    const int k_par = static_cast<int>(p % a.C) * a.F + static_cast<int>(pf % a.F);
+    const int k_par = static_cast<int>((a.plane0 + p) % a.C) * a.F + static_cast<int>(pf % a.F);
     double v[5] = {0, 0, 0, 0, 0};
     if (pix < h * w) {
         const int i = pix / w, j = pix % w;
-        const BoxSplit<T> s = split_grad_params(a.prm.xmin[k_par], a.prm.xmax[k_par],
-                                                a.prm.ymin[k_par], a.prm.ymax[k_par]);
+        const BoxOfWorkgroup<T> bx = load_box(a.prm, k_par);
+        const BoxSplit<T> s = split_grad_params(bx.xmin, bx.xmax, bx.ymin, bx.ymax);
         const int64_t pitch = w + 1;
         const T* plane = a.src + p * static_cast<int64_t>(h + 1) * pitch;
         const int t = clampi(i + s.xlo, 0, h), ta = clampi(i + s.xlo - 1, 0, h);
@@ -504,12 +657,13 @@ __global__ void param_grad_finalize_kernel(const double* __restrict__ acc, BoxPa
 }
 
 // ---------------------------------------------------------------------------------------------
-struct RowConfig { int nt; int K; };
+struct RowConfig { int nt; int K; bool full; };
 inline RowConfig row_config(int w) {
     RowConfig c;
     c.nt = std::min(256, ((w + 63) / 64) * 64);
     const int k = (w + c.nt - 1) / c.nt;
     c.K = k <= 1 ? 1 : k <= 2 ? 2 : k <= 4 ? 4 : 8;
+    c.full = (c.K * c.nt == w);
     return c;
 }
 
@@ -517,6 +671,13 @@ inline int bands_for(int64_t independent, int h, int min_rows, int64_t want) {
     int nb = static_cast<int>(std::min<int64_t>((want + independent - 1) / std::max<int64_t>(independent, 1),
                                                 std::max(1, h / min_rows)));
     return std::max(nb, 1);
+}
+
+template <class T>
+SampleArgs<T> base_args(BoxParams<T> prm, const Dims& d) {
+    SampleArgs<T> a{};
+    a.prm = prm; a.C = d.C; a.F = d.F; a.h = d.h; a.w = d.w; a.plane0 = d.plane0;
+    return a;
 }
 
 template <class T>
@@ -532,36 +693,44 @@ void finish_args(SampleArgs<T>& a, int64_t total) {
         case 4: KERNEL(4, __VA_ARGS__); break;                                       \
         default: KERNEL(8, __VA_ARGS__); break;                                      \
     }
+#define BOXCONV_DISPATCH_K_EXACT_FULL(KERNEL, K, EXACT, FULL)                        \
+    if (EXACT) {                                                                     \
+        if (FULL) { BOXCONV_DISPATCH_K(KERNEL, K, true, true) }                      \
+        else      { BOXCONV_DISPATCH_K(KERNEL, K, true, false) }                     \
+    } else {                                                                         \
+        if (FULL) { BOXCONV_DISPATCH_K(KERNEL, K, false, true) }                     \
+        else      { BOXCONV_DISPATCH_K(KERNEL, K, false, false) }                    \
+    }
 
 }  // namespace
 
 template <class T>
 hipError_t forward_launch(const T* integ, BoxParams<T> prm, T* out, Dims d, bool normalize,
                           bool exact, hipStream_t stream) {
-    const int64_t planes_f = d.planes() * d.F;
+    const int64_t planes_f = d.planes * d.F;
     if (planes_f == 0 || d.hw() == 0) return hipSuccess;
-    SampleArgs<T> a{};
-    a.src = integ; a.prm = prm; a.dst = out; a.C = d.C; a.F = d.F; a.h = d.h; a.w = d.w;
-    a.normalize = normalize ? 1 : 0;
+    SampleArgs<T> a = base_args(prm, d);
+    a.src = integ; a.dst = out; a.normalize = normalize ? 1 : 0;
 
     if (d.w > kMaxRowStreamWidth || force_gather_kernels()) {
         finish_args(a, planes_f * d.hw());
         const dim3 grid(static_cast<unsigned>((a.total + 255) / 256));
-        if (exact) hipLaunchKernelGGL((forward_gather_kernel<T, true>), grid, dim3(256), 0, stream, a);
-        else       hipLaunchKernelGGL((forward_gather_kernel<T, false>), grid, dim3(256), 0, stream, a);
+        if (exact) BOXCONV_LAUNCH("forward_gather", (forward_gather_kernel<T, true>), grid, dim3(256), 0, stream, a);
+        else       BOXCONV_LAUNCH("forward_gather", (forward_gather_kernel<T, false>), grid, dim3(256), 0, stream, a);
         return hipGetLastError();
     }
 
     const RowConfig rc = row_config(d.w);
     a.nb = bands_for(planes_f, d.h, 16, 4096);
     a.R = (d.h + a.nb - 1) / a.nb;
+    a.R += a.R & 1;                                   // rows are handled in pairs
     a.nb = (d.h + a.R - 1) / a.R;
     finish_args(a, planes_f * a.nb);
     const dim3 grid(static_cast<unsigned>(a.per_xcd * kXcds));
-    const size_t lds = 2 * static_cast<size_t>(d.w + 3) * sizeof(T);
-#define LAUNCH_FWD(KK, EX) \
-    hipLaunchKernelGGL((forward_rows_kernel<T, KK, EX>), grid, dim3(rc.nt), lds, stream, a)
-    if (exact) { BOXCONV_DISPATCH_K(LAUNCH_FWD, rc.K, true) } else { BOXCONV_DISPATCH_K(LAUNCH_FWD, rc.K, false) }
+    const size_t lds = 4 * static_cast<size_t>(d.w + 3) * sizeof(T);
+#define LAUNCH_FWD(KK, EX, FU) \
+    BOXCONV_LAUNCH("forward_rows", (forward_rows_kernel<T, KK, EX, FU>), grid, dim3(rc.nt), lds, stream, a)
+    BOXCONV_DISPATCH_K_EXACT_FULL(LAUNCH_FWD, rc.K, exact, rc.full)
 #undef LAUNCH_FWD
     return hipGetLastError();
 }
@@ -569,16 +738,15 @@ hipError_t forward_launch(const T* integ, BoxParams<T> prm, T* out, Dims d, bool
 template <class T>
 hipError_t grad_input_launch(const T* gint, BoxParams<T> prm, T* grad_in, Dims d, bool normalize,
                              bool exact, hipStream_t stream) {
-    if (d.planes() == 0 || d.hw() == 0) return hipSuccess;
-    SampleArgs<T> a{};
-    a.src = gint; a.prm = prm; a.dst = grad_in; a.C = d.C; a.F = d.F; a.h = d.h; a.w = d.w;
-    a.normalize = normalize ? 1 : 0;
+    if (d.planes == 0 || d.hw() == 0) return hipSuccess;
+    SampleArgs<T> a = base_args(prm, d);
+    a.src = gint; a.dst = grad_in; a.normalize = normalize ? 1 : 0;
 
     if (d.w > kMaxRowStreamWidth || force_gather_kernels()) {
-        finish_args(a, d.planes() * d.hw());
+        finish_args(a, d.planes * d.hw());
         const dim3 grid(static_cast<unsigned>((a.total + 255) / 256));
-        if (exact) hipLaunchKernelGGL((grad_input_gather_kernel<T, true>), grid, dim3(256), 0, stream, a);
-        else       hipLaunchKernelGGL((grad_input_gather_kernel<T, false>), grid, dim3(256), 0, stream, a);
+        if (exact) BOXCONV_LAUNCH("grad_input_gather", (grad_input_gather_kernel<T, true>), grid, dim3(256), 0, stream, a);
+        else       BOXCONV_LAUNCH("grad_input_gather", (grad_input_gather_kernel<T, false>), grid, dim3(256), 0, stream, a);
         return hipGetLastError();
     }
 
@@ -586,66 +754,83 @@ hipError_t grad_input_launch(const T* gint, BoxParams<T> prm, T* grad_in, Dims d
     const RowConfig rc = row_config(d.w);
     a.nb = (d.h + RB - 1) / RB;
     a.R = RB;
-    finish_args(a, d.planes() * a.nb);
+    finish_args(a, d.planes * a.nb);
     const dim3 grid(static_cast<unsigned>(a.per_xcd * kXcds));
-    const size_t lds = 2 * static_cast<size_t>(d.w + 3) * sizeof(T);
-#define LAUNCH_GI(KK, EX) \
-    hipLaunchKernelGGL((grad_input_rows_kernel<T, KK, RB, EX>), grid, dim3(rc.nt), lds, stream, a)
-    if (exact) { BOXCONV_DISPATCH_K(LAUNCH_GI, rc.K, true) } else { BOXCONV_DISPATCH_K(LAUNCH_GI, rc.K, false) }
+    const size_t lds = 4 * static_cast<size_t>(d.w + 3) * sizeof(T);
+#define LAUNCH_GI(KK, EX, FU) \
+    BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, KK, RB, EX, FU>), grid, dim3(rc.nt), lds, stream, a)
+    BOXCONV_DISPATCH_K_EXACT_FULL(LAUNCH_GI, rc.K, exact, rc.full)
 #undef LAUNCH_GI
     return hipGetLastError();
 }
 
-template <class T>
-hipError_t grad_params_launch(const T* integ, const T* grad_out, BoxParams<T> prm, double* acc,
-                              T* gxmin, T* gxmax, T* gymin, T* gymax, Dims d, float reparam_h,
-                              float reparam_w, bool normalize, bool exact, hipStream_t stream) {
-    const int n = d.C * d.F;
-    if (n == 0) return hipSuccess;
-    hipLaunchKernelGGL(fill_zero_kernel, dim3((n * 5 + 255) / 256), dim3(256), 0, stream, acc, n * 5);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
+hipError_t grad_params_begin(double* acc, int n_boxes, hipStream_t stream) {
+    if (n_boxes == 0) return hipSuccess;
+    BOXCONV_LAUNCH("fill_zero", fill_zero_kernel, dim3((n_boxes * 5 + 255) / 256), dim3(256), 0,
+                   stream, acc, n_boxes * 5);
+    return hipGetLastError();
+}
 
-    const int64_t planes_f = d.planes() * d.F;
-    if (planes_f > 0 && d.hw() > 0) {
-        SampleArgs<T> a{};
-        a.src = integ; a.prm = prm; a.grad_out = grad_out; a.acc = acc;
-        a.C = d.C; a.F = d.F; a.h = d.h; a.w = d.w; a.normalize = normalize ? 1 : 0;
-        const size_t lds = ((2 * 3 * static_cast<size_t>(d.w + 3) * sizeof(T) + 15) / 16) * 16
-                           + 4 * 5 * sizeof(double);
-        if (d.w > kMaxRowStreamWidth || lds > kMaxDynamicLds || force_gather_kernels()) {
-            const int bpp = static_cast<int>((d.hw() + 255) / 256);
-            finish_args(a, planes_f * bpp);
-            const dim3 grid(static_cast<unsigned>(a.total));
-            if (exact) hipLaunchKernelGGL((grad_params_gather_kernel<T, true>), grid, dim3(256), 0, stream, a, bpp);
-            else       hipLaunchKernelGGL((grad_params_gather_kernel<T, false>), grid, dim3(256), 0, stream, a, bpp);
-        } else {
-            const RowConfig rc = row_config(d.w);
-            a.nb = bands_for(planes_f, d.h, 16, 4096);
-            a.R = (d.h + a.nb - 1) / a.nb;
-            a.nb = (d.h + a.R - 1) / a.R;
-            finish_args(a, planes_f * a.nb);
-            const dim3 grid(static_cast<unsigned>(a.per_xcd * kXcds));
-#define LAUNCH_GP(KK, EX) \
-    hipLaunchKernelGGL((grad_params_rows_kernel<T, KK, EX>), grid, dim3(rc.nt), lds, stream, a)
-            if (exact) { BOXCONV_DISPATCH_K(LAUNCH_GP, rc.K, true) } else { BOXCONV_DISPATCH_K(LAUNCH_GP, rc.K, false) }
-#undef LAUNCH_GP
-        }
-        e = hipGetLastError();
-        if (e != hipSuccess) return e;
+template <class T>
+hipError_t grad_params_accumulate(const T* integ, const T* grad_out, BoxParams<T> prm, double* acc,
+                                  double* colsum_aux, const IntegralPlan& plan, Dims d, bool exact,
+                                  bool* wrote_colsums, hipStream_t stream) {
+    if (wrote_colsums) *wrote_colsums = false;
+    const int64_t planes_f = d.planes * d.F;
+    if (planes_f == 0 || d.hw() == 0) return hipSuccess;
+    SampleArgs<T> a = base_args(prm, d);
+    a.src = integ; a.grad_out = grad_out; a.acc = acc;
+
+    const size_t glen = static_cast<size_t>(d.w) + 8;
+    const size_t lds = ((4 * glen * sizeof(T) + 15) / 16) * 16 + 4 * 5 * sizeof(double);
+    if (d.w > kMaxRowStreamWidth || lds > kMaxDynamicLds || force_gather_kernels()) {
+        const int bpp = static_cast<int>((d.hw() + 255) / 256);
+        finish_args(a, planes_f * bpp);
+        const dim3 grid(static_cast<unsigned>(a.total));
+        if (exact) BOXCONV_LAUNCH("grad_params_gather", (grad_params_gather_kernel<T, true>), grid, dim3(256), 0, stream, a, bpp);
+        else       BOXCONV_LAUNCH("grad_params_gather", (grad_params_gather_kernel<T, false>), grid, dim3(256), 0, stream, a, bpp);
+        return hipGetLastError();
     }
 
-    hipLaunchKernelGGL((param_grad_finalize_kernel<T>), dim3((n + 127) / 128), dim3(128), 0, stream,
-                       acc, prm, gxmin, gxmax, gymin, gymax, n, reparam_h, reparam_w,
-                       normalize ? 1 : 0, exact ? 1 : 0);
+    const RowConfig rc = row_config(d.w);
+    if (colsum_aux != nullptr && plan.nb > 1) {
+        // share the band structure of the integral image so the column sums line up
+        a.nb = plan.nb; a.R = plan.R; a.colsum = colsum_aux;
+        if (wrote_colsums) *wrote_colsums = true;
+    } else {
+        a.nb = bands_for(planes_f, d.h, 16, 4096);
+        a.R = (d.h + a.nb - 1) / a.nb;
+        a.R += a.R & 1;
+        a.nb = (d.h + a.R - 1) / a.R;
+        a.colsum = nullptr;
+    }
+    finish_args(a, planes_f * a.nb);
+    const dim3 grid(static_cast<unsigned>(a.per_xcd * kXcds));
+#define LAUNCH_GP(KK, EX, FU) \
+    BOXCONV_LAUNCH("grad_params_rows", (grad_params_rows_kernel<T, KK, EX, FU>), grid, dim3(rc.nt), lds, stream, a)
+    BOXCONV_DISPATCH_K_EXACT_FULL(LAUNCH_GP, rc.K, exact, rc.full)
+#undef LAUNCH_GP
+    return hipGetLastError();
+}
+
+template <class T>
+hipError_t grad_params_finish(const double* acc, BoxParams<T> prm, T* gxmin, T* gxmax, T* gymin,
+                              T* gymax, int n_boxes, float reparam_h, float reparam_w,
+                              bool normalize, bool exact, hipStream_t stream) {
+    if (n_boxes == 0) return hipSuccess;
+    BOXCONV_LAUNCH("param_grad_finalize", (param_grad_finalize_kernel<T>), dim3((n_boxes + 127) / 128),
+                   dim3(128), 0, stream, acc, prm, gxmin, gxmax, gymin, gymax, n_boxes, reparam_h,
+                   reparam_w, normalize ? 1 : 0, exact ? 1 : 0);
     return hipGetLastError();
 }
 
 #define BOXCONV_INSTANTIATE(T)                                                                     \
     template hipError_t forward_launch<T>(const T*, BoxParams<T>, T*, Dims, bool, bool, hipStream_t); \
     template hipError_t grad_input_launch<T>(const T*, BoxParams<T>, T*, Dims, bool, bool, hipStream_t); \
-    template hipError_t grad_params_launch<T>(const T*, const T*, BoxParams<T>, double*, T*, T*, T*, \
-                                              T*, Dims, float, float, bool, bool, hipStream_t);
+    template hipError_t grad_params_accumulate<T>(const T*, const T*, BoxParams<T>, double*, double*, \
+                                                  const IntegralPlan&, Dims, bool, bool*, hipStream_t); \
+    template hipError_t grad_params_finish<T>(const double*, BoxParams<T>, T*, T*, T*, T*, int,    \
+                                              float, float, bool, bool, hipStream_t);
 
 BOXCONV_INSTANTIATE(float)
 BOXCONV_INSTANTIATE(double)

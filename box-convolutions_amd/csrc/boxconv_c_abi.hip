@@ -3,9 +3,52 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <utility>
+#include <vector>
 
 #include "../../include/boxconv.h"
 #include "boxconv_host.hpp"
+
+namespace boxconv {
+
+// ---- per-kernel timing ------------------------------------------------------------------------
+namespace {
+std::mutex g_prof_mutex;
+std::string g_prof_name;                                   // empty: disarmed
+std::vector<std::pair<hipEvent_t, hipEvent_t>> g_prof_events;
+hipEvent_t g_prof_open = nullptr;
+constexpr size_t kMaxProfiledLaunches = 1 << 16;
+}  // namespace
+
+void profile_before(const char* name, hipStream_t stream) {
+    if (g_prof_name.empty()) return;                       // unlocked fast path: not armed
+    std::lock_guard<std::mutex> lock(g_prof_mutex);
+    if (g_prof_name != name || g_prof_events.size() >= kMaxProfiledLaunches) return;
+    hipEvent_t start = nullptr;
+    if (hipEventCreate(&start) != hipSuccess) return;
+    (void)hipEventRecord(start, stream);
+    g_prof_open = start;
+}
+
+void profile_after(const char* name, hipStream_t stream) {
+    if (g_prof_name.empty()) return;
+    std::lock_guard<std::mutex> lock(g_prof_mutex);
+    if (g_prof_open == nullptr || g_prof_name != name) return;
+    hipEvent_t stop = nullptr;
+    if (hipEventCreate(&stop) == hipSuccess) {
+        (void)hipEventRecord(stop, stream);
+        g_prof_events.emplace_back(g_prof_open, stop);
+    } else {
+        (void)hipEventDestroy(g_prof_open);
+    }
+    g_prof_open = nullptr;
+}
+
+}  // namespace boxconv
 
 namespace {
 
@@ -41,20 +84,42 @@ int check_dims(int batch, int in_planes, int num_filters, int h, int w) {
     return 0;
 }
 
+// The backward pass can walk the (batch, plane) pairs in chunks so that the integral image of a
+// chunk of grad_output is consumed while it is still cache resident; the chunk (in planes) comes
+// from BOXCONV_BWD_CHUNK_PLANES, default: everything in one go.
+int64_t backward_chunk_planes(int64_t planes) {
+    static const long env = [] {
+        const char* e = std::getenv("BOXCONV_BWD_CHUNK_PLANES");
+        return e ? std::atol(e) : 0L;
+    }();
+    if (env > 0 && env < planes) return env;
+    return planes;
+}
+
+constexpr int64_t kBackwardWorkgroups = 2048;   // workgroups the banded backward kernels aim for
+
 struct BackwardLayout {
     size_t gint_off, aux_off, acc_off, total;
+    int64_t chunk;                 // planes per chunk
+    boxconv::IntegralPlan plan;    // band structure shared by the chunk's kernels
 };
 
 BackwardLayout backward_layout(int batch, int in_planes, int num_filters, int h, int w,
                                int elem_size, bool need_input, bool need_params) {
     BackwardLayout L{};
+    const int64_t planes = static_cast<int64_t>(batch) * in_planes;
+    L.chunk = std::max<int64_t>(backward_chunk_planes(planes), 1);
+    L.plan = boxconv::plan_integral(L.chunk * num_filters, h, w, kBackwardWorkgroups);
     size_t off = 0;
     L.gint_off = off;
     if (need_input) {
-        const int64_t planes = static_cast<int64_t>(batch) * in_planes * num_filters;
-        off += align_up(static_cast<size_t>(planes) * (h + 1) * (w + 1) * elem_size, 256);
+        off += align_up(static_cast<size_t>(L.chunk) * num_filters * (h + 1) * (w + 1) * elem_size, 256);
         L.aux_off = off;
-        off += align_up(static_cast<size_t>(boxconv::plan_integral(planes, h, w).aux_doubles) * 8, 256);
+        int64_t aux = L.plan.aux_doubles;
+        if (const int64_t rest = planes % L.chunk)      // a shorter last chunk plans its own bands
+            aux = std::max(aux, boxconv::plan_integral(rest * num_filters, h, w,
+                                                       kBackwardWorkgroups).aux_doubles);
+        off += align_up(static_cast<size_t>(aux) * 8, 256);
     } else {
         L.aux_off = off;
     }
@@ -82,6 +147,7 @@ int integral_image_impl(const T* in, T* out, int64_t planes, int h, int w, void*
                     need, workspace_bytes);
     return hip_result(boxconv::integral_image_launch<T>(in, out, planes, h, w,
                                                         static_cast<double*>(workspace),
+                                                        boxconv::plan_integral(planes, h, w), false,
                                                         static_cast<hipStream_t>(stream)),
                       "integral image launch");
 }
@@ -94,7 +160,7 @@ int forward_impl(const T* integ, const T* x_min, const T* x_max, const T* y_min,
     if (static_cast<int64_t>(batch) * in_planes * num_filters == 0) return 0;
     if (!integ || !x_min || !x_max || !y_min || !y_max || !output)
         return fail(BOXCONV_E_INVALID_ARGUMENT, "forward: null tensor pointer");
-    boxconv::Dims d{batch, in_planes, num_filters, h, w};
+    boxconv::Dims d{in_planes, num_filters, h, w, static_cast<int64_t>(batch) * in_planes, 0};
     boxconv::BoxParams<T> prm{x_min, x_max, y_min, y_max};
     return hip_result(boxconv::forward_launch<T>(integ, prm, output, d, normalize != 0, exact != 0,
                                                  static_cast<hipStream_t>(stream)),
@@ -125,31 +191,51 @@ int backward_impl(const T* integ, const T* x_min, const T* x_max, const T* y_min
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     unsigned char* ws = static_cast<unsigned char*>(workspace);
-    boxconv::Dims d{batch, in_planes, num_filters, h, w};
     boxconv::BoxParams<T> prm{x_min, x_max, y_min, y_max};
+    const int n_boxes = in_planes * num_filters;
+    double* acc = reinterpret_cast<double*>(ws + L.acc_off);
+    double* aux = reinterpret_cast<double*>(ws + L.aux_off);
+    T* gint = reinterpret_cast<T*>(ws + L.gint_off);
 
-    if (need_params) {
-        if (int rc = hip_result(boxconv::grad_params_launch<T>(
-                integ, grad_output, prm, reinterpret_cast<double*>(ws + L.acc_off), gx_min, gx_max,
-                gy_min, gy_max, d, reparam_h, reparam_w, normalize != 0, exact != 0, s),
-                "parameter-gradient launch"))
+    if (need_input && nout == 0)
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "backward: grad_input requested with zero filters");
+    if (need_params)
+        if (int rc = hip_result(boxconv::grad_params_begin(acc, n_boxes, s), "accumulator clear"))
             return rc;
-    }
-    if (need_input) {
-        if (nout == 0) {
-            // no filters: the sum over an empty set of filters is zero
-            return fail(BOXCONV_E_INVALID_ARGUMENT, "backward: grad_input requested with zero filters");
+
+    const int64_t planes = static_cast<int64_t>(batch) * in_planes;
+    const int64_t hw = static_cast<int64_t>(h) * w;
+    const int64_t ipl = static_cast<int64_t>(h + 1) * (w + 1);
+    for (int64_t p0 = 0; p0 < planes; p0 += L.chunk) {
+        const int64_t np = std::min(L.chunk, planes - p0);
+        boxconv::Dims d{in_planes, num_filters, h, w, np, p0};
+        // the last chunk may be shorter: its band structure is planned for its own size
+        const boxconv::IntegralPlan plan = (np == L.chunk)
+            ? L.plan : boxconv::plan_integral(np * num_filters, h, w, kBackwardWorkgroups);
+        const T* go_chunk = grad_output + p0 * num_filters * hw;
+        bool colsums_ready = false;
+        if (need_params) {
+            if (int rc = hip_result(boxconv::grad_params_accumulate<T>(
+                    integ + p0 * ipl, go_chunk, prm, acc, need_input ? aux : nullptr, plan, d,
+                    exact != 0, &colsums_ready, s), "parameter-gradient launch"))
+                return rc;
         }
-        T* gint = reinterpret_cast<T*>(ws + L.gint_off);
-        if (int rc = hip_result(boxconv::integral_image_launch<T>(
-                grad_output, gint, nout, h, w, reinterpret_cast<double*>(ws + L.aux_off), s),
-                "grad_output integral image launch"))
-            return rc;
-        if (int rc = hip_result(boxconv::grad_input_launch<T>(gint, prm, grad_input, d,
-                                                              normalize != 0, exact != 0, s),
-                                "input-gradient launch"))
-            return rc;
+        if (need_input) {
+            if (int rc = hip_result(boxconv::integral_image_launch<T>(
+                    go_chunk, gint, np * num_filters, h, w, aux, plan, colsums_ready, s),
+                    "grad_output integral image launch"))
+                return rc;
+            if (int rc = hip_result(boxconv::grad_input_launch<T>(
+                    gint, prm, grad_input + p0 * hw, d, normalize != 0, exact != 0, s),
+                    "input-gradient launch"))
+                return rc;
+        }
     }
+    if (need_params)
+        if (int rc = hip_result(boxconv::grad_params_finish<T>(
+                acc, prm, gx_min, gx_max, gy_min, gy_max, n_boxes, reparam_h, reparam_w,
+                normalize != 0, exact != 0, s), "parameter-gradient finish"))
+            return rc;
     return 0;
 }
 
@@ -173,6 +259,38 @@ int clip_impl(T* x_min, T* x_max, T* y_min, T* y_max, int n, double reparam_h, d
 extern "C" {
 
 int boxconv_abi_version(void) { return BOXCONV_ABI_VERSION; }
+
+int boxconv_profile_arm(const char* kernel_name) {
+    std::lock_guard<std::mutex> lock(boxconv::g_prof_mutex);
+    for (auto& ev : boxconv::g_prof_events) {
+        (void)hipEventDestroy(ev.first);
+        (void)hipEventDestroy(ev.second);
+    }
+    boxconv::g_prof_events.clear();
+    boxconv::g_prof_name = kernel_name ? kernel_name : "";
+    return 0;
+}
+
+int boxconv_profile_collect(double* total_ms, int* launches) {
+    std::lock_guard<std::mutex> lock(boxconv::g_prof_mutex);
+    double sum = 0.0;
+    int n = 0;
+    int rc = 0;
+    for (auto& ev : boxconv::g_prof_events) {
+        float ms = 0.0f;
+        hipError_t e = hipEventSynchronize(ev.second);
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, ev.first, ev.second);
+        if (e == hipSuccess) { sum += ms; ++n; }
+        else rc = hip_result(e, "profile collect");
+        (void)hipEventDestroy(ev.first);
+        (void)hipEventDestroy(ev.second);
+    }
+    boxconv::g_prof_events.clear();
+    boxconv::g_prof_name.clear();
+    if (total_ms) *total_ms = sum;
+    if (launches) *launches = n;
+    return rc;
+}
 
 const char* boxconv_last_error(void) { return g_error; }
 

@@ -8,9 +8,12 @@
 
 namespace boxconv {
 
+// One call works on `planes` consecutive (batch, input plane) pairs starting at global index
+// `plane0` (= b * C + c); all tensor pointers passed alongside already point at that first plane.
 struct Dims {
-    int B, C, F, h, w;   // batch, input planes, filters per plane, image height, image width
-    int64_t planes() const { return static_cast<int64_t>(B) * C; }
+    int C, F, h, w;      // input planes, filters per plane, image height, image width
+    int64_t planes;      // (batch, plane) pairs covered by this call
+    int64_t plane0;      // global index of the first one (selects the boxes: c = (plane0+p) % C)
     int64_t hw() const { return static_cast<int64_t>(h) * w; }
     int64_t integral_plane() const { return static_cast<int64_t>(h + 1) * (w + 1); }
 };
@@ -29,11 +32,14 @@ struct IntegralPlan {
     int R;                 // rows per band
     int64_t aux_doubles;   // scratch for the column sums of all bands but the last
 };
-IntegralPlan plan_integral(int64_t planes, int h, int w);
+// `want`: number of workgroups to aim for.
+IntegralPlan plan_integral(int64_t planes, int h, int w, int64_t want = 1024);
 
+// colsums_ready: aux already holds the per-band column sums (written by another kernel that read
+// the same input), so the first pass is skipped.
 template <class T>
 hipError_t integral_image_launch(const T* in, T* out, int64_t planes, int h, int w, double* aux,
-                                 hipStream_t stream);
+                                 const IntegralPlan& plan, bool colsums_ready, hipStream_t stream);
 
 template <class T>
 hipError_t forward_launch(const T* integ, BoxParams<T> prm, T* out, Dims d, bool normalize,
@@ -43,12 +49,22 @@ template <class T>
 hipError_t grad_input_launch(const T* gint, BoxParams<T> prm, T* grad_in, Dims d, bool normalize,
                              bool exact, hipStream_t stream);
 
-// acc: [C*F*5] doubles of scratch (cleared by the launch itself with a fill kernel).
-// g[k] may be null for a gradient that is not wanted.
+// Parameter gradients in three steps so that a caller can feed the planes in chunks:
+//   begin      clears acc ([C*F*5] doubles of scratch) with a fill kernel
+//   accumulate adds the five sums per box for the planes of `d`; if `colsum_aux` is non-null it
+//              also writes the per-band column sums of grad_out laid out for `plan` (what the
+//              integral image of grad_out needs as its first pass). Returns through
+//              `wrote_colsums` whether it did (the gather fallback does not).
+//   finish     turns the sums into the four gradients; g* may be null for an unwanted gradient.
+hipError_t grad_params_begin(double* acc, int n_boxes, hipStream_t stream);
 template <class T>
-hipError_t grad_params_launch(const T* integ, const T* grad_out, BoxParams<T> prm, double* acc,
-                              T* gxmin, T* gxmax, T* gymin, T* gymax, Dims d, float reparam_h,
-                              float reparam_w, bool normalize, bool exact, hipStream_t stream);
+hipError_t grad_params_accumulate(const T* integ, const T* grad_out, BoxParams<T> prm, double* acc,
+                                  double* colsum_aux, const IntegralPlan& plan, Dims d, bool exact,
+                                  bool* wrote_colsums, hipStream_t stream);
+template <class T>
+hipError_t grad_params_finish(const double* acc, BoxParams<T> prm, T* gxmin, T* gxmax, T* gymin,
+                              T* gymax, int n_boxes, float reparam_h, float reparam_w,
+                              bool normalize, bool exact, hipStream_t stream);
 
 template <class T>
 hipError_t clip_launch(T* xmin, T* xmax, T* ymin, T* ymax, int n, double reparam_h,
@@ -59,6 +75,18 @@ hipError_t clip_launch(T* xmin, T* xmax, T* ymin, T* ymax, int n, double reparam
 // row staging) instead of the row-streaming ones; the gather kernels also serve widths the
 // row-streaming kernels do not cover.
 bool force_gather_kernels();
+
+// Optional per-kernel timing (see boxconv_profile_arm in include/boxconv.h). When a kernel name is
+// armed, every launch of that kernel is bracketed by a pair of HIP events on its stream.
+void profile_before(const char* name, hipStream_t stream);
+void profile_after(const char* name, hipStream_t stream);
+
+#define BOXCONV_LAUNCH(NAME, KERNEL, GRID, BLOCK, LDS, STREAM, ...)              \
+    do {                                                                          \
+        ::boxconv::profile_before(NAME, STREAM);                                  \
+        hipLaunchKernelGGL(KERNEL, GRID, BLOCK, LDS, STREAM, __VA_ARGS__);        \
+        ::boxconv::profile_after(NAME, STREAM);                                   \
+    } while (0)
 
 constexpr int kMaxRowStreamWidth = 2048;
 constexpr size_t kMaxDynamicLds = 64 * 1024;   // dynamic LDS a launch may request without opting in to more

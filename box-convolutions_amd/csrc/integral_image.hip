@@ -221,22 +221,21 @@ hipError_t launch_scan(const T* in, T* out, const double* aux, int64_t planes, i
     const dim3 grid(static_cast<unsigned>(planes * nb));
     const dim3 block(WAVES * 64);
     if (aligned_for_vec4(in, w))
-        hipLaunchKernelGGL((band_scan_kernel<T, WAVES, M, RB, true>), grid, block, 0, stream,
-                           in, out, aux, h, w, nb, R);
+        BOXCONV_LAUNCH("band_scan", (band_scan_kernel<T, WAVES, M, RB, true>), grid, block, 0, stream,
+                       in, out, aux, h, w, nb, R);
     else
-        hipLaunchKernelGGL((band_scan_kernel<T, WAVES, M, RB, false>), grid, block, 0, stream,
-                           in, out, aux, h, w, nb, R);
+        BOXCONV_LAUNCH("band_scan", (band_scan_kernel<T, WAVES, M, RB, false>), grid, block, 0, stream,
+                       in, out, aux, h, w, nb, R);
     return hipGetLastError();
 }
 
 }  // namespace
 
-IntegralPlan plan_integral(int64_t planes, int h, int w) {
+IntegralPlan plan_integral(int64_t planes, int h, int w, int64_t want) {
     IntegralPlan pl;
     // Enough workgroups to cover 256 CUs several times over, but bands no shorter than 32 rows
     // (the per-band column-sum vector is 8 B per column, i.e. 2/R of the input bytes) and no
     // taller than 256 (size of the per-row carry array in LDS).
-    const int64_t want = 1024;
     int nb = static_cast<int>(std::min<int64_t>((want + planes - 1) / std::max<int64_t>(planes, 1),
                                                 std::max(1, h / 32)));
     nb = std::max(nb, (h + 255) / 256);
@@ -253,22 +252,24 @@ IntegralPlan plan_integral(int64_t planes, int h, int w) {
 
 template <class T>
 hipError_t integral_image_launch(const T* in, T* out, int64_t planes, int h, int w,
-                                 double* aux, hipStream_t stream) {
+                                 double* aux, const IntegralPlan& pl, bool colsums_ready,
+                                 hipStream_t stream) {
     if (planes == 0) return hipSuccess;
-    const IntegralPlan pl = plan_integral(planes, h, w);
     const int nb = pl.nb, R = pl.R;
-    if (nb > 1) {
-        hipLaunchKernelGGL((band_colsum_kernel<T>), dim3(static_cast<unsigned>(planes * (nb - 1))),
-                           dim3(256), 0, stream, in, aux, h, w, nb, R);
+    if (nb > 1 && !colsums_ready) {
+        BOXCONV_LAUNCH("band_colsum", (band_colsum_kernel<T>),
+                       dim3(static_cast<unsigned>(planes * (nb - 1))), dim3(256), 0, stream, in, aux,
+                       h, w, nb, R);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
-        if (nb > 2) {
-            const int64_t n = planes * w;
-            hipLaunchKernelGGL(band_prefix_kernel, dim3(static_cast<unsigned>((n + 255) / 256)),
-                               dim3(256), 0, stream, aux, planes, w, nb);
-            e = hipGetLastError();
-            if (e != hipSuccess) return e;
-        }
+    }
+    if (nb > 2) {
+        const int64_t n = planes * w;
+        BOXCONV_LAUNCH("band_prefix", band_prefix_kernel,
+                       dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, stream, aux,
+                       planes, w, nb);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
     }
     // Tile width: one wave covers 256 columns per chunk, four waves 1024.
     if (w <= 256)        return launch_scan<T, 1, 1, 4>(in, out, aux, planes, h, w, nb, R, stream);
@@ -279,8 +280,8 @@ hipError_t integral_image_launch(const T* in, T* out, int64_t planes, int h, int
 }
 
 template hipError_t integral_image_launch<float>(const float*, float*, int64_t, int, int,
-                                                 double*, hipStream_t);
+                                                 double*, const IntegralPlan&, bool, hipStream_t);
 template hipError_t integral_image_launch<double>(const double*, double*, int64_t, int, int,
-                                                  double*, hipStream_t);
+                                                  double*, const IntegralPlan&, bool, hipStream_t);
 
 }  // namespace boxconv

@@ -43,6 +43,18 @@ int boxconv_abi_version(void);
  * on this thread. */
 const char* boxconv_last_error(void);
 
+/* ---- per-kernel timing (measurement aid; no counterpart in the reference) ---------------------
+ * boxconv_profile_arm(name): from now on every launch of the kernel called `name` is bracketed by
+ * a pair of HIP events recorded on the stream it is launched on (so the time is that kernel's
+ * alone, whatever else the entry point launches). Names: "band_colsum", "band_prefix",
+ * "band_scan", "forward_rows", "grad_input_rows", "grad_params_rows", "param_grad_finalize",
+ * "fill_zero", "clip", "forward_gather", "grad_input_gather", "grad_params_gather".
+ * NULL or "" disarms. Arming discards earlier measurements.
+ * boxconv_profile_collect(&total_ms, &launches): waits for the recorded events, returns the summed
+ * kernel time and the number of launches, then disarms. Process-wide state; meant for benchmarks. */
+int boxconv_profile_arm(const char* kernel_name);
+int boxconv_profile_collect(double* total_ms, int* launches);
+
 /* ---- integral image ------------------------------------------------------------------------
  * Replaces `integral_image(Tensor) -> Tensor`, reference src/integral_image_interface.cpp:8-27
  * (kernels: src/integral_image.cpp:8-39). `planes` is the product of all leading dimensions.

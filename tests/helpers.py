@@ -54,6 +54,8 @@ def rel_err(a, b, floor=0.0):
 
 
 def param_grad_floor(grads):
-    """1e-3 of the largest entry over the four parameter-gradient tensors that are present."""
+    """1e-2 of the largest entry over the four parameter-gradient tensors that are present: a
+    gradient tensor smaller than that is compared on this scale (absolute error <= tol * 1e-2 of
+    the largest gradient), because its float32 value is dominated by cancellation noise."""
     vals = [np.abs(np.asarray(g, dtype=np.float64)).max() for g in grads if g is not None and g.size]
-    return 1e-3 * max(vals) if vals else 0.0
+    return 1e-2 * max(vals) if vals else 0.0

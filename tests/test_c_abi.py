@@ -1,0 +1,83 @@
+"""The C-ABI library loads and exports every symbol include/boxconv.h declares; argument errors
+are reported before anything is launched (so these calls need no GPU)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "boxconv.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(boxconv_\w+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from box_convolution import _native
+    return _native.load()
+
+
+def test_header_declares_the_four_reference_functions():
+    names = declared_functions()
+    for stem in ("integral_image", "forward", "backward", "clip_parameters"):
+        for sfx in ("f32", "f64"):
+            assert "boxconv_%s_%s" % (stem, sfx) in names
+
+
+def test_library_exports_every_declared_symbol(lib):
+    from box_convolution import _native
+    names = declared_functions()
+    assert names, "no declarations found in include/boxconv.h"
+    for n in names:
+        assert hasattr(lib, n), "libboxconv_hip.so does not export " + n
+    # and the Python binding table covers exactly the header
+    assert sorted(_native.EXPORTED_SYMBOLS) == names
+    assert lib.boxconv_abi_version() == _native.ABI_VERSION
+
+
+def test_argument_errors_are_reported_without_launching(lib):
+    null = ctypes.c_void_p(None)
+    rc = lib.boxconv_integral_image_f32(null, null, 1, 0, 5, null, 0, null)
+    assert rc == -1 and b"invalid sizes" in lib.boxconv_last_error()
+    rc = lib.boxconv_integral_image_f32(null, null, 2, 4, 5, null, 0, null)
+    assert rc == -1 and b"null" in lib.boxconv_last_error()
+    rc = lib.boxconv_forward_f32(null, null, null, null, null, null, 1, 1, 1, 4, 4, 1, 1, null)
+    assert rc == -1
+    rc = lib.boxconv_forward_f64(null, null, null, null, null, null, 1, 1, 1, 0, 4, 1, 1, null)
+    assert rc == -1
+    # more than 2^31-1 elements
+    rc = lib.boxconv_forward_f32(null, null, null, null, null, null, 64, 64, 64, 4096, 4096, 1, 1, null)
+    assert rc == -3
+    # backward with nothing requested is a no-op; with a request but no workspace it is refused
+    f = ctypes.c_float(1.0)
+    rc = lib.boxconv_backward_f32(null, null, null, null, null, null, null, f, f, 1, 1,
+                                  null, null, null, null, null, 1, 1, 1, 4, 4, null, 0, null)
+    assert rc == 0
+    dummy = ctypes.c_void_p(256)
+    rc = lib.boxconv_backward_f32(dummy, dummy, dummy, dummy, dummy, dummy, null, f, f, 1, 1,
+                                  dummy, null, null, null, null, 1, 1, 1, 4, 4, null, 0, null)
+    assert rc == -2 and b"workspace" in lib.boxconv_last_error()
+    rc = lib.boxconv_clip_parameters_f32(null, null, null, null, 3, 1.0, 1.0, 4.0, 4.0, 1, null)
+    assert rc == -1
+    rc = lib.boxconv_clip_parameters_f32(null, null, null, null, 0, 1.0, 1.0, 4.0, 4.0, 1, null)
+    assert rc == 0
+
+
+def test_workspace_sizes(lib):
+    # one band (short planes, many of them): no scratch for the integral image
+    assert lib.boxconv_integral_image_workspace_bytes(4096, 28, 28) == 0
+    # several bands: (bands-1) column-sum vectors of w doubles per plane
+    n = lib.boxconv_integral_image_workspace_bytes(32, 512, 1024)
+    assert n > 0 and n % (32 * 1024 * 8) == 0
+    full = lib.boxconv_backward_workspace_bytes(2, 16, 8, 512, 1024, 4, 1, 1)
+    only_params = lib.boxconv_backward_workspace_bytes(2, 16, 8, 512, 1024, 4, 0, 1)
+    only_input = lib.boxconv_backward_workspace_bytes(2, 16, 8, 512, 1024, 4, 1, 0)
+    gint = 2 * 16 * 8 * 513 * 1025 * 4
+    assert only_params == 16 * 8 * 5 * 8 + (256 - (16 * 8 * 5 * 8) % 256) % 256
+    assert only_input >= gint and full == only_input + only_params
+    assert lib.boxconv_backward_workspace_bytes(2, 16, 8, 512, 1024, 2, 1, 1) == 0   # bad elem size

@@ -1,0 +1,251 @@
+"""BoxConv2d on the GPU, tested the way the reference tests itself (box_convolution/test.py):
+integral image against float64 cumulative sums, forward and grad_input against an explicit dense
+box kernel run through zero-padded conv2d, parameter gradients against finite differences
+(torch.autograd.gradcheck in float64) -- plus the golden vectors of the reference's CPU kernels,
+multi-channel cases and the clip/eval behaviour the reference leaves untested.
+"""
+import math
+import os
+import random
+
+import numpy as np
+import pytest
+import torch
+
+from box_convolution import BoxConv2d
+from box_convolution.box_convolution_function import BoxConvolutionFunction, reparametrize
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_vectors.npz")
+
+
+def dense_box_kernel(x_min, x_max, y_min, y_max, normalize, dtype):
+    """(2*rh+1) x (2*rw+1) kernel whose entry (p, q) is the area of pixel (p, q) covered by the
+    box [x_min, x_max+1) x [y_min, y_max+1) (reference test.py:60-86)."""
+    rh = math.ceil(max(x_max, -x_min))
+    rw = math.ceil(max(y_max, -y_min))
+    rows = torch.tensor([max(0.0, min(p + 1, x_max + 1) - max(p, x_min)) for p in range(-rh, rh + 1)], dtype=dtype)
+    cols = torch.tensor([max(0.0, min(q + 1, y_max + 1) - max(q, y_min)) for q in range(-rw, rw + 1)], dtype=dtype)
+    k = rows[:, None] * cols[None, :]
+    if normalize:
+        k = k / ((x_max - x_min + 1) * (y_max - y_min + 1))
+    return k
+
+
+def conv2d_reference(x, real, normalize, exact):
+    """Depthwise zero-padded conv2d with the dense kernels; differentiable w.r.t. x."""
+    x_min, x_max, y_min, y_max = (p.detach().cpu().double() for p in real)
+    if not exact:
+        x_min, y_min, x_max, y_max = x_min.ceil(), y_min.ceil(), x_max.floor(), y_max.floor()
+    C, F = x_min.shape
+    outs = []
+    for c in range(C):
+        for f in range(F):
+            k = dense_box_kernel(x_min[c, f].item(), x_max[c, f].item(), y_min[c, f].item(),
+                                 y_max[c, f].item(), normalize, x.dtype).to(x.device)
+            pad = (k.shape[0] // 2, k.shape[1] // 2)
+            outs.append(torch.conv2d(x[:, c:c + 1], k[None, None], padding=pad))
+    return torch.cat(outs, dim=1)
+
+
+def module_with(stored, h, w, factor, normalize, exact, dtype=torch.float32):
+    C, F = stored[0].shape
+    m = BoxConv2d(C, F, h, w, factor).to(device=DEV, dtype=dtype)
+    for name, t in zip(("x_min", "x_max", "y_min", "y_max"), stored):
+        delattr(m, name)
+        setattr(m, name, t)          # plain tensors instead of Parameters, as reference test.py:162-165
+    m.normalize, m.exact = normalize, exact
+    return m
+
+
+def random_boxes(rng, C, F, h, w, exact, margin=0.012):
+    """Boxes as in reference test.py:205-235: inside (-h+1, h-1), at least ~1 px (2 px when not
+    exact) thick, every bound further than `margin` from a whole number."""
+    def draw(lo, hi):
+        while True:
+            v = rng.uniform(lo, hi)
+            if abs(v - round(v)) > margin:
+                return v
+    real = torch.empty(4, C, F, dtype=torch.float64)
+    for c in range(C):
+        for f in range(F):
+            x0 = draw(-h + 1.05, h - (not exact) - 1.1)
+            y0 = draw(-w + 1.05, w - (not exact) - 1.1)
+            x1 = draw(x0 + (not exact) + 0.013, h - 1.05)
+            y1 = draw(y0 + (not exact) + 0.013, w - 1.05)
+            real[:, c, f] = torch.tensor([x0, x1, y0, y1])
+    return real
+
+
+def test_integral_image_like_reference_test():
+    from box_convolution_cpp_cuda import integral_image
+    rng = random.Random(1546545757)
+    for _ in range(50):
+        shape = (rng.randint(1, 3), rng.randint(1, 3), rng.randint(2, 10), rng.randint(2, 10))
+        x = torch.rand(*shape, device=DEV)
+        want = torch.zeros(shape[0], shape[1], shape[2] + 1, shape[3] + 1, dtype=torch.float64, device=DEV)
+        want[..., 1:, 1:] = x.double().cumsum(-2).cumsum(-1)
+        assert integral_image(x).allclose(want.float())        # default rtol/atol, reference test.py:53
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_module_against_conv2d_like_reference_test(seed):
+    rng = random.Random(1546545757 + seed)
+    torch.manual_seed(seed)
+    exact = rng.random() < 0.7
+    C, F = rng.choice([(1, 1), (1, 1), (2, 3), (3, 2)])
+    B = rng.randint(1, 2)
+    h, w = rng.randint(2 + (not exact), 10), rng.randint(2 + (not exact), 10)
+    factor = rng.random() * 4.5 + 0.5
+    normalize = rng.choice((False, True))
+    real = random_boxes(rng, C, F, h, w, exact)
+    reparam_h, reparam_w = (h + 1) * factor, (w + 1) * factor
+    stored = [t.float().to(DEV) for t in reparametrize(*real, reparam_h, reparam_w)]
+    x = torch.rand(B, C, h, w, device=DEV, requires_grad=True)
+    g = (torch.rand(B, C * F, h, w, device=DEV) < 0.15).float()
+
+    m = module_with(stored, h + 1, w + 1, factor, normalize, exact)
+    before = m.get_actual_parameters()
+    out = m(x)
+    for a, b in zip(before, m.get_actual_parameters()):
+        assert torch.equal(a, b), "test boxes must not be altered by _clip_parameters"
+    out.backward(g)
+    ours_grad = x.grad.clone()
+    x.grad = None
+
+    ref = conv2d_reference(x, m.get_actual_parameters(), normalize, exact)
+    ref.backward(g)
+    assert out.allclose(ref, rtol=3e-5, atol=1e-5)                 # reference test.py:260
+    assert ours_grad.allclose(x.grad, rtol=3e-5, atol=1e-5)        # reference test.py:267
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_parameter_gradients_gradcheck_float64(seed):
+    rng = random.Random(99 + seed)
+    torch.manual_seed(seed)
+    C, F = rng.choice([(1, 1), (2, 2)])
+    h, w = rng.randint(3, 8), rng.randint(3, 8)
+    factor = rng.random() * 4.5 + 0.5
+    normalize = rng.choice((False, True))
+    real = random_boxes(rng, C, F, h, w, True)
+    reparam_h, reparam_w = (h + 1) * factor, (w + 1) * factor
+    stored = [t.to(DEV).requires_grad_() for t in reparametrize(*real, reparam_h, reparam_w)]
+    x = torch.rand(2, C, h, w, device=DEV, dtype=torch.float64)
+
+    def fn(x_min, x_max, y_min, y_max):
+        return BoxConvolutionFunction.apply(x, x_min, x_max, y_min, y_max, reparam_h, reparam_w,
+                                            normalize, True)
+
+    assert torch.autograd.gradcheck(fn, stored, eps=0.004 / max(reparam_h, reparam_w),
+                                    raise_exception=True)           # reference test.py:296-301
+
+
+@pytest.mark.parametrize("case", ["inside_f32", "hanging_f32", "integer_f32", "unit_f32",
+                                  "hanging_f64", "integer_f64", "tall_f32"])
+def test_hip_matches_golden_vectors_of_the_reference(hip, case):
+    gold = np.load(GOLDEN)
+    x = torch.from_numpy(gold[case + "/x"]).to(DEV)
+    g = torch.from_numpy(gold[case + "/grad_output"]).to(DEV)
+    reparam_h, reparam_w = (float(v) for v in gold[case + "/reparam"])
+    f32 = x.dtype == torch.float32
+    tol_f, tol_p = (1e-4, 1e-3) if f32 else (1e-9, 1e-9)
+    integ = hip.integral_image(x)
+    want_i = gold[case + "/integral"]
+    assert np.abs(integ.cpu().numpy() - want_i).max() <= (1e-6 if f32 else 1e-13) * max(1.0, np.abs(want_i).max())
+    eps = np.finfo(want_i.dtype).eps
+    noise = 8 * eps * float(np.abs(want_i).max())
+    gnoise = 8 * eps * float(hip.integral_image(g).abs().max())
+    for exact in (1, 0):
+        bx = [torch.from_numpy(gold["%s/exact%d/%s" % (case, exact, n)]).to(DEV)
+              for n in ("x_min", "x_max", "y_min", "y_max")]
+        for normalize in (1, 0):
+            tag = "%s/exact%d/norm%d" % (case, exact, normalize)
+            out = hip.box_convolution_forward(integ, *bx, normalize, exact)
+            back = hip.box_convolution_backward(integ, *bx, g, out, reparam_h, reparam_w, normalize,
+                                                exact, True, True, True, True, True)
+            want = gold[tag + "/output"]
+            assert np.abs(out.cpu().numpy() - want).max() <= tol_f * np.abs(want).max() + noise, tag
+            want = gold[tag + "/grad_input"]
+            assert np.abs(back[0].cpu().numpy() - want).max() <= tol_f * np.abs(want).max() + gnoise, tag
+            names = ("grad_x_min", "grad_x_max", "grad_y_min", "grad_y_max")
+            scale = max(np.abs(gold[tag + "/" + n]).max() for n in names)
+            for k, n in enumerate(names):
+                want = gold[tag + "/" + n]
+                assert np.abs(back[1 + k].cpu().numpy() - want).max() <= tol_p * max(np.abs(want).max(), 1e-2 * scale), (tag, n)
+
+
+def test_clip_matches_golden_vectors_bit_for_bit(hip):
+    gold = np.load(GOLDEN)
+    for tag in ("clip_f32", "clip_f64"):
+        rh, rw, mh, mw = (float(v) for v in gold[tag + "/meta"])
+        for exact in (1, 0):
+            p = [torch.from_numpy(gold["%s/in%d" % (tag, k)]).to(DEV) for k in range(4)]
+            hip.clip_parameters(*p, rh, rw, mh, mw, exact)
+            for k in range(4):
+                assert np.array_equal(p[k].cpu().numpy(), gold["%s/exact%d/out%d" % (tag, exact, k)])
+
+
+def test_training_forward_clips_and_eval_clips_once():
+    random.seed(3)
+    m = BoxConv2d(2, 3, 16, 16).to(DEV)
+    with torch.no_grad():
+        m.x_min.fill_(0.5)       # 64 px: far outside [-(16+1), 16-1]
+        m.x_max.fill_(0.5)
+    m.eval()
+    assert torch.all(m.x_max * m.reparametrization_h <= 15 + 1e-3)
+    assert torch.all((m.x_max - m.x_min) * m.reparametrization_h >= 0.0011 - 1e-4)
+    with torch.no_grad():
+        m.y_min.fill_(-1.0)
+    m.train()
+    x = torch.randn(1, 2, 16, 16, device=DEV)
+    m(x)
+    assert torch.all(m.y_min * m.reparametrization_w >= -17 - 1e-3)
+    # eval-mode forward leaves the parameters alone
+    m.training = False
+    with torch.no_grad():
+        m.y_min.fill_(-1.0)
+    m(x)
+    assert torch.all(m.y_min == -1.0)
+
+
+def test_eval_before_moving_to_gpu_uses_the_hip_kernel():
+    random.seed(4)
+    m = BoxConv2d(1, 4, 12, 12)
+    with torch.no_grad():
+        m.x_max.copy_(m.x_min)                     # zero-thickness boxes on the host
+    m.eval()
+    assert m.x_min.device.type == "cpu"
+    thick = (m.x_max - m.x_min) * m.reparametrization_h
+    assert torch.allclose(thick, torch.full_like(thick, 1.001 - 0.9999), atol=1e-4)
+
+
+def test_module_trains_end_to_end():
+    random.seed(5)
+    torch.manual_seed(5)
+    m = BoxConv2d(3, 4, 24, 32).to(DEV)
+    opt = torch.optim.SGD(m.parameters(), lr=1e-4)
+    x = torch.randn(2, 3, 24, 32, device=DEV, requires_grad=True)
+    target = torch.randn(2, 12, 24, 32, device=DEV)
+    losses = []
+    for _ in range(5):
+        opt.zero_grad()
+        loss = ((m(x) - target) ** 2).mean()
+        loss.backward()
+        opt.step()
+        losses.append(loss.item())
+    assert all(np.isfinite(losses)) and x.grad is not None and x.grad.shape == x.shape
+    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in m.parameters())
+
+
+def test_noncontiguous_input_and_dtype_errors(hip):
+    x = torch.randn(2, 2, 9, 20, device=DEV)[..., ::2]
+    assert not x.is_contiguous()
+    assert torch.equal(hip.integral_image(x), hip.integral_image(x.contiguous()))
+    with pytest.raises(RuntimeError, match="float32 or float64"):
+        hip.integral_image(torch.zeros(1, 4, 4, device=DEV, dtype=torch.float16))
+    z = torch.zeros(2, 1, device=DEV)
+    with pytest.raises(RuntimeError, match="as many rows"):
+        hip.box_convolution_forward(torch.zeros(1, 3, 5, 5, device=DEV), z, z, z, z, True, True)
+    with pytest.raises(RuntimeError, match="different devices"):
+        hip.box_convolution_forward(torch.zeros(1, 2, 5, 5, device=DEV), z.cpu(), z, z, z, True, True)

@@ -31,14 +31,14 @@ METRIC = "BoxConv2d fwd+bwd ms/iter + effective HBM GB/s (% peak) at 2x16ch 512x
 
 def kernel_algorithmic_bytes(ab, elem=4):
     """Algorithmic bytes moved by ONE launch of each kernel at a given workload: the share of the
-    step's data flow that the kernel is responsible for. band_scan is launched twice per step (input,
-    then grad_output); the figure is the grad_output launch, the larger one."""
+    step's data flow that the kernel is responsible for (each is launched once per step)."""
     return {
-        "band_scan": elem * (ab["n_out"] + ab["n_gint"]),        # read grad_output, write its integral
-        "band_colsum": elem * ab["n_out"],                       # pre-pass over grad_output
+        # read grad_output and the input's integral, write the (band-local) integral of grad_output
+        "grad_output_stream": elem * (ab["n_out"] + ab["n_int"] + ab["n_gint"]),
+        "band_scan": elem * (ab["n_in"] + ab["n_int"]),          # read input, write its integral
+        "band_colsum": elem * ab["n_in"],                        # pre-pass over the input
         "forward_rows": elem * (ab["n_int"] + ab["n_out"]),      # read integral, write output
         "grad_input_rows": elem * (ab["n_gint"] + ab["n_in"]),   # read integral of grad_output, write grad_input
-        "grad_params_rows": elem * (ab["n_out"] + ab["n_int"]),  # read grad_output and integral
     }
 
 
@@ -141,7 +141,7 @@ def main():
 
     # which kernel takes the most time per step (one untimed step per candidate)
     per_kernel = {}
-    for name in ("band_scan", "band_colsum", "forward_rows", "grad_input_rows", "grad_params_rows"):
+    for name in ("grad_output_stream", "band_scan", "band_colsum", "forward_rows", "grad_input_rows"):
         _native.profile_arm(name)
         step()
         ms, launches = _native.profile_collect()
@@ -164,13 +164,7 @@ def main():
     ms_per_step = 1e3 * elapsed / args.steps
     value = ab["alg"] / (elapsed / args.steps) / 1e9
 
-    kbytes = kernel_algorithmic_bytes(ab)
-    if dominant == "band_scan":
-        # two launches per step (input planes, then grad_output planes): price the pair
-        launches_per_step = dom_launches / args.steps
-        bytes_per_launch = (kbytes["band_scan"] + 4 * (ab["n_in"] + ab["n_int"])) / launches_per_step
-    else:
-        bytes_per_launch = kbytes[dominant]
+    bytes_per_launch = kernel_algorithmic_bytes(ab)[dominant]
     avg_launch_s = dom_ms / 1e3 / max(dom_launches, 1)
     achieved = bytes_per_launch / avg_launch_s / 1e9
 

@@ -46,6 +46,12 @@ namespace {
 
 extern __shared__ __align__(16) unsigned char smem_raw[];
 
+// Largest workgroup of the row-streaming kernels (8 waves). A wide row is spread over more lanes
+// rather than more columns per lane: per-lane state (sliding rows, prefetched rows, accumulators)
+// scales with the columns per lane, and these kernels hide HBM latency with occupancy.
+constexpr int kMaxRowThreads = 512;
+constexpr int kMaxRowWaves = kMaxRowThreads / 64;
+
 template <class T>
 struct SampleArgs {
     const T* src;         // integral planes, (h+1) x (w+1) each, contiguous
@@ -53,7 +59,8 @@ struct SampleArgs {
     T* dst;               // forward: [planes,F,h,w]; grad input: [planes,h,w]
     const T* grad_out;    // param grads only: [planes,F,h,w]
     double* acc;          // param grads only: [C*F*5]
-    double* colsum;       // param grads only: per-band column sums of grad_out, or null
+    const double* band_off;   // grad input only: per-band offsets of a band-local integral, or null
+    int off_nb, off_R;        // band structure of band_off
     int C, F, h, w;
     int nb, R;            // bands per plane and rows per band
     int64_t plane0;       // global index of the first plane (selects the boxes)
@@ -133,7 +140,7 @@ __device__ __forceinline__ BoxOfWorkgroup<T> load_box(const BoxParams<T>& prm, i
 // Forward. Work item = (plane p, filter f, band). blockDim = nt, K >= ceil(w / nt).
 // LDS: [2 buffers][2 rows][w+3] T.
 template <class T, int K, bool EXACT, bool FULL>
-__global__ void __launch_bounds__(256) forward_rows_kernel(SampleArgs<T> a) {
+__global__ void __launch_bounds__(kMaxRowThreads) forward_rows_kernel(SampleArgs<T> a) {
     const int64_t vid = xcd_contiguous_id(a.per_xcd);
     if (vid >= a.total) return;
     const int band = static_cast<int>(vid % a.nb);
@@ -212,8 +219,13 @@ __global__ void __launch_bounds__(256) forward_rows_kernel(SampleArgs<T> a) {
 // ---------------------------------------------------------------------------------------------
 // Gradient w.r.t. the input. Work item = (plane p = (b,c), band of RB rows); the F mirrored boxes
 // are visited in order and summed in registers, so no [B,C,F,h,w] temporary exists.
-template <class T, int K, int RB, bool EXACT, bool FULL>
-__global__ void __launch_bounds__(256) grad_input_rows_kernel(SampleArgs<T> a) {
+//
+// OFFS: `src` holds BAND-LOCAL integral images (see grad_output_stream_kernel) and a.band_off the
+// per-band offsets. A box sum only involves differences between rows, so a row is corrected by
+// off[its band] - off[reference band], the reference being the band of the first row this
+// workgroup touches for the filter; the bulk of the integral cancels before it is ever added.
+template <class T, int K, int RB, bool EXACT, bool FULL, bool OFFS>
+__global__ void __launch_bounds__(kMaxRowThreads) grad_input_rows_kernel(SampleArgs<T> a) {
     static_assert(RB % 2 == 0, "rows are handled in pairs");
     const int64_t vid = xcd_contiguous_id(a.per_xcd);
     if (vid >= a.total) return;
@@ -244,17 +256,49 @@ __global__ void __launch_bounds__(256) grad_input_rows_kernel(SampleArgs<T> a) {
         int lo[K], hi[K];
         column_taps<K>(lo, hi, s.ylo, s.yhi, w, nt);
 
+        // offsets of the band a row lies in, relative to the reference band (OFFS only)
+        const double* offp = OFFS ? a.band_off + (p * a.F + f) * static_cast<int64_t>(a.off_nb) * pitch : nullptr;
+        auto band_of = [&](int row) { return max(row - 1, 0) / a.off_R; };
+        const int ref_band = OFFS ? band_of(clampi(i0 + s.xlo - 1, 0, h)) : 0;
+        int band_t = ref_band, band_b = -1;
+        T off_t[K], off_b[K];
+#pragma unroll
+        for (int k = 0; k < K; ++k) { off_t[k] = T(0); off_b[k] = T(0); }
+        auto correct = [&](T (&row)[K], int row_index, int& cached_band, T (&cached)[K]) {
+            if (!OFFS) return;
+            const int bnd = band_of(row_index);
+            if (bnd != cached_band) {                       // uniform: depends on the row only
+                cached_band = bnd;
+                const double* ob = offp + static_cast<int64_t>(bnd) * pitch;
+                const double* orf = offp + static_cast<int64_t>(ref_band) * pitch;
+#pragma unroll
+                for (int k = 0; k < K; ++k) {
+                    const int q = q0 + nt * k;
+                    cached[k] = (FULL || q <= w) ? static_cast<T>(ob[q] - orf[q]) : T(0);
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < K; ++k) row[k] += cached[k];
+        };
+
         T ta[K], bc[K], t0[K], t1[K], b1[K], b2[K];
         load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), w, q0, nt, ta);
         load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xhi, 0, h), w, q0, nt, bc);
         load_pair<T, K, FULL>(plane, pitch, i0, s.xlo, s.xhi, h, w, q0, nt, t0, t1, b1, b2);
+        correct(ta, clampi(i0 + s.xlo - 1, 0, h), band_t, off_t);
+        correct(t0, clampi(i0 + s.xlo, 0, h), band_t, off_t);
+        correct(t1, clampi(i0 + 1 + s.xlo, 0, h), band_t, off_t);
+        correct(bc, clampi(i0 + s.xhi, 0, h), band_b, off_b);
+        correct(b1, clampi(i0 + 1 + s.xhi, 0, h), band_b, off_b);
+        correct(b2, clampi(i0 + 2 + s.xhi, 0, h), band_b, off_b);
 
 #pragma unroll
         for (int r = 0; r < RB; r += 2) {
             const int i = i0 + r;
             if (i < h) {                                   // uniform across the workgroup
                 T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {};
-                if (r + 2 < RB && i + 2 < h)
+                const bool more = r + 2 < RB && i + 2 < h;
+                if (more)
                     load_pair<T, K, FULL>(plane, pitch, i + 2, s.xlo, s.xhi, h, w, q0, nt, n0, n1, n2, n3);
                 T* V0 = vbuf + flip * 2 * vlen;
                 T* V1 = V0 + vlen;
@@ -283,6 +327,12 @@ __global__ void __launch_bounds__(256) grad_input_rows_kernel(SampleArgs<T> a) {
                     ta[k] = t1[k]; bc[k] = b2[k];
                     t0[k] = n0[k]; t1[k] = n1[k]; b1[k] = n2[k]; b2[k] = n3[k];
                 }
+                if (OFFS && more) {
+                    correct(t0, clampi(i + 2 + s.xlo, 0, h), band_t, off_t);
+                    correct(t1, clampi(i + 3 + s.xlo, 0, h), band_t, off_t);
+                    correct(b1, clampi(i + 3 + s.xhi, 0, h), band_b, off_b);
+                    correct(b2, clampi(i + 4 + s.xhi, 0, h), band_b, off_b);
+                }
             }
         }
     }
@@ -304,7 +354,7 @@ __global__ void __launch_bounds__(256) grad_input_rows_kernel(SampleArgs<T> a) {
 // ---------------------------------------------------------------------------------------------
 // Sum of 5 per-lane values over the workgroup, then one atomic per value.
 __device__ __forceinline__ void block_accumulate5(const double (&v)[5], double* __restrict__ dst,
-                                                  double* __restrict__ lds /* [4*5] */) {
+                                                  double* __restrict__ lds /* [waves*5] */) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = (blockDim.x + 63) >> 6;
 #pragma unroll
     for (int n = 0; n < 5; ++n) {
@@ -319,11 +369,14 @@ __device__ __forceinline__ void block_accumulate5(const double (&v)[5], double* 
     }
 }
 
-// Gradient w.r.t. the box bounds. Work item = (plane p, filter f, band). Accumulates, per (c,f):
-//   [0] sum g*dS/dxmin  [1] sum g*dS/dxmax  [2] sum g*dS/dymin  [3] sum g*dS/dymax  [4] sum g*S
+// Streaming pass over grad_output. Work item = (plane p, filter f, band of R rows). Each row of
+// grad_output is read from HBM once, placed in LDS, and used for both products of the backward
+// pass:
 //
-// Transposed access: for X in {V, DT = I[t]-I[tAdv], DB = I[bAdv]-I[b]} (per-column values of the
-// current output row, held in registers by the lane that owns column q),
+// (PARAMS) the five sums per box that the parameter gradients need,
+//   [0] sum g*dS/dxmin  [1] sum g*dS/dxmax  [2] sum g*dS/dymin  [3] sum g*dS/dymax  [4] sum g*S
+// by transposed access: for X in {V, DT = I[t]-I[tAdv], DB = I[bAdv]-I[b]} (per-column values of
+// the current output row, held in registers by the lane that owns column q),
 //   sum_j g[j]*H(X)[j] = sum_{q=1..w} X[q]*W[q] + X[w]*tail,
 //   W[q] = (gr - gl) + fyhi*(grA - gr) + fylo*(gl - glA),
 //   gr = g[q-yhi], grA = g[q-yhi-1], gl = g[q-ylo], glA = g[q-ylo+1]   (0 outside [0,w)).
@@ -334,11 +387,50 @@ __device__ __forceinline__ void block_accumulate5(const double (&v)[5], double* 
 //          dS/dymin = -sum_q V[q]*(gl - glA) - V[w]*g[w-ylo+1].
 // Column 0 of the integral image is zero, so clamping at the left edge needs no correction.
 //
-// LDS: [2 buffers][2 rows] of { grad_output row with two zeros on either side (w+4), X[w] (3) }.
-// If a.colsum is set, the per-band column sums of grad_output are written too (first pass of
-// the integral image of grad_output, which therefore does not have to read it a second time).
-template <class T, int K, bool EXACT, bool FULL>
-__global__ void __launch_bounds__(256) grad_params_rows_kernel(SampleArgs<T> a) {
+// (SCAN) the BAND-LOCAL integral image of grad_output: L[i+1][c+1] = sum of grad_output over rows
+// band_start..i and columns 0..c. Bands do not depend on each other, so nothing has to be known
+// about the rows above: the true integral is L plus a per-band row vector (band_offsets_kernel)
+// that the grad-input kernel adds when it loads a row. Column accumulators and the row prefix are
+// carried in double; lanes own K consecutive columns for this part (read back from the LDS row),
+// results go through an LDS stage so that global stores are lane-consecutive dwords.
+//
+// LDS: [2 buffers][2 rows][K*nt + 8] grad_output rows (4 zeros in front, >= 4 behind),
+//      [2][2][4] X[w] triples, [2][K*nt] stage, [2][8] doubles wave totals, [8*5] doubles.
+constexpr int kGPad = 4;
+
+template <class T>
+struct StreamLds {
+    T* grow;          // [2][2][glen]
+    T* xw;            // [2][2][4]
+    T* stage;         // [2][K*nt]
+    double* wave_tot; // [2][kMaxRowWaves]
+    double* red;      // [5 * kMaxRowWaves]
+    int glen;
+};
+
+__host__ __device__ inline size_t stream_lds_bytes(int K, int nt, size_t elem) {
+    const size_t glen = static_cast<size_t>(K) * nt + 8;
+    size_t b = (4 * glen + 16 + 2 * static_cast<size_t>(K) * nt) * elem;
+    b = (b + 15) / 16 * 16;
+    return b + (2 * kMaxRowWaves + 5 * kMaxRowWaves) * sizeof(double);
+}
+
+template <class T>
+__device__ __forceinline__ StreamLds<T> carve_stream_lds(int K, int nt) {
+    StreamLds<T> l;
+    l.glen = K * nt + 8;
+    l.grow = reinterpret_cast<T*>(smem_raw);
+    l.xw = l.grow + 4 * l.glen;
+    l.stage = l.xw + 16;
+    size_t b = (4 * static_cast<size_t>(l.glen) + 16 + 2 * static_cast<size_t>(K) * nt) * sizeof(T);
+    b = (b + 15) / 16 * 16;
+    l.wave_tot = reinterpret_cast<double*>(smem_raw + b);
+    l.red = l.wave_tot + 2 * kMaxRowWaves;
+    return l;
+}
+
+template <class T, int K, bool EXACT, bool FULL, bool PARAMS, bool SCAN>
+__global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(SampleArgs<T> a) {
     const int64_t vid = xcd_contiguous_id(a.per_xcd);
     if (vid >= a.total) return;                      // whole workgroup leaves together
     const int band = static_cast<int>(vid % a.nb);
@@ -347,59 +439,64 @@ __global__ void __launch_bounds__(256) grad_params_rows_kernel(SampleArgs<T> a) 
     const int64_t p = pf / a.F;
     const int k_par = static_cast<int>((a.plane0 + p) % a.C) * a.F + f;
     const int h = a.h, w = a.w, nt = blockDim.x, tid = threadIdx.x, q0 = 1 + tid;
+    const int lane = tid & 63, wave = tid >> 6;
 
     const BoxOfWorkgroup<T> bx = load_box(a.prm, k_par);
     const BoxSplit<T> s = split_grad_params(bx.xmin, bx.xmax, bx.ymin, bx.ymax);
 
     const int64_t pitch = w + 1;
-    const T* plane = a.src + p * static_cast<int64_t>(h + 1) * pitch;
+    const T* plane = a.src + p * static_cast<int64_t>(h + 1) * pitch;          // integral of input
     const T* gout = a.grad_out + pf * static_cast<int64_t>(h) * w;
-    const int glen = w + 8;                          // row (w), 2+2 zero pads, X[w] triple, spare
-    T* gbuf = reinterpret_cast<T*>(smem_raw);        // [2][2][glen]
-    double* red = reinterpret_cast<double*>(smem_raw + ((4 * glen * sizeof(T) + 15) / 16) * 16);
+    T* lrows = SCAN ? a.dst + pf * static_cast<int64_t>(h + 1) * pitch : nullptr; // band-local integral
+    const StreamLds<T> lds = carve_stream_lds<T>(K, nt);
+    const int glen = lds.glen;
 
     const int i0 = band * a.R;
     const int i1 = min(h, i0 + a.R);
 
-    // zero pads of all four rows (never overwritten)
-    if (tid < 16) {
-        T* row = gbuf + (tid >> 2) * glen;
-        const int e = tid & 3;
-        row[e < 2 ? e : w + e] = T(0);
-    }
+    // clear the grad_output rows once: pads and the columns beyond w stay zero for good
+    for (int e = tid; e < 4 * glen; e += nt) lds.grow[e] = T(0);
+    if (SCAN && band == 0)
+        for (int c = tid; c <= w; c += nt) lrows[c] = T(0);                    // integral row 0
+    __syncthreads();
 
     // lane-constant LDS indices of the pairs (grA, gr) and (gl, glA), and the tail weights
     int ir[K], il[K];
     T delta[K];
+    int idx_ymax = 0, idx_ymin = 0;
+    if (PARAMS) {
 #pragma unroll
-    for (int k = 0; k < K; ++k) {
-        const int j = tid + nt * k;
-        const int q = j + 1;
-        ir[k] = clampi(q - s.yhi - 1, -2, w) + 2;
-        il[k] = clampi(q - s.ylo, -2, w) + 2;
-        T d = T(0);
-        if (FULL || j < w) {
-            const T one = T(1);
-            d = (EXACT ? (one - s.fyhi) : one) * T(j > w - s.yhi)
-              + (EXACT ? s.fyhi : T(0)) * T(j > w - s.yhi - 1)
-              - (EXACT ? (one - s.fylo) : one) * T(j > w - s.ylo)
-              - (EXACT ? s.fylo : T(0)) * T(j > w - s.ylo + 1);
+        for (int k = 0; k < K; ++k) {
+            const int j = tid + nt * k;
+            const int q = j + 1;
+            ir[k] = clampi(q - s.yhi - 1, -2, w) + kGPad;
+            il[k] = clampi(q - s.ylo, -2, w) + kGPad;
+            T d = T(0);
+            if (FULL || j < w) {
+                const T one = T(1);
+                d = (EXACT ? (one - s.fyhi) : one) * T(j > w - s.yhi)
+                  + (EXACT ? s.fyhi : T(0)) * T(j > w - s.yhi - 1)
+                  - (EXACT ? (one - s.fylo) : one) * T(j > w - s.ylo)
+                  - (EXACT ? s.fylo : T(0)) * T(j > w - s.ylo + 1);
+            }
+            delta[k] = d;
         }
-        delta[k] = d;
+        const int j_ymax = w - s.yhi, j_ymin = w - s.ylo + 1;
+        idx_ymax = (j_ymax >= 0 && j_ymax < w) ? j_ymax + kGPad : 0;          // index 0 holds a zero
+        idx_ymin = (j_ymin >= 0 && j_ymin < w) ? j_ymin + kGPad : 0;
     }
-    const int j_ymax = w - s.yhi, j_ymin = w - s.ylo + 1;
-    const int idx_ymax = (j_ymax >= 0 && j_ymax < w) ? j_ymax + 2 : 0;     // index 0 holds a zero
-    const int idx_ymin = (j_ymin >= 0 && j_ymin < w) ? j_ymin + 2 : 0;
 
     T sum[5] = {T(0), T(0), T(0), T(0), T(0)};
-    double cs[K];
+    double colacc[K];                                 // SCAN: columns K*tid .. K*tid+K-1
 #pragma unroll
-    for (int k = 0; k < K; ++k) cs[k] = 0.0;
+    for (int k = 0; k < K; ++k) colacc[k] = 0.0;
 
     T ta[K], bc[K], t0[K], t1[K], b1[K], b2[K], g0[K], g1[K];
-    load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), w, q0, nt, ta);
-    load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xhi, 0, h), w, q0, nt, bc);
-    load_pair<T, K, FULL>(plane, pitch, i0, s.xlo, s.xhi, h, w, q0, nt, t0, t1, b1, b2);
+    if (PARAMS) {
+        load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), w, q0, nt, ta);
+        load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xhi, 0, h), w, q0, nt, bc);
+        load_pair<T, K, FULL>(plane, pitch, i0, s.xlo, s.xhi, h, w, q0, nt, t0, t1, b1, b2);
+    }
     auto load_g = [&](int i, T (&dst)[K]) {
         const T* grow = gout + static_cast<int64_t>(min(i, h - 1)) * w;
         const bool valid = i < i1;
@@ -416,70 +513,76 @@ __global__ void __launch_bounds__(256) grad_params_rows_kernel(SampleArgs<T> a) 
     for (int i = i0; i < i1; i += 2) {
         T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {}, m0[K] = {}, m1[K] = {};
         if (i + 2 < i1) {
-            load_pair<T, K, FULL>(plane, pitch, i + 2, s.xlo, s.xhi, h, w, q0, nt, n0, n1, n2, n3);
+            if (PARAMS)
+                load_pair<T, K, FULL>(plane, pitch, i + 2, s.xlo, s.xhi, h, w, q0, nt, n0, n1, n2, n3);
             load_g(i + 2, m0);
             load_g(i + 3, m1);
         }
 
-        T* G0 = gbuf + flip * 2 * glen;
+        T* G0 = lds.grow + flip * 2 * glen;
         T* G1 = G0 + glen;
+        T* X0 = lds.xw + flip * 8;
+        T* X1 = X0 + 4;
         flip ^= 1;
-
-        T v0[K], dt0[K], db0[K], v1[K], dt1[K], db1[K];
-#pragma unroll
-        for (int k = 0; k < K; ++k) {
-            dt0[k] = t0[k] - ta[k];  db0[k] = b1[k] - bc[k];
-            dt1[k] = t1[k] - t0[k];  db1[k] = b2[k] - b1[k];
-            v0[k] = bc[k] - t0[k];
-            v1[k] = b1[k] - t1[k];
-            if (EXACT) {
-                v0[k] += s.fxhi * db0[k] + s.fxlo * dt0[k];
-                v1[k] += s.fxhi * db1[k] + s.fxlo * dt1[k];
-            }
-            const int j = tid + nt * k;
-            if (FULL || j < w) {
-                G0[j + 2] = g0[k];
-                G1[j + 2] = g1[k];
-                cs[k] += static_cast<double>(g0[k]) + static_cast<double>(g1[k]);
-            }
-            if (FULL ? (k == K - 1 && tid == nt - 1) : (j == w - 1)) {      // owner of column q = w
-                G0[w + 4] = v0[k]; G0[w + 5] = dt0[k]; G0[w + 6] = db0[k];
-                G1[w + 4] = v1[k]; G1[w + 5] = dt1[k]; G1[w + 6] = db1[k];
-            }
-        }
-        __syncthreads();
 
         T tail0 = T(0), tail1 = T(0);
 #pragma unroll
         for (int k = 0; k < K; ++k) {
-            {
-                const T grA = G0[ir[k]], gr = G0[ir[k] + 1], gl = G0[il[k]], glA = G0[il[k] + 1];
-                const T dr = grA - gr, dl = gl - glA;
-                T wq = gr - gl;
-                if (EXACT) wq += s.fyhi * dr + s.fylo * dl;
-                sum[4] += v0[k] * wq;
-                sum[1] += db0[k] * wq;
-                sum[0] -= dt0[k] * wq;
-                sum[3] += v0[k] * dr;
-                sum[2] -= v0[k] * dl;
-                tail0 += delta[k] * g0[k];
+            const int j = tid + nt * k;
+            if (FULL || j < w) {
+                G0[j + kGPad] = g0[k];
+                G1[j + kGPad] = g1[k];
             }
-            {
-                const T grA = G1[ir[k]], gr = G1[ir[k] + 1], gl = G1[il[k]], glA = G1[il[k] + 1];
-                const T dr = grA - gr, dl = gl - glA;
-                T wq = gr - gl;
-                if (EXACT) wq += s.fyhi * dr + s.fylo * dl;
-                sum[4] += v1[k] * wq;
-                sum[1] += db1[k] * wq;
-                sum[0] -= dt1[k] * wq;
-                sum[3] += v1[k] * dr;
-                sum[2] -= v1[k] * dl;
-                tail1 += delta[k] * g1[k];
+            if (PARAMS) { tail0 += delta[k] * g0[k]; tail1 += delta[k] * g1[k]; }
+            if (PARAMS && (FULL ? (k == K - 1 && tid == nt - 1) : (j == w - 1))) {   // owner of column q = w
+                const T dt0 = t0[k] - ta[k], db0 = b1[k] - bc[k];
+                const T dt1 = t1[k] - t0[k], db1 = b2[k] - b1[k];
+                T v0 = bc[k] - t0[k], v1 = b1[k] - t1[k];
+                if (EXACT) {
+                    v0 += s.fxhi * db0 + s.fxlo * dt0;
+                    v1 += s.fxhi * db1 + s.fxlo * dt1;
+                }
+                X0[0] = v0; X0[1] = dt0; X0[2] = db0;
+                X1[0] = v1; X1[1] = dt1; X1[2] = db1;
             }
         }
-        {
-            const T vw0 = G0[w + 4], dtw0 = G0[w + 5], dbw0 = G0[w + 6];
-            const T vw1 = G1[w + 4], dtw1 = G1[w + 5], dbw1 = G1[w + 6];
+        __syncthreads();                                                     // rows are in LDS
+
+        if (PARAMS) {
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                const T dt0 = t0[k] - ta[k], db0 = b1[k] - bc[k];
+                const T dt1 = t1[k] - t0[k], db1 = b2[k] - b1[k];
+                T v0 = bc[k] - t0[k], v1 = b1[k] - t1[k];
+                if (EXACT) {
+                    v0 += s.fxhi * db0 + s.fxlo * dt0;
+                    v1 += s.fxhi * db1 + s.fxlo * dt1;
+                }
+                {
+                    const T grA = G0[ir[k]], gr = G0[ir[k] + 1], gl = G0[il[k]], glA = G0[il[k] + 1];
+                    const T dr = grA - gr, dl = gl - glA;
+                    T wq = gr - gl;
+                    if (EXACT) wq += s.fyhi * dr + s.fylo * dl;
+                    sum[4] += v0 * wq;
+                    sum[1] += db0 * wq;
+                    sum[0] -= dt0 * wq;
+                    sum[3] += v0 * dr;
+                    sum[2] -= v0 * dl;
+                }
+                {
+                    const T grA = G1[ir[k]], gr = G1[ir[k] + 1], gl = G1[il[k]], glA = G1[il[k] + 1];
+                    const T dr = grA - gr, dl = gl - glA;
+                    T wq = gr - gl;
+                    if (EXACT) wq += s.fyhi * dr + s.fylo * dl;
+                    sum[4] += v1 * wq;
+                    sum[1] += db1 * wq;
+                    sum[0] -= dt1 * wq;
+                    sum[3] += v1 * dr;
+                    sum[2] -= v1 * dl;
+                }
+            }
+            const T vw0 = X0[0], dtw0 = X0[1], dbw0 = X0[2];
+            const T vw1 = X1[0], dtw1 = X1[1], dbw1 = X1[2];
             sum[4] += vw0 * tail0 + vw1 * tail1;
             sum[1] += dbw0 * tail0 + dbw1 * tail1;
             sum[0] -= dtw0 * tail0 + dtw1 * tail1;
@@ -488,28 +591,101 @@ __global__ void __launch_bounds__(256) grad_params_rows_kernel(SampleArgs<T> a) 
                 sum[2] -= vw0 * G0[idx_ymin] + vw1 * G1[idx_ymin];
             }
         }
+
+        if (SCAN) {
+            // lane owns columns K*tid .. K*tid+K-1; two rows of the band-local integral.
+            // loc*: prefix inside the lane (small numbers, kept in T); carry*: everything to
+            // the left of the lane (double).
+            T loc0[K], loc1[K];
+            double carry0, carry1;
+            {
+                const T* r0 = G0 + kGPad + K * tid;
+                const T* r1 = G1 + kGPad + K * tid;
+                double run0 = 0.0, run1 = 0.0;
+#pragma unroll
+                for (int k = 0; k < K; ++k) {
+                    colacc[k] += static_cast<double>(r0[k]);
+                    run0 += colacc[k];
+                    loc0[k] = static_cast<T>(run0);
+                    colacc[k] += static_cast<double>(r1[k]);
+                    run1 += colacc[k];
+                    loc1[k] = static_cast<T>(run1);
+                }
+                const double inc0 = wave_inclusive_scan(run0);
+                const double inc1 = wave_inclusive_scan(run1);
+                carry0 = inc0 - run0;
+                carry1 = inc1 - run1;
+                if (lane == 63) { lds.wave_tot[wave] = inc0; lds.wave_tot[kMaxRowWaves + wave] = inc1; }
+            }
+            __syncthreads();                                                 // wave totals visible
+            {
+                for (int wv = 0; wv < wave; ++wv) { carry0 += lds.wave_tot[wv]; carry1 += lds.wave_tot[kMaxRowWaves + wv]; }
+                T* s0 = lds.stage + K * tid;
+                T* s1 = lds.stage + K * nt + K * tid;
+#pragma unroll
+                for (int k = 0; k < K; ++k) {
+                    s0[k] = static_cast<T>(carry0 + static_cast<double>(loc0[k]));
+                    s1[k] = static_cast<T>(carry1 + static_cast<double>(loc1[k]));
+                }
+            }
+            __syncthreads();                                                 // stage visible
+            {
+                T* o0 = lrows + static_cast<int64_t>(i + 1) * pitch;
+                const bool second = i + 1 < i1;
+#pragma unroll
+                for (int k = 0; k < K; ++k) {
+                    const int j = tid + nt * k;
+                    if (FULL || j < w) {
+                        o0[j + 1] = lds.stage[j];
+                        if (second) o0[pitch + j + 1] = lds.stage[K * nt + j];
+                    }
+                }
+                if (tid == 0) {
+                    o0[0] = T(0);
+                    if (second) o0[pitch] = T(0);
+                }
+            }
+        }
+
 #pragma unroll
         for (int k = 0; k < K; ++k) {
-            ta[k] = t1[k]; bc[k] = b2[k];
-            t0[k] = n0[k]; t1[k] = n1[k]; b1[k] = n2[k]; b2[k] = n3[k];
+            if (PARAMS) {
+                ta[k] = t1[k]; bc[k] = b2[k];
+                t0[k] = n0[k]; t1[k] = n1[k]; b1[k] = n2[k]; b2[k] = n3[k];
+            }
             g0[k] = m0[k]; g1[k] = m1[k];
         }
     }
 
-    if (a.colsum != nullptr && band < a.nb - 1) {
-        double* dst = a.colsum + (pf * (a.nb - 1) + band) * static_cast<int64_t>(w);
-#pragma unroll
-        for (int k = 0; k < K; ++k) {
-            const int j = tid + nt * k;
-            if (FULL || j < w) dst[j] = cs[k];
-        }
+    if (PARAMS) {
+        __syncthreads();
+        const double v[5] = {static_cast<double>(sum[0]), static_cast<double>(sum[1]),
+                             static_cast<double>(sum[2]), static_cast<double>(sum[3]),
+                             static_cast<double>(sum[4])};
+        block_accumulate5(v, a.acc + static_cast<int64_t>(k_par) * 5, lds.red);
     }
+}
 
-    __syncthreads();
-    const double v[5] = {static_cast<double>(sum[0]), static_cast<double>(sum[1]),
-                         static_cast<double>(sum[2]), static_cast<double>(sum[3]),
-                         static_cast<double>(sum[4])};
-    block_accumulate5(v, a.acc + static_cast<int64_t>(k_par) * 5, red);
+// Per-band offsets of the band-local integral written by grad_output_stream_kernel:
+// off[pf][k][c] = true integral at the top edge of band k = sum of the bottom rows of the bands
+// above (double). One thread per (plane, column).
+template <class T>
+__global__ void __launch_bounds__(256)
+band_offsets_kernel(const T* __restrict__ lrows, double* __restrict__ off, int64_t planes_f, int h,
+                    int w, int nb, int R) {
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const int64_t W1 = w + 1;
+    if (idx >= planes_f * W1) return;
+    const int64_t pf = idx / W1;
+    const int c = static_cast<int>(idx % W1);
+    const T* plane = lrows + pf * static_cast<int64_t>(h + 1) * W1;
+    double* o = off + pf * static_cast<int64_t>(nb) * W1 + c;
+    double run = 0.0;
+    for (int k = 0; k < nb; ++k) {
+        o[static_cast<int64_t>(k) * W1] = run;
+        const int bottom = min(h, (k + 1) * R);
+        run += static_cast<double>(plane[static_cast<int64_t>(bottom) * W1 + c]);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -658,9 +834,17 @@ __global__ void param_grad_finalize_kernel(const double* __restrict__ acc, BoxPa
 
 // ---------------------------------------------------------------------------------------------
 struct RowConfig { int nt; int K; bool full; };
+inline int max_row_threads() {
+    static const int v = [] {
+        const char* e = std::getenv("BOXCONV_ROW_THREADS");
+        const int n = e ? std::atoi(e) : kMaxRowThreads;
+        return (n == 64 || n == 128 || n == 256 || n == 512) ? n : kMaxRowThreads;
+    }();
+    return v;
+}
 inline RowConfig row_config(int w) {
     RowConfig c;
-    c.nt = std::min(256, ((w + 63) / 64) * 64);
+    c.nt = std::min(max_row_threads(), ((w + 63) / 64) * 64);
     const int k = (w + c.nt - 1) / c.nt;
     c.K = k <= 1 ? 1 : k <= 2 ? 2 : k <= 4 ? 4 : 8;
     c.full = (c.K * c.nt == w);
@@ -736,13 +920,16 @@ hipError_t forward_launch(const T* integ, BoxParams<T> prm, T* out, Dims d, bool
 }
 
 template <class T>
-hipError_t grad_input_launch(const T* gint, BoxParams<T> prm, T* grad_in, Dims d, bool normalize,
-                             bool exact, hipStream_t stream) {
+hipError_t grad_input_launch(const T* gint, const double* band_off, int off_nb, int off_R,
+                             BoxParams<T> prm, T* grad_in, Dims d, bool normalize, bool exact,
+                             hipStream_t stream) {
     if (d.planes == 0 || d.hw() == 0) return hipSuccess;
     SampleArgs<T> a = base_args(prm, d);
     a.src = gint; a.dst = grad_in; a.normalize = normalize ? 1 : 0;
+    a.band_off = band_off; a.off_nb = off_nb; a.off_R = std::max(off_R, 1);
 
     if (d.w > kMaxRowStreamWidth || force_gather_kernels()) {
+        if (band_off != nullptr) return hipErrorInvalidValue;   // the gather kernel needs a true integral
         finish_args(a, d.planes * d.hw());
         const dim3 grid(static_cast<unsigned>((a.total + 255) / 256));
         if (exact) BOXCONV_LAUNCH("grad_input_gather", (grad_input_gather_kernel<T, true>), grid, dim3(256), 0, stream, a);
@@ -758,7 +945,8 @@ hipError_t grad_input_launch(const T* gint, BoxParams<T> prm, T* grad_in, Dims d
     const dim3 grid(static_cast<unsigned>(a.per_xcd * kXcds));
     const size_t lds = 4 * static_cast<size_t>(d.w + 3) * sizeof(T);
 #define LAUNCH_GI(KK, EX, FU) \
-    BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, KK, RB, EX, FU>), grid, dim3(rc.nt), lds, stream, a)
+    if (band_off != nullptr) BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, KK, RB, EX, FU, true>), grid, dim3(rc.nt), lds, stream, a); \
+    else BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, KK, RB, EX, FU, false>), grid, dim3(rc.nt), lds, stream, a)
     BOXCONV_DISPATCH_K_EXACT_FULL(LAUNCH_GI, rc.K, exact, rc.full)
 #undef LAUNCH_GI
     return hipGetLastError();
@@ -771,45 +959,62 @@ hipError_t grad_params_begin(double* acc, int n_boxes, hipStream_t stream) {
     return hipGetLastError();
 }
 
+StreamPlan plan_grad_output_stream(int64_t planes_f, int h, int w, size_t elem_size) {
+    StreamPlan sp{};
+    const RowConfig rc = row_config(std::max(w, 1));
+    sp.usable = w <= kMaxRowStreamWidth && !force_gather_kernels() &&
+                stream_lds_bytes(rc.K, rc.nt, elem_size) <= kMaxDynamicLds;
+    int nb = bands_for(std::max<int64_t>(planes_f, 1), h, 32, 2048);
+    int R = (h + nb - 1) / nb;
+    R += R & 1;                                        // rows are handled in pairs
+    sp.R = std::max(R, 2);
+    sp.nb = (h + sp.R - 1) / sp.R;
+    sp.offset_doubles = planes_f * static_cast<int64_t>(sp.nb) * (w + 1);
+    return sp;
+}
+
 template <class T>
-hipError_t grad_params_accumulate(const T* integ, const T* grad_out, BoxParams<T> prm, double* acc,
-                                  double* colsum_aux, const IntegralPlan& plan, Dims d, bool exact,
-                                  bool* wrote_colsums, hipStream_t stream) {
-    if (wrote_colsums) *wrote_colsums = false;
+hipError_t grad_output_stream_launch(const T* integ, const T* grad_out, BoxParams<T> prm,
+                                     double* acc, T* local_integral, double* band_off,
+                                     const StreamPlan& sp, Dims d, bool exact, hipStream_t stream) {
+    const int64_t planes_f = d.planes * d.F;
+    if (planes_f == 0 || d.hw() == 0) return hipSuccess;
+    const bool params = acc != nullptr, scan = local_integral != nullptr;
+    if (!sp.usable || (!params && !scan)) return hipErrorInvalidValue;
+    SampleArgs<T> a = base_args(prm, d);
+    a.src = integ; a.grad_out = grad_out; a.acc = acc; a.dst = local_integral;
+    a.nb = sp.nb; a.R = sp.R;
+    finish_args(a, planes_f * a.nb);
+    const RowConfig rc = row_config(d.w);
+    const dim3 grid(static_cast<unsigned>(a.per_xcd * kXcds));
+    const size_t lds = stream_lds_bytes(rc.K, rc.nt, sizeof(T));
+#define LAUNCH_GS(KK, EX, FU) \
+    if (params && scan) BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_kernel<T, KK, EX, FU, true, true>), grid, dim3(rc.nt), lds, stream, a); \
+    else if (params)    BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_kernel<T, KK, EX, FU, true, false>), grid, dim3(rc.nt), lds, stream, a); \
+    else                BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_kernel<T, KK, EX, FU, false, true>), grid, dim3(rc.nt), lds, stream, a)
+    BOXCONV_DISPATCH_K_EXACT_FULL(LAUNCH_GS, rc.K, exact, rc.full)
+#undef LAUNCH_GS
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || !scan) return e;
+    const int64_t n = planes_f * (d.w + 1);
+    BOXCONV_LAUNCH("band_offsets", (band_offsets_kernel<T>), dim3(static_cast<unsigned>((n + 255) / 256)),
+                   dim3(256), 0, stream, local_integral, band_off, planes_f, d.h, d.w, sp.nb, sp.R);
+    return hipGetLastError();
+}
+
+// Parameter-gradient sums from a true integral image with the gather kernel (any width).
+template <class T>
+hipError_t grad_params_gather_launch(const T* integ, const T* grad_out, BoxParams<T> prm,
+                                     double* acc, Dims d, bool exact, hipStream_t stream) {
     const int64_t planes_f = d.planes * d.F;
     if (planes_f == 0 || d.hw() == 0) return hipSuccess;
     SampleArgs<T> a = base_args(prm, d);
     a.src = integ; a.grad_out = grad_out; a.acc = acc;
-
-    const size_t glen = static_cast<size_t>(d.w) + 8;
-    const size_t lds = ((4 * glen * sizeof(T) + 15) / 16) * 16 + 4 * 5 * sizeof(double);
-    if (d.w > kMaxRowStreamWidth || lds > kMaxDynamicLds || force_gather_kernels()) {
-        const int bpp = static_cast<int>((d.hw() + 255) / 256);
-        finish_args(a, planes_f * bpp);
-        const dim3 grid(static_cast<unsigned>(a.total));
-        if (exact) BOXCONV_LAUNCH("grad_params_gather", (grad_params_gather_kernel<T, true>), grid, dim3(256), 0, stream, a, bpp);
-        else       BOXCONV_LAUNCH("grad_params_gather", (grad_params_gather_kernel<T, false>), grid, dim3(256), 0, stream, a, bpp);
-        return hipGetLastError();
-    }
-
-    const RowConfig rc = row_config(d.w);
-    if (colsum_aux != nullptr && plan.nb > 1) {
-        // share the band structure of the integral image so the column sums line up
-        a.nb = plan.nb; a.R = plan.R; a.colsum = colsum_aux;
-        if (wrote_colsums) *wrote_colsums = true;
-    } else {
-        a.nb = bands_for(planes_f, d.h, 16, 4096);
-        a.R = (d.h + a.nb - 1) / a.nb;
-        a.R += a.R & 1;
-        a.nb = (d.h + a.R - 1) / a.R;
-        a.colsum = nullptr;
-    }
-    finish_args(a, planes_f * a.nb);
-    const dim3 grid(static_cast<unsigned>(a.per_xcd * kXcds));
-#define LAUNCH_GP(KK, EX, FU) \
-    BOXCONV_LAUNCH("grad_params_rows", (grad_params_rows_kernel<T, KK, EX, FU>), grid, dim3(rc.nt), lds, stream, a)
-    BOXCONV_DISPATCH_K_EXACT_FULL(LAUNCH_GP, rc.K, exact, rc.full)
-#undef LAUNCH_GP
+    const int bpp = static_cast<int>((d.hw() + 255) / 256);
+    finish_args(a, planes_f * bpp);
+    const dim3 grid(static_cast<unsigned>(a.total));
+    if (exact) BOXCONV_LAUNCH("grad_params_gather", (grad_params_gather_kernel<T, true>), grid, dim3(256), 0, stream, a, bpp);
+    else       BOXCONV_LAUNCH("grad_params_gather", (grad_params_gather_kernel<T, false>), grid, dim3(256), 0, stream, a, bpp);
     return hipGetLastError();
 }
 
@@ -826,9 +1031,13 @@ hipError_t grad_params_finish(const double* acc, BoxParams<T> prm, T* gxmin, T* 
 
 #define BOXCONV_INSTANTIATE(T)                                                                     \
     template hipError_t forward_launch<T>(const T*, BoxParams<T>, T*, Dims, bool, bool, hipStream_t); \
-    template hipError_t grad_input_launch<T>(const T*, BoxParams<T>, T*, Dims, bool, bool, hipStream_t); \
-    template hipError_t grad_params_accumulate<T>(const T*, const T*, BoxParams<T>, double*, double*, \
-                                                  const IntegralPlan&, Dims, bool, bool*, hipStream_t); \
+    template hipError_t grad_input_launch<T>(const T*, const double*, int, int, BoxParams<T>, T*,  \
+                                             Dims, bool, bool, hipStream_t);                       \
+    template hipError_t grad_output_stream_launch<T>(const T*, const T*, BoxParams<T>, double*, T*, \
+                                                     double*, const StreamPlan&, Dims, bool,       \
+                                                     hipStream_t);                                 \
+    template hipError_t grad_params_gather_launch<T>(const T*, const T*, BoxParams<T>, double*,    \
+                                                     Dims, bool, hipStream_t);                     \
     template hipError_t grad_params_finish<T>(const double*, BoxParams<T>, T*, T*, T*, T*, int,    \
                                               float, float, bool, bool, hipStream_t);
 

@@ -96,32 +96,51 @@ int64_t backward_chunk_planes(int64_t planes) {
     return planes;
 }
 
-constexpr int64_t kBackwardWorkgroups = 2048;   // workgroups the banded backward kernels aim for
+// Walk the planes last to first in the second pass over a tensor (see integral_image_launch).
+bool reverse_second_pass() {
+    static const bool v = [] {
+        const char* e = std::getenv("BOXCONV_BWD_REVERSE");
+        return e == nullptr || e[0] != '0';
+    }();
+    return v;
+}
 
+// Workspace of the backward pass:
+//   [integral of grad_output: chunk*F planes of (h+1)(w+1)]   only if grad_input is wanted
+//   [aux doubles: band offsets (streaming path) or band column sums (three-pass fallback)]
+//   [acc: C*F*5 doubles]                                       only if parameter gradients are wanted
 struct BackwardLayout {
     size_t gint_off, aux_off, acc_off, total;
-    int64_t chunk;                 // planes per chunk
-    boxconv::IntegralPlan plan;    // band structure shared by the chunk's kernels
+    int64_t chunk;        // planes per chunk
+    bool streaming;       // grad_output_stream_kernel usable for this shape
 };
+
+template <class F>
+int64_t max_over_chunks(int64_t planes, int64_t chunk, F f) {
+    int64_t m = f(std::min(chunk, planes));
+    if (const int64_t rest = planes % chunk) m = std::max(m, f(rest));   // shorter last chunk
+    return m;
+}
 
 BackwardLayout backward_layout(int batch, int in_planes, int num_filters, int h, int w,
                                int elem_size, bool need_input, bool need_params) {
     BackwardLayout L{};
     const int64_t planes = static_cast<int64_t>(batch) * in_planes;
     L.chunk = std::max<int64_t>(backward_chunk_planes(planes), 1);
-    L.plan = boxconv::plan_integral(L.chunk * num_filters, h, w, kBackwardWorkgroups);
+    L.streaming = boxconv::plan_grad_output_stream(L.chunk * num_filters, h, w, elem_size).usable;
     size_t off = 0;
     L.gint_off = off;
+    L.aux_off = off;
     if (need_input) {
-        off += align_up(static_cast<size_t>(L.chunk) * num_filters * (h + 1) * (w + 1) * elem_size, 256);
+        off += align_up(static_cast<size_t>(std::min(L.chunk, std::max<int64_t>(planes, 1))) *
+                        num_filters * (h + 1) * (w + 1) * elem_size, 256);
         L.aux_off = off;
-        int64_t aux = L.plan.aux_doubles;
-        if (const int64_t rest = planes % L.chunk)      // a shorter last chunk plans its own bands
-            aux = std::max(aux, boxconv::plan_integral(rest * num_filters, h, w,
-                                                       kBackwardWorkgroups).aux_doubles);
+        const int64_t aux = max_over_chunks(std::max<int64_t>(planes, 1), L.chunk, [&](int64_t np) {
+            return L.streaming
+                ? boxconv::plan_grad_output_stream(np * num_filters, h, w, elem_size).offset_doubles
+                : boxconv::plan_integral(np * num_filters, h, w).aux_doubles;
+        });
         off += align_up(static_cast<size_t>(aux) * 8, 256);
-    } else {
-        L.aux_off = off;
     }
     L.acc_off = off;
     if (need_params) off += align_up(static_cast<size_t>(in_planes) * num_filters * 5 * 8, 256);
@@ -147,7 +166,7 @@ int integral_image_impl(const T* in, T* out, int64_t planes, int h, int w, void*
                     need, workspace_bytes);
     return hip_result(boxconv::integral_image_launch<T>(in, out, planes, h, w,
                                                         static_cast<double*>(workspace),
-                                                        boxconv::plan_integral(planes, h, w), false,
+                                                        boxconv::plan_integral(planes, h, w), false, false,
                                                         static_cast<hipStream_t>(stream)),
                       "integral image launch");
 }
@@ -193,9 +212,9 @@ int backward_impl(const T* integ, const T* x_min, const T* x_max, const T* y_min
     unsigned char* ws = static_cast<unsigned char*>(workspace);
     boxconv::BoxParams<T> prm{x_min, x_max, y_min, y_max};
     const int n_boxes = in_planes * num_filters;
-    double* acc = reinterpret_cast<double*>(ws + L.acc_off);
+    double* acc = need_params ? reinterpret_cast<double*>(ws + L.acc_off) : nullptr;
     double* aux = reinterpret_cast<double*>(ws + L.aux_off);
-    T* gint = reinterpret_cast<T*>(ws + L.gint_off);
+    T* gint = need_input ? reinterpret_cast<T*>(ws + L.gint_off) : nullptr;
 
     if (need_input && nout == 0)
         return fail(BOXCONV_E_INVALID_ARGUMENT, "backward: grad_input requested with zero filters");
@@ -209,26 +228,41 @@ int backward_impl(const T* integ, const T* x_min, const T* x_max, const T* y_min
     for (int64_t p0 = 0; p0 < planes; p0 += L.chunk) {
         const int64_t np = std::min(L.chunk, planes - p0);
         boxconv::Dims d{in_planes, num_filters, h, w, np, p0};
-        // the last chunk may be shorter: its band structure is planned for its own size
-        const boxconv::IntegralPlan plan = (np == L.chunk)
-            ? L.plan : boxconv::plan_integral(np * num_filters, h, w, kBackwardWorkgroups);
         const T* go_chunk = grad_output + p0 * num_filters * hw;
-        bool colsums_ready = false;
-        if (need_params) {
-            if (int rc = hip_result(boxconv::grad_params_accumulate<T>(
-                    integ + p0 * ipl, go_chunk, prm, acc, need_input ? aux : nullptr, plan, d,
-                    exact != 0, &colsums_ready, s), "parameter-gradient launch"))
+        const T* integ_chunk = integ ? integ + p0 * ipl : nullptr;
+        T* gin_chunk = need_input ? grad_input + p0 * hw : nullptr;
+        if (L.streaming) {
+            // one pass over grad_output: parameter sums + band-local integral, then grad_input
+            const boxconv::StreamPlan sp =
+                boxconv::plan_grad_output_stream(np * num_filters, h, w, sizeof(T));
+            if (int rc = hip_result(boxconv::grad_output_stream_launch<T>(
+                    integ_chunk, go_chunk, prm, acc, gint, aux, sp, d, exact != 0, s),
+                    "grad_output streaming launch"))
                 return rc;
-        }
-        if (need_input) {
-            if (int rc = hip_result(boxconv::integral_image_launch<T>(
-                    go_chunk, gint, np * num_filters, h, w, aux, plan, colsums_ready, s),
-                    "grad_output integral image launch"))
-                return rc;
-            if (int rc = hip_result(boxconv::grad_input_launch<T>(
-                    gint, prm, grad_input + p0 * hw, d, normalize != 0, exact != 0, s),
-                    "input-gradient launch"))
-                return rc;
+            if (need_input)
+                if (int rc = hip_result(boxconv::grad_input_launch<T>(
+                        gint, aux, sp.nb, sp.R, prm, gin_chunk, d, normalize != 0, exact != 0, s),
+                        "input-gradient launch"))
+                    return rc;
+        } else {
+            // any width: gather kernels on true integral images
+            if (need_params)
+                if (int rc = hip_result(boxconv::grad_params_gather_launch<T>(
+                        integ_chunk, go_chunk, prm, acc, d, exact != 0, s),
+                        "parameter-gradient launch"))
+                    return rc;
+            if (need_input) {
+                const boxconv::IntegralPlan plan = boxconv::plan_integral(np * num_filters, h, w);
+                if (int rc = hip_result(boxconv::integral_image_launch<T>(
+                        go_chunk, gint, np * num_filters, h, w, aux, plan, false,
+                        need_params && reverse_second_pass(), s),
+                        "grad_output integral image launch"))
+                    return rc;
+                if (int rc = hip_result(boxconv::grad_input_launch<T>(
+                        gint, nullptr, 0, 1, prm, gin_chunk, d, normalize != 0, exact != 0, s),
+                        "input-gradient launch"))
+                    return rc;
+            }
         }
     }
     if (need_params)

@@ -37,30 +37,45 @@ IntegralPlan plan_integral(int64_t planes, int h, int w, int64_t want = 1024);
 
 // colsums_ready: aux already holds the per-band column sums (written by another kernel that read
 // the same input), so the first pass is skipped.
+// reverse_order: walk the planes last to first. A kernel that re-reads what the previous kernel
+// on the stream just streamed through finds the most recently touched planes still in the
+// 256 MB memory-side cache if it starts with those.
 template <class T>
 hipError_t integral_image_launch(const T* in, T* out, int64_t planes, int h, int w, double* aux,
-                                 const IntegralPlan& plan, bool colsums_ready, hipStream_t stream);
+                                 const IntegralPlan& plan, bool colsums_ready, bool reverse_order,
+                                 hipStream_t stream);
 
 template <class T>
 hipError_t forward_launch(const T* integ, BoxParams<T> prm, T* out, Dims d, bool normalize,
                           bool exact, hipStream_t stream);
 
+// band_off: null when `gint` holds true integral images; otherwise `gint` holds band-local
+// integrals with bands of off_R rows (off_nb per plane) and band_off their offsets.
 template <class T>
-hipError_t grad_input_launch(const T* gint, BoxParams<T> prm, T* grad_in, Dims d, bool normalize,
-                             bool exact, hipStream_t stream);
+hipError_t grad_input_launch(const T* gint, const double* band_off, int off_nb, int off_R,
+                             BoxParams<T> prm, T* grad_in, Dims d, bool normalize, bool exact,
+                             hipStream_t stream);
 
-// Parameter gradients in three steps so that a caller can feed the planes in chunks:
-//   begin      clears acc ([C*F*5] doubles of scratch) with a fill kernel
-//   accumulate adds the five sums per box for the planes of `d`; if `colsum_aux` is non-null it
-//              also writes the per-band column sums of grad_out laid out for `plan` (what the
-//              integral image of grad_out needs as its first pass). Returns through
-//              `wrote_colsums` whether it did (the gather fallback does not).
-//   finish     turns the sums into the four gradients; g* may be null for an unwanted gradient.
+// The streaming pass over grad_output (parameter-gradient sums and/or band-local integral).
+struct StreamPlan {
+    bool usable;             // false: width or LDS need outside what the streaming kernel covers
+    int nb, R;               // bands per plane, rows per band (R even)
+    int64_t offset_doubles;  // size of the band-offset array: planes*F * nb * (w+1)
+};
+StreamPlan plan_grad_output_stream(int64_t planes_f, int h, int w, size_t elem_size);
+
+// acc ([C*F*5] doubles, cleared by grad_params_begin) may be null: no parameter sums.
+// local_integral ([planes*F, h+1, w+1]) may be null: no integral; with it band_off receives the
+// per-band offsets. At least one of the two must be given.
+template <class T>
+hipError_t grad_output_stream_launch(const T* integ, const T* grad_out, BoxParams<T> prm,
+                                     double* acc, T* local_integral, double* band_off,
+                                     const StreamPlan& sp, Dims d, bool exact, hipStream_t stream);
+
 hipError_t grad_params_begin(double* acc, int n_boxes, hipStream_t stream);
 template <class T>
-hipError_t grad_params_accumulate(const T* integ, const T* grad_out, BoxParams<T> prm, double* acc,
-                                  double* colsum_aux, const IntegralPlan& plan, Dims d, bool exact,
-                                  bool* wrote_colsums, hipStream_t stream);
+hipError_t grad_params_gather_launch(const T* integ, const T* grad_out, BoxParams<T> prm,
+                                     double* acc, Dims d, bool exact, hipStream_t stream);
 template <class T>
 hipError_t grad_params_finish(const double* acc, BoxParams<T> prm, T* gxmin, T* gxmax, T* gymin,
                               T* gymax, int n_boxes, float reparam_h, float reparam_w,

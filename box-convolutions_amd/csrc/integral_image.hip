@@ -79,7 +79,7 @@ band_prefix_kernel(double* __restrict__ aux, int64_t planes, int w, int nb) {
 template <class T, int WAVES, int M, int RB, bool VEC>
 __global__ void __launch_bounds__(WAVES * 64)
 band_scan_kernel(const T* __restrict__ in, T* __restrict__ out, const double* __restrict__ aux,
-                 int h, int w, int nb, int R) {
+                 int h, int w, int nb, int R, int64_t total, int64_t per_xcd, int reverse) {
     constexpr int NT = WAVES * 64;
     constexpr int CW = NT * 4;          // columns per chunk
     constexpr int TW = CW * M;          // columns per tile
@@ -88,7 +88,9 @@ band_scan_kernel(const T* __restrict__ in, T* __restrict__ out, const double* __
     __shared__ __align__(32) T stage[RB][TW];
     __shared__ double row_carry[256];   // prefix of each band row up to the current tile; R <= 256
 
-    const int64_t blk = blockIdx.x;     // p * nb + band
+    int64_t blk = xcd_contiguous_id(per_xcd);     // p * nb + band
+    if (blk >= total) return;
+    if (reverse) blk = total - 1 - blk;
     const int band = static_cast<int>(blk % nb);
     const int64_t p = blk / nb;
     const int r0 = band * R;
@@ -217,15 +219,18 @@ bool aligned_for_vec4(const T* p, int w) {
 
 template <class T, int WAVES, int M, int RB>
 hipError_t launch_scan(const T* in, T* out, const double* aux, int64_t planes, int h, int w,
-                       int nb, int R, hipStream_t stream) {
-    const dim3 grid(static_cast<unsigned>(planes * nb));
+                       int nb, int R, bool reverse, hipStream_t stream) {
+    const int64_t total = planes * nb;
+    const int64_t per_xcd = (total + kXcds - 1) / kXcds;
+    const int rev = reverse ? 1 : 0;
+    const dim3 grid(static_cast<unsigned>(per_xcd * kXcds));
     const dim3 block(WAVES * 64);
     if (aligned_for_vec4(in, w))
         BOXCONV_LAUNCH("band_scan", (band_scan_kernel<T, WAVES, M, RB, true>), grid, block, 0, stream,
-                       in, out, aux, h, w, nb, R);
+                       in, out, aux, h, w, nb, R, total, per_xcd, rev);
     else
         BOXCONV_LAUNCH("band_scan", (band_scan_kernel<T, WAVES, M, RB, false>), grid, block, 0, stream,
-                       in, out, aux, h, w, nb, R);
+                       in, out, aux, h, w, nb, R, total, per_xcd, rev);
     return hipGetLastError();
 }
 
@@ -253,7 +258,7 @@ IntegralPlan plan_integral(int64_t planes, int h, int w, int64_t want) {
 template <class T>
 hipError_t integral_image_launch(const T* in, T* out, int64_t planes, int h, int w,
                                  double* aux, const IntegralPlan& pl, bool colsums_ready,
-                                 hipStream_t stream) {
+                                 bool reverse_order, hipStream_t stream) {
     if (planes == 0) return hipSuccess;
     const int nb = pl.nb, R = pl.R;
     if (nb > 1 && !colsums_ready) {
@@ -272,16 +277,16 @@ hipError_t integral_image_launch(const T* in, T* out, int64_t planes, int h, int
         if (e != hipSuccess) return e;
     }
     // Tile width: one wave covers 256 columns per chunk, four waves 1024.
-    if (w <= 256)        return launch_scan<T, 1, 1, 4>(in, out, aux, planes, h, w, nb, R, stream);
-    else if (w <= 512)   return launch_scan<T, 2, 1, 4>(in, out, aux, planes, h, w, nb, R, stream);
-    else if (w <= 1024)  return launch_scan<T, 4, 1, 4>(in, out, aux, planes, h, w, nb, R, stream);
-    else if (w <= 2048)  return launch_scan<T, 4, 2, 2>(in, out, aux, planes, h, w, nb, R, stream);
-    else                 return launch_scan<T, 4, 4, 1>(in, out, aux, planes, h, w, nb, R, stream);
+    if (w <= 256)        return launch_scan<T, 1, 1, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
+    else if (w <= 512)   return launch_scan<T, 2, 1, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
+    else if (w <= 1024)  return launch_scan<T, 4, 1, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
+    else if (w <= 2048)  return launch_scan<T, 4, 2, 2>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
+    else                 return launch_scan<T, 4, 4, 1>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
 }
 
 template hipError_t integral_image_launch<float>(const float*, float*, int64_t, int, int,
-                                                 double*, const IntegralPlan&, bool, hipStream_t);
+                                                 double*, const IntegralPlan&, bool, bool, hipStream_t);
 template hipError_t integral_image_launch<double>(const double*, double*, int64_t, int, int,
-                                                  double*, const IntegralPlan&, bool, hipStream_t);
+                                                  double*, const IntegralPlan&, bool, bool, hipStream_t);
 
 }  // namespace boxconv

@@ -47,8 +47,9 @@ const char* boxconv_last_error(void);
  * boxconv_profile_arm(name): from now on every launch of the kernel called `name` is bracketed by
  * a pair of HIP events recorded on the stream it is launched on (so the time is that kernel's
  * alone, whatever else the entry point launches). Names: "band_colsum", "band_prefix",
- * "band_scan", "forward_rows", "grad_input_rows", "grad_params_rows", "param_grad_finalize",
- * "fill_zero", "clip", "forward_gather", "grad_input_gather", "grad_params_gather".
+ * "band_scan", "forward_rows", "grad_output_stream", "band_offsets", "grad_input_rows",
+ * "param_grad_finalize", "fill_zero", "clip", "forward_gather", "grad_input_gather",
+ * "grad_params_gather".
  * NULL or "" disarms. Arming discards earlier measurements.
  * boxconv_profile_collect(&total_ms, &launches): waits for the recorded events, returns the summed
  * kernel time and the number of launches, then disarms. Process-wide state; meant for benchmarks. */
@@ -93,7 +94,7 @@ int boxconv_forward_f64(const double* input_integrated, const double* x_min, con
  * normalisation term sum(grad_output*output) is recomputed from input_integrated instead of
  * re-reading it.
  * workspace: boxconv_backward_workspace_bytes(...) bytes, 256-byte aligned. It receives the
- * integral image of grad_output (the bulk), band sums and the per-box accumulators. */
+ * integral image of grad_output (the bulk), per-band row vectors and the per-box accumulators. */
 size_t boxconv_backward_workspace_bytes(int batch, int in_planes, int num_filters, int h, int w,
                                         int elem_size, int input_needs_grad,
                                         int params_need_grad);

@@ -43,15 +43,19 @@ def kernel_algorithmic_bytes(ab, elem=4):
 
 
 def load_measured_traffic(kernel, workload_name):
-    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), if a summary
-    for this kernel and workload has been recorded under profiles/."""
-    path = os.path.join(ROOT, "profiles", "traffic.json")
+    """HBM bytes per launch of `kernel` measured with rocprofv3 --pmc (FETCH_SIZE scaled by the
+    copy-kernel factor, plus WRITE_SIZE), read from the summary recorded under profiles/ for this
+    workload; None if there is none."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic_%s.txt" % workload_name)
     try:
         with open(path) as fh:
-            table = json.load(fh)
-        return table[workload_name][kernel]["bytes_per_launch"]
-    except (OSError, KeyError, ValueError):
-        return None
+            for line in fh:
+                parts = line.split()
+                if parts and not line.startswith("#") and parts[0] == kernel + "_kernel":
+                    return int(parts[3])
+    except (OSError, ValueError, IndexError):
+        pass
+    return None
 
 
 def cpu_baseline(k, ab_full):

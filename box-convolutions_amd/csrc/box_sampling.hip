@@ -503,7 +503,7 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
 #pragma unroll
         for (int k = 0; k < K; ++k) {
             const int j = tid + nt * k;
-            dst[k] = (valid && (FULL || j < w)) ? grow[j] : T(0);
+            dst[k] = (valid && (FULL || j < w)) ? __builtin_nontemporal_load(grow + j) : T(0);
         }
     };
     load_g(i0, g0);
@@ -636,8 +636,8 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
                 for (int k = 0; k < K; ++k) {
                     const int j = tid + nt * k;
                     if (FULL || j < w) {
-                        o0[j + 1] = lds.stage[j];
-                        if (second) o0[pitch + j + 1] = lds.stage[K * nt + j];
+                        __builtin_nontemporal_store(lds.stage[j], o0 + j + 1);
+                        if (second) __builtin_nontemporal_store(lds.stage[K * nt + j], o0 + pitch + j + 1);
                     }
                 }
                 if (tid == 0) {
@@ -842,9 +842,9 @@ inline int max_row_threads() {
     }();
     return v;
 }
-inline RowConfig row_config(int w) {
+inline RowConfig row_config(int w, int cap = 256) {
     RowConfig c;
-    c.nt = std::min(max_row_threads(), ((w + 63) / 64) * 64);
+    c.nt = std::min(std::min(max_row_threads(), cap), ((w + 63) / 64) * 64);
     const int k = (w + c.nt - 1) / c.nt;
     c.K = k <= 1 ? 1 : k <= 2 ? 2 : k <= 4 ? 4 : 8;
     c.full = (c.K * c.nt == w);
@@ -961,7 +961,7 @@ hipError_t grad_params_begin(double* acc, int n_boxes, hipStream_t stream) {
 
 StreamPlan plan_grad_output_stream(int64_t planes_f, int h, int w, size_t elem_size) {
     StreamPlan sp{};
-    const RowConfig rc = row_config(std::max(w, 1));
+    const RowConfig rc = row_config(std::max(w, 1), kMaxRowThreads);
     sp.usable = w <= kMaxRowStreamWidth && !force_gather_kernels() &&
                 stream_lds_bytes(rc.K, rc.nt, elem_size) <= kMaxDynamicLds;
     int nb = bands_for(std::max<int64_t>(planes_f, 1), h, 32, 2048);
@@ -985,7 +985,7 @@ hipError_t grad_output_stream_launch(const T* integ, const T* grad_out, BoxParam
     a.src = integ; a.grad_out = grad_out; a.acc = acc; a.dst = local_integral;
     a.nb = sp.nb; a.R = sp.R;
     finish_args(a, planes_f * a.nb);
-    const RowConfig rc = row_config(d.w);
+    const RowConfig rc = row_config(d.w, kMaxRowThreads);
     const dim3 grid(static_cast<unsigned>(a.per_xcd * kXcds));
     const size_t lds = stream_lds_bytes(rc.K, rc.nt, sizeof(T));
 #define LAUNCH_GS(KK, EX, FU) \

@@ -268,7 +268,7 @@ def clip_parameters(x_min, x_max, y_min, y_max, reparametrization_h, reparametri
 
 
 KERNEL_NAMES = ("band_colsum", "band_prefix", "band_scan", "forward_rows", "grad_output_stream",
-                "band_offsets", "grad_input_rows", "param_grad_finalize", "fill_zero", "clip",
+                "grad_input_rows", "param_grad_finalize", "fill_zero", "clip",
                 "forward_gather", "grad_input_gather", "grad_params_gather")
 
 

@@ -28,7 +28,9 @@ def reparametrize(
             y_min *= scale_w
             y_max *= scale_w
             return None
-        return x_min * scale_h, x_max * scale_h, y_min * scale_w, y_max * scale_w
+        # one multi-tensor launch instead of four; element-wise identical to `t * scale`
+        return tuple(torch._foreach_mul([x_min, x_max, y_min, y_max],
+                                        [scale_h, scale_h, scale_w, scale_w]))
 
 
 class BoxConvolutionFunction(torch.autograd.Function):

@@ -31,6 +31,7 @@
 // on one XCD and its integral plane stays in that XCD's L2.
 
 #include <cstdlib>
+#include <type_traits>
 
 #include "boxconv_device.hpp"
 #include "boxconv_host.hpp"
@@ -50,6 +51,16 @@ extern __shared__ __align__(16) unsigned char smem_raw[];
 // rather than more columns per lane: per-lane state (sliding rows, prefetched rows, accumulators)
 // scales with the columns per lane, and these kernels hide HBM latency with occupancy.
 constexpr int kMaxRowThreads = 512;
+#ifndef BOXCONV_GI_PREFETCH
+#define BOXCONV_GI_PREFETCH 1
+#endif
+#ifndef BOXCONV_GI_WAVES
+#define BOXCONV_GI_WAVES 1
+#endif
+#ifndef BOXCONV_GI_THREADS
+#define BOXCONV_GI_THREADS 256
+#endif
+constexpr bool kGradInputPrefetch = BOXCONV_GI_PREFETCH != 0;
 constexpr int kMaxRowWaves = kMaxRowThreads / 64;
 
 template <class T>
@@ -59,8 +70,7 @@ struct SampleArgs {
     T* dst;               // forward: [planes,F,h,w]; grad input: [planes,h,w]
     const T* grad_out;    // param grads only: [planes,F,h,w]
     double* acc;          // param grads only: [C*F*5]
-    const double* band_off;   // grad input only: per-band offsets of a band-local integral, or null
-    int off_nb, off_R;        // band structure of band_off
+    int off_R;                // grad input only: rows per band of a band-local integral, 0 = true integral
     int C, F, h, w;
     int nb, R;            // bands per plane and rows per band
     int64_t plane0;       // global index of the first plane (selects the boxes)
@@ -78,7 +88,7 @@ __device__ __forceinline__ void load_row(const T* __restrict__ plane, int64_t pi
 #pragma unroll
     for (int k = 0; k < K; ++k) {
         const int q = q0 + nt * k;
-        dst[k] = (FULL || q <= w) ? r[q] : T(0);
+        dst[k] = (FULL || q <= w) ? r[static_cast<unsigned>(q)] : T(0);
     }
 }
 
@@ -173,10 +183,14 @@ __global__ void __launch_bounds__(kMaxRowThreads) forward_rows_kernel(SampleArgs
     load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xhi, 0, h), w, q0, nt, bc);
     load_pair<T, K, FULL>(plane, pitch, i0, s.xlo, s.xhi, h, w, q0, nt, t0, t1, b1, b2);
 
+    // One row pair. PREFETCH is a compile-time tag: the loop body always issues the next pair's
+    // loads and the last pair is peeled, so no branch joins a path with loads in flight to one
+    // without (the wait-count insertion would have to drain the prefetch at such a join).
     int flip = 0;
-    for (int i = i0; i < i1; i += 2) {
+    auto row_pair = [&](int i, auto prefetch_tag) {
+        constexpr bool PREFETCH = decltype(prefetch_tag)::value;
         T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {};
-        if (i + 2 < i1)
+        if (PREFETCH)
             load_pair<T, K, FULL>(plane, pitch, i + 2, s.xlo, s.xhi, h, w, q0, nt, n0, n1, n2, n3);
 
         T* V0 = vbuf + flip * 2 * vlen;
@@ -200,32 +214,37 @@ __global__ void __launch_bounds__(kMaxRowThreads) forward_rows_kernel(SampleArgs
             if (FULL || j < w) {
                 const T o0 = blend<T, EXACT>(V0[lo[k]], V0[lo[k] + 1], V0[hi[k]], V0[hi[k] + 1],
                                              s.fylo, s.fyhi);
-                __builtin_nontemporal_store(o0 * scale, orow + j);
+                __builtin_nontemporal_store(o0 * scale, orow + static_cast<unsigned>(j));
                 if (second) {
                     const T o1 = blend<T, EXACT>(V1[lo[k]], V1[lo[k] + 1], V1[hi[k]],
                                                  V1[hi[k] + 1], s.fylo, s.fyhi);
-                    __builtin_nontemporal_store(o1 * scale, orow + w + j);
+                    __builtin_nontemporal_store(o1 * scale, orow + static_cast<unsigned>(w + j));
                 }
             }
         }
+        if (PREFETCH) {
 #pragma unroll
-        for (int k = 0; k < K; ++k) {
-            ta[k] = t1[k]; bc[k] = b2[k];
-            t0[k] = n0[k]; t1[k] = n1[k]; b1[k] = n2[k]; b2[k] = n3[k];
+            for (int k = 0; k < K; ++k) {
+                ta[k] = t1[k]; bc[k] = b2[k];
+                t0[k] = n0[k]; t1[k] = n1[k]; b1[k] = n2[k]; b2[k] = n3[k];
+            }
         }
-    }
+    };
+    int i = i0;
+    for (; i + 2 < i1; i += 2) row_pair(i, std::true_type{});
+    row_pair(i, std::false_type{});
 }
 
 // ---------------------------------------------------------------------------------------------
 // Gradient w.r.t. the input. Work item = (plane p = (b,c), band of RB rows); the F mirrored boxes
 // are visited in order and summed in registers, so no [B,C,F,h,w] temporary exists.
 //
-// OFFS: `src` holds BAND-LOCAL integral images (see grad_output_stream_kernel) and a.band_off the
-// per-band offsets. A box sum only involves differences between rows, so a row is corrected by
-// off[its band] - off[reference band], the reference being the band of the first row this
-// workgroup touches for the filter; the bulk of the integral cancels before it is ever added.
+// OFFS: `src` holds BAND-LOCAL integral images (see grad_output_stream_kernel). A box sum only
+// involves differences between rows, so a row is corrected relative to a reference band (that of
+// the first row this workgroup touches for the filter): the bulk of the integral cancels before
+// it is ever added.
 template <class T, int K, int RB, bool EXACT, bool FULL, bool OFFS>
-__global__ void __launch_bounds__(kMaxRowThreads) grad_input_rows_kernel(SampleArgs<T> a) {
+__global__ void __launch_bounds__(kMaxRowThreads, BOXCONV_GI_WAVES) grad_input_rows_kernel(SampleArgs<T> a) {
     static_assert(RB % 2 == 0, "rows are handled in pairs");
     const int64_t vid = xcd_contiguous_id(a.per_xcd);
     if (vid >= a.total) return;
@@ -256,26 +275,35 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_input_rows_kernel(SampleA
         int lo[K], hi[K];
         column_taps<K>(lo, hi, s.ylo, s.yhi, w, nt);
 
-        // offsets of the band a row lies in, relative to the reference band (OFFS only)
-        const double* offp = OFFS ? a.band_off + (p * a.F + f) * static_cast<int64_t>(a.off_nb) * pitch : nullptr;
-        auto band_of = [&](int row) { return max(row - 1, 0) / a.off_R; };
-        const int ref_band = OFFS ? band_of(clampi(i0 + s.xlo - 1, 0, h)) : 0;
-        int band_t = ref_band, band_b = -1;
+        // OFFS: `plane` holds a band-local integral (bands of off_R rows, each restarting at
+        // zero). Integral row r (1..h) belongs to band (r-1)/off_R; row 0 counts as band 0. The
+        // true integral is the stored row plus the bottom rows of all bands above it; relative to
+        // the reference band (that of the first row touched) only the bottom rows of the bands in
+        // between remain, summed in double. Rows only move down, so each side tracks the last row
+        // of its current band instead of dividing.
+        const int ref_band = OFFS ? max(clampi(i0 + s.xlo - 1, 0, h) - 1, 0) / a.off_R : 0;
+        int band_t = ref_band, band_b = ref_band;
+        int last_t = (ref_band + 1) * a.off_R, last_b = last_t;     // last row of the cached band
         T off_t[K], off_b[K];
 #pragma unroll
         for (int k = 0; k < K; ++k) { off_t[k] = T(0); off_b[k] = T(0); }
-        auto correct = [&](T (&row)[K], int row_index, int& cached_band, T (&cached)[K]) {
+        auto correct = [&](T (&row)[K], int row_index, int& cached_band, int& cached_last, T (&cached)[K]) {
             if (!OFFS) return;
-            const int bnd = band_of(row_index);
-            if (bnd != cached_band) {                       // uniform: depends on the row only
-                cached_band = bnd;
-                const double* ob = offp + static_cast<int64_t>(bnd) * pitch;
-                const double* orf = offp + static_cast<int64_t>(ref_band) * pitch;
+            if (row_index > cached_last) {                  // uniform: depends on the row only
+                do { ++cached_band; cached_last += a.off_R; } while (row_index > cached_last);
+                double sum[K];
 #pragma unroll
-                for (int k = 0; k < K; ++k) {
-                    const int q = q0 + nt * k;
-                    cached[k] = (FULL || q <= w) ? static_cast<T>(ob[q] - orf[q]) : T(0);
+                for (int k = 0; k < K; ++k) sum[k] = 0.0;
+                for (int b = ref_band; b < cached_band; ++b) {
+                    const T* bottom = plane + static_cast<int64_t>(min(h, (b + 1) * a.off_R)) * pitch;
+#pragma unroll
+                    for (int k = 0; k < K; ++k) {
+                        const int q = q0 + nt * k;
+                        if (FULL || q <= w) sum[k] += static_cast<double>(bottom[static_cast<unsigned>(q)]);
+                    }
                 }
+#pragma unroll
+                for (int k = 0; k < K; ++k) cached[k] = static_cast<T>(sum[k]);
             }
 #pragma unroll
             for (int k = 0; k < K; ++k) row[k] += cached[k];
@@ -285,21 +313,33 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_input_rows_kernel(SampleA
         load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), w, q0, nt, ta);
         load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xhi, 0, h), w, q0, nt, bc);
         load_pair<T, K, FULL>(plane, pitch, i0, s.xlo, s.xhi, h, w, q0, nt, t0, t1, b1, b2);
-        correct(ta, clampi(i0 + s.xlo - 1, 0, h), band_t, off_t);
-        correct(t0, clampi(i0 + s.xlo, 0, h), band_t, off_t);
-        correct(t1, clampi(i0 + 1 + s.xlo, 0, h), band_t, off_t);
-        correct(bc, clampi(i0 + s.xhi, 0, h), band_b, off_b);
-        correct(b1, clampi(i0 + 1 + s.xhi, 0, h), band_b, off_b);
-        correct(b2, clampi(i0 + 2 + s.xhi, 0, h), band_b, off_b);
+        correct(ta, clampi(i0 + s.xlo - 1, 0, h), band_t, last_t, off_t);
+        correct(t0, clampi(i0 + s.xlo, 0, h), band_t, last_t, off_t);
+        correct(t1, clampi(i0 + 1 + s.xlo, 0, h), band_t, last_t, off_t);
+        correct(bc, clampi(i0 + s.xhi, 0, h), band_b, last_b, off_b);
+        correct(b1, clampi(i0 + 1 + s.xhi, 0, h), band_b, last_b, off_b);
+        correct(b2, clampi(i0 + 2 + s.xhi, 0, h), band_b, last_b, off_b);
 
+        // All RB rows are always computed (rows past the image read clamped, valid rows and are
+        // not stored) and the prefetch of the next pair is decided at compile time: straight-line
+        // code, so loads stay in flight across the barrier.
 #pragma unroll
         for (int r = 0; r < RB; r += 2) {
             const int i = i0 + r;
-            if (i < h) {                                   // uniform across the workgroup
+            {
                 T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {};
-                const bool more = r + 2 < RB && i + 2 < h;
+                const bool more = kGradInputPrefetch && (r + 2 < RB);   // known after unrolling
                 if (more)
                     load_pair<T, K, FULL>(plane, pitch, i + 2, s.xlo, s.xhi, h, w, q0, nt, n0, n1, n2, n3);
+                if (!kGradInputPrefetch && r > 0) {
+                    load_pair<T, K, FULL>(plane, pitch, i, s.xlo, s.xhi, h, w, q0, nt, t0, t1, b1, b2);
+                    if (OFFS) {
+                        correct(t0, clampi(i + s.xlo, 0, h), band_t, last_t, off_t);
+                        correct(t1, clampi(i + 1 + s.xlo, 0, h), band_t, last_t, off_t);
+                        correct(b1, clampi(i + 1 + s.xhi, 0, h), band_b, last_b, off_b);
+                        correct(b2, clampi(i + 2 + s.xhi, 0, h), band_b, last_b, off_b);
+                    }
+                }
                 T* V0 = vbuf + flip * 2 * vlen;
                 T* V1 = V0 + vlen;
                 flip ^= 1;
@@ -325,13 +365,13 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_input_rows_kernel(SampleA
 #pragma unroll
                 for (int k = 0; k < K; ++k) {
                     ta[k] = t1[k]; bc[k] = b2[k];
-                    t0[k] = n0[k]; t1[k] = n1[k]; b1[k] = n2[k]; b2[k] = n3[k];
+                    if (more) { t0[k] = n0[k]; t1[k] = n1[k]; b1[k] = n2[k]; b2[k] = n3[k]; }
                 }
                 if (OFFS && more) {
-                    correct(t0, clampi(i + 2 + s.xlo, 0, h), band_t, off_t);
-                    correct(t1, clampi(i + 3 + s.xlo, 0, h), band_t, off_t);
-                    correct(b1, clampi(i + 3 + s.xhi, 0, h), band_b, off_b);
-                    correct(b2, clampi(i + 4 + s.xhi, 0, h), band_b, off_b);
+                    correct(t0, clampi(i + 2 + s.xlo, 0, h), band_t, last_t, off_t);
+                    correct(t1, clampi(i + 3 + s.xlo, 0, h), band_t, last_t, off_t);
+                    correct(b1, clampi(i + 3 + s.xhi, 0, h), band_b, last_b, off_b);
+                    correct(b2, clampi(i + 4 + s.xhi, 0, h), band_b, last_b, off_b);
                 }
             }
         }
@@ -345,7 +385,7 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_input_rows_kernel(SampleA
 #pragma unroll
             for (int k = 0; k < K; ++k) {
                 const int j = static_cast<int>(threadIdx.x) + nt * k;
-                if (FULL || j < w) out[static_cast<int64_t>(i) * w + j] = acc[r][k];
+                if (FULL || j < w) (out + static_cast<int64_t>(i) * w)[static_cast<unsigned>(j)] = acc[r][k];
             }
         }
     }
@@ -389,8 +429,8 @@ __device__ __forceinline__ void block_accumulate5(const double (&v)[5], double* 
 //
 // (SCAN) the BAND-LOCAL integral image of grad_output: L[i+1][c+1] = sum of grad_output over rows
 // band_start..i and columns 0..c. Bands do not depend on each other, so nothing has to be known
-// about the rows above: the true integral is L plus a per-band row vector (band_offsets_kernel)
-// that the grad-input kernel adds when it loads a row. Column accumulators and the row prefix are
+// about the rows above: the true integral is L plus the bottom rows of the bands above, which
+// the grad-input kernel adds when it loads a row. Column accumulators and the row prefix are
 // carried in double; lanes own K consecutive columns for this part (read back from the LDS row),
 // results go through an LDS stage so that global stores are lane-consecutive dwords.
 //
@@ -439,7 +479,8 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
     const int64_t p = pf / a.F;
     const int k_par = static_cast<int>((a.plane0 + p) % a.C) * a.F + f;
     const int h = a.h, w = a.w, nt = blockDim.x, tid = threadIdx.x, q0 = 1 + tid;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keep it scalar
 
     const BoxOfWorkgroup<T> bx = load_box(a.prm, k_par);
     const BoxSplit<T> s = split_grad_params(bx.xmin, bx.xmax, bx.ymin, bx.ymax);
@@ -503,16 +544,17 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
 #pragma unroll
         for (int k = 0; k < K; ++k) {
             const int j = tid + nt * k;
-            dst[k] = (valid && (FULL || j < w)) ? __builtin_nontemporal_load(grow + j) : T(0);
+            dst[k] = (valid && (FULL || j < w)) ? __builtin_nontemporal_load(grow + static_cast<unsigned>(j)) : T(0);
         }
     };
     load_g(i0, g0);
     load_g(i0 + 1, g1);
 
     int flip = 0;
-    for (int i = i0; i < i1; i += 2) {
+    auto row_pair = [&](int i, auto prefetch_tag) {
+        constexpr bool PREFETCH = decltype(prefetch_tag)::value;   // see forward_rows_kernel
         T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {}, m0[K] = {}, m1[K] = {};
-        if (i + 2 < i1) {
+        if (PREFETCH) {
             if (PARAMS)
                 load_pair<T, K, FULL>(plane, pitch, i + 2, s.xlo, s.xhi, h, w, q0, nt, n0, n1, n2, n3);
             load_g(i + 2, m0);
@@ -619,7 +661,12 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
             }
             __syncthreads();                                                 // wave totals visible
             {
-                for (int wv = 0; wv < wave; ++wv) { carry0 += lds.wave_tot[wv]; carry1 += lds.wave_tot[kMaxRowWaves + wv]; }
+#pragma unroll
+                for (int wv = 0; wv < kMaxRowWaves - 1; ++wv)
+                    if (wv < wave) {                                         // scalar condition
+                        carry0 += lds.wave_tot[wv];
+                        carry1 += lds.wave_tot[kMaxRowWaves + wv];
+                    }
                 T* s0 = lds.stage + K * tid;
                 T* s1 = lds.stage + K * nt + K * tid;
 #pragma unroll
@@ -631,13 +678,14 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
             __syncthreads();                                                 // stage visible
             {
                 T* o0 = lrows + static_cast<int64_t>(i + 1) * pitch;
+                T* o1 = o0 + pitch;
                 const bool second = i + 1 < i1;
 #pragma unroll
                 for (int k = 0; k < K; ++k) {
                     const int j = tid + nt * k;
                     if (FULL || j < w) {
-                        __builtin_nontemporal_store(lds.stage[j], o0 + j + 1);
-                        if (second) __builtin_nontemporal_store(lds.stage[K * nt + j], o0 + pitch + j + 1);
+                        __builtin_nontemporal_store(lds.stage[j], o0 + static_cast<unsigned>(j + 1));
+                        if (second) __builtin_nontemporal_store(lds.stage[K * nt + j], o1 + static_cast<unsigned>(j + 1));
                     }
                 }
                 if (tid == 0) {
@@ -647,15 +695,20 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
             }
         }
 
+        if (PREFETCH) {
 #pragma unroll
-        for (int k = 0; k < K; ++k) {
-            if (PARAMS) {
-                ta[k] = t1[k]; bc[k] = b2[k];
-                t0[k] = n0[k]; t1[k] = n1[k]; b1[k] = n2[k]; b2[k] = n3[k];
+            for (int k = 0; k < K; ++k) {
+                if (PARAMS) {
+                    ta[k] = t1[k]; bc[k] = b2[k];
+                    t0[k] = n0[k]; t1[k] = n1[k]; b1[k] = n2[k]; b2[k] = n3[k];
+                }
+                g0[k] = m0[k]; g1[k] = m1[k];
             }
-            g0[k] = m0[k]; g1[k] = m1[k];
         }
-    }
+    };
+    int i = i0;
+    for (; i + 2 < i1; i += 2) row_pair(i, std::true_type{});
+    row_pair(i, std::false_type{});
 
     if (PARAMS) {
         __syncthreads();
@@ -663,28 +716,6 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
                              static_cast<double>(sum[2]), static_cast<double>(sum[3]),
                              static_cast<double>(sum[4])};
         block_accumulate5(v, a.acc + static_cast<int64_t>(k_par) * 5, lds.red);
-    }
-}
-
-// Per-band offsets of the band-local integral written by grad_output_stream_kernel:
-// off[pf][k][c] = true integral at the top edge of band k = sum of the bottom rows of the bands
-// above (double). One thread per (plane, column).
-template <class T>
-__global__ void __launch_bounds__(256)
-band_offsets_kernel(const T* __restrict__ lrows, double* __restrict__ off, int64_t planes_f, int h,
-                    int w, int nb, int R) {
-    const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    const int64_t W1 = w + 1;
-    if (idx >= planes_f * W1) return;
-    const int64_t pf = idx / W1;
-    const int c = static_cast<int>(idx % W1);
-    const T* plane = lrows + pf * static_cast<int64_t>(h + 1) * W1;
-    double* o = off + pf * static_cast<int64_t>(nb) * W1 + c;
-    double run = 0.0;
-    for (int k = 0; k < nb; ++k) {
-        o[static_cast<int64_t>(k) * W1] = run;
-        const int bottom = min(h, (k + 1) * R);
-        run += static_cast<double>(plane[static_cast<int64_t>(bottom) * W1 + c]);
     }
 }
 
@@ -844,7 +875,11 @@ inline int max_row_threads() {
 }
 inline RowConfig row_config(int w, int cap = 256) {
     RowConfig c;
+    // `cap` threads are preferred (measured fastest at widths up to 1024); wider rows take the
+    // largest workgroup instead of more than 4 columns per lane, which keeps the register
+    // footprint and the length of the per-lane float accumulation chains bounded.
     c.nt = std::min(std::min(max_row_threads(), cap), ((w + 63) / 64) * 64);
+    if ((w + c.nt - 1) / c.nt > 4) c.nt = std::min(max_row_threads(), ((w + 63) / 64) * 64);
     const int k = (w + c.nt - 1) / c.nt;
     c.K = k <= 1 ? 1 : k <= 2 ? 2 : k <= 4 ? 4 : 8;
     c.full = (c.K * c.nt == w);
@@ -920,16 +955,15 @@ hipError_t forward_launch(const T* integ, BoxParams<T> prm, T* out, Dims d, bool
 }
 
 template <class T>
-hipError_t grad_input_launch(const T* gint, const double* band_off, int off_nb, int off_R,
-                             BoxParams<T> prm, T* grad_in, Dims d, bool normalize, bool exact,
-                             hipStream_t stream) {
+hipError_t grad_input_launch(const T* gint, int band_rows, BoxParams<T> prm, T* grad_in, Dims d,
+                             bool normalize, bool exact, hipStream_t stream) {
     if (d.planes == 0 || d.hw() == 0) return hipSuccess;
     SampleArgs<T> a = base_args(prm, d);
     a.src = gint; a.dst = grad_in; a.normalize = normalize ? 1 : 0;
-    a.band_off = band_off; a.off_nb = off_nb; a.off_R = std::max(off_R, 1);
+    a.off_R = band_rows;
 
     if (d.w > kMaxRowStreamWidth || force_gather_kernels()) {
-        if (band_off != nullptr) return hipErrorInvalidValue;   // the gather kernel needs a true integral
+        if (band_rows > 0) return hipErrorInvalidValue;         // the gather kernel needs a true integral
         finish_args(a, d.planes * d.hw());
         const dim3 grid(static_cast<unsigned>((a.total + 255) / 256));
         if (exact) BOXCONV_LAUNCH("grad_input_gather", (grad_input_gather_kernel<T, true>), grid, dim3(256), 0, stream, a);
@@ -938,14 +972,18 @@ hipError_t grad_input_launch(const T* gint, const double* band_off, int off_nb, 
     }
 
     constexpr int RB = 8;
-    const RowConfig rc = row_config(d.w);
+    static const int gi_threads = [] {
+        const char* e = std::getenv("BOXCONV_GI_THREADS");
+        return e ? std::atoi(e) : BOXCONV_GI_THREADS;
+    }();
+    const RowConfig rc = row_config(d.w, gi_threads);
     a.nb = (d.h + RB - 1) / RB;
     a.R = RB;
     finish_args(a, d.planes * a.nb);
     const dim3 grid(static_cast<unsigned>(a.per_xcd * kXcds));
     const size_t lds = 4 * static_cast<size_t>(d.w + 3) * sizeof(T);
 #define LAUNCH_GI(KK, EX, FU) \
-    if (band_off != nullptr) BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, KK, RB, EX, FU, true>), grid, dim3(rc.nt), lds, stream, a); \
+    if (band_rows > 0) BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, KK, RB, EX, FU, true>), grid, dim3(rc.nt), lds, stream, a); \
     else BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, KK, RB, EX, FU, false>), grid, dim3(rc.nt), lds, stream, a)
     BOXCONV_DISPATCH_K_EXACT_FULL(LAUNCH_GI, rc.K, exact, rc.full)
 #undef LAUNCH_GI
@@ -961,7 +999,7 @@ hipError_t grad_params_begin(double* acc, int n_boxes, hipStream_t stream) {
 
 StreamPlan plan_grad_output_stream(int64_t planes_f, int h, int w, size_t elem_size) {
     StreamPlan sp{};
-    const RowConfig rc = row_config(std::max(w, 1), kMaxRowThreads);
+    const RowConfig rc = row_config(std::max(w, 1));
     sp.usable = w <= kMaxRowStreamWidth && !force_gather_kernels() &&
                 stream_lds_bytes(rc.K, rc.nt, elem_size) <= kMaxDynamicLds;
     int nb = bands_for(std::max<int64_t>(planes_f, 1), h, 32, 2048);
@@ -969,14 +1007,13 @@ StreamPlan plan_grad_output_stream(int64_t planes_f, int h, int w, size_t elem_s
     R += R & 1;                                        // rows are handled in pairs
     sp.R = std::max(R, 2);
     sp.nb = (h + sp.R - 1) / sp.R;
-    sp.offset_doubles = planes_f * static_cast<int64_t>(sp.nb) * (w + 1);
     return sp;
 }
 
 template <class T>
 hipError_t grad_output_stream_launch(const T* integ, const T* grad_out, BoxParams<T> prm,
-                                     double* acc, T* local_integral, double* band_off,
-                                     const StreamPlan& sp, Dims d, bool exact, hipStream_t stream) {
+                                     double* acc, T* local_integral, const StreamPlan& sp, Dims d,
+                                     bool exact, hipStream_t stream) {
     const int64_t planes_f = d.planes * d.F;
     if (planes_f == 0 || d.hw() == 0) return hipSuccess;
     const bool params = acc != nullptr, scan = local_integral != nullptr;
@@ -985,7 +1022,7 @@ hipError_t grad_output_stream_launch(const T* integ, const T* grad_out, BoxParam
     a.src = integ; a.grad_out = grad_out; a.acc = acc; a.dst = local_integral;
     a.nb = sp.nb; a.R = sp.R;
     finish_args(a, planes_f * a.nb);
-    const RowConfig rc = row_config(d.w, kMaxRowThreads);
+    const RowConfig rc = row_config(d.w);
     const dim3 grid(static_cast<unsigned>(a.per_xcd * kXcds));
     const size_t lds = stream_lds_bytes(rc.K, rc.nt, sizeof(T));
 #define LAUNCH_GS(KK, EX, FU) \
@@ -994,11 +1031,6 @@ hipError_t grad_output_stream_launch(const T* integ, const T* grad_out, BoxParam
     else                BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_kernel<T, KK, EX, FU, false, true>), grid, dim3(rc.nt), lds, stream, a)
     BOXCONV_DISPATCH_K_EXACT_FULL(LAUNCH_GS, rc.K, exact, rc.full)
 #undef LAUNCH_GS
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess || !scan) return e;
-    const int64_t n = planes_f * (d.w + 1);
-    BOXCONV_LAUNCH("band_offsets", (band_offsets_kernel<T>), dim3(static_cast<unsigned>((n + 255) / 256)),
-                   dim3(256), 0, stream, local_integral, band_off, planes_f, d.h, d.w, sp.nb, sp.R);
     return hipGetLastError();
 }
 
@@ -1031,11 +1063,10 @@ hipError_t grad_params_finish(const double* acc, BoxParams<T> prm, T* gxmin, T* 
 
 #define BOXCONV_INSTANTIATE(T)                                                                     \
     template hipError_t forward_launch<T>(const T*, BoxParams<T>, T*, Dims, bool, bool, hipStream_t); \
-    template hipError_t grad_input_launch<T>(const T*, const double*, int, int, BoxParams<T>, T*,  \
-                                             Dims, bool, bool, hipStream_t);                       \
+    template hipError_t grad_input_launch<T>(const T*, int, BoxParams<T>, T*, Dims, bool, bool,    \
+                                             hipStream_t);                                         \
     template hipError_t grad_output_stream_launch<T>(const T*, const T*, BoxParams<T>, double*, T*, \
-                                                     double*, const StreamPlan&, Dims, bool,       \
-                                                     hipStream_t);                                 \
+                                                     const StreamPlan&, Dims, bool, hipStream_t);  \
     template hipError_t grad_params_gather_launch<T>(const T*, const T*, BoxParams<T>, double*,    \
                                                      Dims, bool, hipStream_t);                     \
     template hipError_t grad_params_finish<T>(const double*, BoxParams<T>, T*, T*, T*, T*, int,    \

@@ -107,7 +107,7 @@ bool reverse_second_pass() {
 
 // Workspace of the backward pass:
 //   [integral of grad_output: chunk*F planes of (h+1)(w+1)]   only if grad_input is wanted
-//   [aux doubles: band offsets (streaming path) or band column sums (three-pass fallback)]
+//   [aux doubles: band column sums, three-pass fallback only]
 //   [acc: C*F*5 doubles]                                       only if parameter gradients are wanted
 struct BackwardLayout {
     size_t gint_off, aux_off, acc_off, total;
@@ -136,9 +136,8 @@ BackwardLayout backward_layout(int batch, int in_planes, int num_filters, int h,
                         num_filters * (h + 1) * (w + 1) * elem_size, 256);
         L.aux_off = off;
         const int64_t aux = max_over_chunks(std::max<int64_t>(planes, 1), L.chunk, [&](int64_t np) {
-            return L.streaming
-                ? boxconv::plan_grad_output_stream(np * num_filters, h, w, elem_size).offset_doubles
-                : boxconv::plan_integral(np * num_filters, h, w).aux_doubles;
+            return L.streaming ? int64_t(0)
+                               : boxconv::plan_integral(np * num_filters, h, w).aux_doubles;
         });
         off += align_up(static_cast<size_t>(aux) * 8, 256);
     }
@@ -236,12 +235,12 @@ int backward_impl(const T* integ, const T* x_min, const T* x_max, const T* y_min
             const boxconv::StreamPlan sp =
                 boxconv::plan_grad_output_stream(np * num_filters, h, w, sizeof(T));
             if (int rc = hip_result(boxconv::grad_output_stream_launch<T>(
-                    integ_chunk, go_chunk, prm, acc, gint, aux, sp, d, exact != 0, s),
+                    integ_chunk, go_chunk, prm, acc, gint, sp, d, exact != 0, s),
                     "grad_output streaming launch"))
                 return rc;
             if (need_input)
                 if (int rc = hip_result(boxconv::grad_input_launch<T>(
-                        gint, aux, sp.nb, sp.R, prm, gin_chunk, d, normalize != 0, exact != 0, s),
+                        gint, sp.R, prm, gin_chunk, d, normalize != 0, exact != 0, s),
                         "input-gradient launch"))
                     return rc;
         } else {
@@ -259,7 +258,7 @@ int backward_impl(const T* integ, const T* x_min, const T* x_max, const T* y_min
                         "grad_output integral image launch"))
                     return rc;
                 if (int rc = hip_result(boxconv::grad_input_launch<T>(
-                        gint, nullptr, 0, 1, prm, gin_chunk, d, normalize != 0, exact != 0, s),
+                        gint, 0, prm, gin_chunk, d, normalize != 0, exact != 0, s),
                         "input-gradient launch"))
                     return rc;
             }

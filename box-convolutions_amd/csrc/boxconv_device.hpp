@@ -86,32 +86,35 @@ __device__ __forceinline__ T inverse_extent(T xmin, T xmax, T ymin, T ymax, bool
 
 // ---------------------------------------------------------------------------------------------
 // Cross-lane data movement (DPP). `Ctrl` values used: 0x111..0x11f row_shr:1..15,
-// 0x142 row_bcast:15, 0x143 row_bcast:31. Lanes without a valid source, or disabled by the
-// row mask, receive 0.
+// 0x142 row_bcast:15, 0x143 row_bcast:31. A lane whose source lane does not exist reads 0
+// (bound_ctrl); a lane in a row disabled by RowMask keeps `keep`.
 template <int Ctrl, int RowMask>
-__device__ __forceinline__ int dpp_or_zero(int v) {
-    return __builtin_amdgcn_update_dpp(0, v, Ctrl, RowMask, 0xf, true);
+__device__ __forceinline__ int dpp_move(int keep, int v) {
+    return __builtin_amdgcn_update_dpp(keep, v, Ctrl, RowMask, 0xf, true);
 }
 template <int Ctrl, int RowMask>
-__device__ __forceinline__ double dpp_or_zero(double v) {
-    const int lo = dpp_or_zero<Ctrl, RowMask>(__double2loint(v));
-    const int hi = dpp_or_zero<Ctrl, RowMask>(__double2hiint(v));
+__device__ __forceinline__ double dpp_move(double keep, double v) {
+    const int lo = dpp_move<Ctrl, RowMask>(__double2loint(keep), __double2loint(v));
+    const int hi = dpp_move<Ctrl, RowMask>(__double2hiint(keep), __double2hiint(v));
     return __hiloint2double(hi, lo);
 }
 template <int Ctrl, int RowMask>
-__device__ __forceinline__ float dpp_or_zero(float v) {
-    return __int_as_float(dpp_or_zero<Ctrl, RowMask>(__float_as_int(v)));
+__device__ __forceinline__ float dpp_move(float keep, float v) {
+    return __int_as_float(dpp_move<Ctrl, RowMask>(__float_as_int(keep), __float_as_int(v)));
 }
 
 // Inclusive prefix sum across the 64 lanes of a wave. All lanes must be active.
 template <class A>
 __device__ __forceinline__ A wave_inclusive_scan(A x) {
-    x += dpp_or_zero<0x111, 0xf>(x);   // within each row of 16 lanes
-    x += dpp_or_zero<0x112, 0xf>(x);
-    x += dpp_or_zero<0x114, 0xf>(x);
-    x += dpp_or_zero<0x118, 0xf>(x);
-    x += dpp_or_zero<0x142, 0xa>(x);   // lane 15 of rows 0,2 into rows 1,3
-    x += dpp_or_zero<0x143, 0xc>(x);   // lane 31 into rows 2,3
+    // within each row of 16 lanes (every row enabled, so `keep` is never used: pass x itself
+    // and no register has to be cleared first)
+    x += dpp_move<0x111, 0xf>(x, x);
+    x += dpp_move<0x112, 0xf>(x, x);
+    x += dpp_move<0x114, 0xf>(x, x);
+    x += dpp_move<0x118, 0xf>(x, x);
+    const A zero = A(0);
+    x += dpp_move<0x142, 0xa>(zero, x);   // lane 15 of rows 0,2 into rows 1,3
+    x += dpp_move<0x143, 0xc>(zero, x);   // lane 31 into rows 2,3
     return x;
 }
 

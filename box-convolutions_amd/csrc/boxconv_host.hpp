@@ -49,28 +49,26 @@ template <class T>
 hipError_t forward_launch(const T* integ, BoxParams<T> prm, T* out, Dims d, bool normalize,
                           bool exact, hipStream_t stream);
 
-// band_off: null when `gint` holds true integral images; otherwise `gint` holds band-local
-// integrals with bands of off_R rows (off_nb per plane) and band_off their offsets.
+// band_rows: 0 when `gint` holds true integral images; otherwise `gint` holds band-local
+// integrals (each band of band_rows rows restarts at zero).
 template <class T>
-hipError_t grad_input_launch(const T* gint, const double* band_off, int off_nb, int off_R,
-                             BoxParams<T> prm, T* grad_in, Dims d, bool normalize, bool exact,
-                             hipStream_t stream);
+hipError_t grad_input_launch(const T* gint, int band_rows, BoxParams<T> prm, T* grad_in, Dims d,
+                             bool normalize, bool exact, hipStream_t stream);
 
 // The streaming pass over grad_output (parameter-gradient sums and/or band-local integral).
 struct StreamPlan {
     bool usable;             // false: width or LDS need outside what the streaming kernel covers
     int nb, R;               // bands per plane, rows per band (R even)
-    int64_t offset_doubles;  // size of the band-offset array: planes*F * nb * (w+1)
 };
 StreamPlan plan_grad_output_stream(int64_t planes_f, int h, int w, size_t elem_size);
 
 // acc ([C*F*5] doubles, cleared by grad_params_begin) may be null: no parameter sums.
-// local_integral ([planes*F, h+1, w+1]) may be null: no integral; with it band_off receives the
-// per-band offsets. At least one of the two must be given.
+// local_integral ([planes*F, h+1, w+1]) may be null: no integral. At least one of the two must
+// be given.
 template <class T>
 hipError_t grad_output_stream_launch(const T* integ, const T* grad_out, BoxParams<T> prm,
-                                     double* acc, T* local_integral, double* band_off,
-                                     const StreamPlan& sp, Dims d, bool exact, hipStream_t stream);
+                                     double* acc, T* local_integral, const StreamPlan& sp, Dims d,
+                                     bool exact, hipStream_t stream);
 
 hipError_t grad_params_begin(double* acc, int n_boxes, hipStream_t stream);
 template <class T>

@@ -97,7 +97,7 @@ band_scan_kernel(const T* __restrict__ in, T* __restrict__ out, const double* __
     const int r1 = min(h, r0 + R);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keep it scalar
     const int64_t W1 = static_cast<int64_t>(w) + 1;
 
     const T* src = in + p * static_cast<int64_t>(h) * w;

@@ -8,6 +8,14 @@ result), plus a size-independent property on the whole tensors: the adjoint iden
 <boxconv(x), g> = <x, grad_input(g)>.
 
 Tolerances: forward, grad_input 1e-4; parameter gradients 1e-3 (max|gpu-cpu| / max|cpu|).
+
+Workload 5 (inputs near 10.5, integral-image entries up to 2.2e7 where a float32 ulp is 2) is at
+the precision limit of the float32 reference itself: its parameter gradients are differences of
+two nearly equal terms (for a constant image the gradient of a normalised box vanishes), and the
+reference's float32 result deviates from the same algorithm run in float64 by about 2e-3
+(measured: y_max 1.8e-3), the GPU result by about 3e-4. There the GPU is held to 1e-3 against
+the float64 oracle, must be at least as close to it as the float32 oracle is, and to 4e-3
+against the float32 oracle.
 """
 import numpy as np
 import pytest
@@ -67,4 +75,22 @@ def test_baseline_workload(oracle, k):
     print("workload %d: forward %.2e grad_input %.2e grad_params %s" % (k, e_out, e_gin, ["%.2e" % e for e in e_par]))
     assert e_out <= 1e-4
     assert e_gin <= 1e-4
-    assert max(e_par) <= 1e-3
+    if k != 5:
+        assert max(e_par) <= 1e-3
+        return
+
+    # workload 5: the same algorithm in float64 on the same (float32-rounded) real-unit boxes
+    real = [(a.astype(np.float32) * np.float32(r)).astype(np.float64) for a, r in
+            zip(args[1:], (sub.reparametrization_h,) * 2 + (sub.reparametrization_w,) * 2)]
+    integ64 = oracle.integral_image(args[0].astype(np.float64))
+    out64 = oracle.box_forward(integ64, *real, True, True)
+    grads64 = oracle.box_backward(integ64, *real, sub.grad_output.numpy().astype(np.float64), out64,
+                                  sub.reparametrization_h, sub.reparametrization_w, True, True)
+    floor64 = param_grad_floor(grads64[1:])
+    e_gpu64 = [rel_err(gp[:c].cpu().numpy(), g64, floor64) for gp, g64 in zip(gpar, grads64[1:])]
+    e_cpu64 = [rel_err(gc, g64, floor64) for gc, g64 in zip(grads_c[1:], grads64[1:])]
+    print("workload 5 vs float64 oracle: gpu %s  float32 oracle %s"
+          % (["%.2e" % e for e in e_gpu64], ["%.2e" % e for e in e_cpu64]))
+    assert max(e_gpu64) <= 1e-3
+    assert max(e_gpu64) <= max(max(e_cpu64), 1e-4)
+    assert max(e_par) <= 4e-3

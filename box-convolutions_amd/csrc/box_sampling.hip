@@ -51,16 +51,12 @@ extern __shared__ __align__(16) unsigned char smem_raw[];
 // rather than more columns per lane: per-lane state (sliding rows, prefetched rows, accumulators)
 // scales with the columns per lane, and these kernels hide HBM latency with occupancy.
 constexpr int kMaxRowThreads = 512;
-#ifndef BOXCONV_GI_PREFETCH
-#define BOXCONV_GI_PREFETCH 1
-#endif
 #ifndef BOXCONV_GI_WAVES
 #define BOXCONV_GI_WAVES 1
 #endif
 #ifndef BOXCONV_GI_THREADS
 #define BOXCONV_GI_THREADS 256
 #endif
-constexpr bool kGradInputPrefetch = BOXCONV_GI_PREFETCH != 0;
 constexpr int kMaxRowWaves = kMaxRowThreads / 64;
 
 template <class T>
@@ -79,29 +75,53 @@ struct SampleArgs {
     int normalize;
 };
 
+// Two rows of the same column, adjacent in LDS: every LDS access of the row kernels moves the
+// values of both rows of the current row pair at once.
+template <class T>
+struct alignas(2 * sizeof(T)) RowPair {
+    T r0, r1;
+};
+
+// Pointer plus a byte offset held in a 32-bit register. Global accesses written this way use a
+// scalar base and one VGPR offset, LDS accesses an immediate base; no per-access address math.
+template <class P>
+__device__ __forceinline__ P* at_bytes(P* base, unsigned bytes) {
+    using Byte = std::conditional_t<std::is_const<P>::value, const char, char>;
+    return reinterpret_cast<P*>(reinterpret_cast<Byte*>(base) + bytes);
+}
+
+// Per-lane column slots. Lane `tid` owns integral columns q = 1 + tid + nt*k (pixel columns
+// j = q - 1), k < K. qoff[k] = q * sizeof(T) is the byte offset of column q in a row of T.
 // FULL: w == K * blockDim.x, so every (lane, k) slot is a valid column and no bounds checks are
-// compiled in.
+// compiled in; otherwise a slot is valid iff qoff[k] <= w * sizeof(T).
+template <class T, int K>
+__device__ __forceinline__ void lane_columns(unsigned (&qoff)[K], int nt) {
+#pragma unroll
+    for (int k = 0; k < K; ++k)
+        qoff[k] = static_cast<unsigned>(1 + static_cast<int>(threadIdx.x) + nt * k) *
+                  static_cast<unsigned>(sizeof(T));
+}
+
 template <class T, int K, bool FULL>
 __device__ __forceinline__ void load_row(const T* __restrict__ plane, int64_t pitch, int row,
-                                         int w, int q0, int nt, T (&dst)[K]) {
+                                         unsigned row_bytes, const unsigned (&qoff)[K], T (&dst)[K]) {
     const T* r = plane + static_cast<int64_t>(row) * pitch;
 #pragma unroll
-    for (int k = 0; k < K; ++k) {
-        const int q = q0 + nt * k;
-        dst[k] = (FULL || q <= w) ? r[static_cast<unsigned>(q)] : T(0);
-    }
+    for (int k = 0; k < K; ++k)
+        dst[k] = (FULL || qoff[k] <= row_bytes) ? *at_bytes(r, qoff[k]) : T(0);
 }
 
 // The four rows that become new when the window moves from output rows (i-2, i-1) to (i, i+1):
 // I[t(i)], I[t(i+1)], I[b(i+1)], I[b(i+2)].
 template <class T, int K, bool FULL>
 __device__ __forceinline__ void load_pair(const T* __restrict__ plane, int64_t pitch, int i,
-                                          int xlo, int xhi, int h, int w, int q0, int nt,
-                                          T (&t0)[K], T (&t1)[K], T (&b1)[K], T (&b2)[K]) {
-    load_row<T, K, FULL>(plane, pitch, clampi(i + xlo, 0, h), w, q0, nt, t0);
-    load_row<T, K, FULL>(plane, pitch, clampi(i + 1 + xlo, 0, h), w, q0, nt, t1);
-    load_row<T, K, FULL>(plane, pitch, clampi(i + 1 + xhi, 0, h), w, q0, nt, b1);
-    load_row<T, K, FULL>(plane, pitch, clampi(i + 2 + xhi, 0, h), w, q0, nt, b2);
+                                          int xlo, int xhi, int h, unsigned row_bytes,
+                                          const unsigned (&qoff)[K], T (&t0)[K], T (&t1)[K],
+                                          T (&b1)[K], T (&b2)[K]) {
+    load_row<T, K, FULL>(plane, pitch, clampi(i + xlo, 0, h), row_bytes, qoff, t0);
+    load_row<T, K, FULL>(plane, pitch, clampi(i + 1 + xlo, 0, h), row_bytes, qoff, t1);
+    load_row<T, K, FULL>(plane, pitch, clampi(i + 1 + xhi, 0, h), row_bytes, qoff, b1);
+    load_row<T, K, FULL>(plane, pitch, clampi(i + 2 + xhi, 0, h), row_bytes, qoff, b2);
 }
 
 template <class T, bool EXACT>
@@ -111,30 +131,50 @@ __device__ __forceinline__ T blend(T lo_adv, T lo, T hi, T hi_adv, T flo, T fhi)
     return v;
 }
 
-// Row vector into LDS. Layout: V[q+1] for q = -1..w+1 with V(-1) = V(0) = 0 and V(w+1) = V(w), so
-// a clamped column pair is always two adjacent entries.
+// Row vectors V(i), V(i+1) into LDS. Layout: V[q+1] for q = -1..w+1 with V(-1) = V(0) = 0 (written
+// once by clear_row_pads) and V(w+1) = V(w), so a clamped column pair is always two adjacent
+// entries.
 template <class T, int K, bool FULL>
-__device__ __forceinline__ void publish_row(T* __restrict__ V, const T (&val)[K], int w, int q0,
-                                            int nt) {
+__device__ __forceinline__ void publish_rows(RowPair<T>* __restrict__ V, const T (&v0)[K],
+                                             const T (&v1)[K], int w, unsigned row_bytes,
+                                             const unsigned (&qoff)[K], int nt) {
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-        const int q = q0 + nt * k;
-        if (FULL || q <= w) V[q + 1] = val[k];
-        if (FULL ? (k == K - 1 && q0 == nt) : (q == w)) V[w + 2] = val[k];
+        const RowPair<T> pr{v0[k], v1[k]};
+        if (FULL || qoff[k] <= row_bytes) *at_bytes(V + 1, 2 * qoff[k]) = pr;
+        if (FULL ? (k == K - 1 && static_cast<int>(threadIdx.x) == nt - 1) : (qoff[k] == row_bytes))
+            V[w + 2] = pr;
     }
-    if (q0 == 1) { V[0] = T(0); V[1] = T(0); }
+}
+template <class T>
+__device__ __forceinline__ void clear_row_pads(RowPair<T>* vbuf, int vlen) {
+    if (threadIdx.x < 4) vbuf[(threadIdx.x >> 1) * vlen + (threadIdx.x & 1)] = RowPair<T>{T(0), T(0)};
 }
 
-// LDS indices of the column pairs (lAdv, l) = (lo, lo+1) and (r, rAdv) = (hi, hi+1) of pixel j.
-template <int K>
-__device__ __forceinline__ void column_taps(int (&lo)[K], int (&hi)[K], int ylo, int yhi, int w,
-                                            int nt) {
+// LDS byte offsets of the column pairs (lAdv, l) = (lo, lo+1) and (r, rAdv) = (hi, hi+1) of the
+// lane's pixels.
+template <class T, int K>
+__device__ __forceinline__ void column_taps(unsigned (&lo)[K], unsigned (&hi)[K], int ylo, int yhi,
+                                            int w, int nt) {
 #pragma unroll
     for (int k = 0; k < K; ++k) {
         const int j = static_cast<int>(threadIdx.x) + nt * k;
-        lo[k] = clampi(j + ylo, 0, w + 1);
-        hi[k] = clampi(j + yhi, -1, w) + 1;
+        lo[k] = static_cast<unsigned>(clampi(j + ylo, 0, w + 1)) * static_cast<unsigned>(sizeof(RowPair<T>));
+        hi[k] = static_cast<unsigned>(clampi(j + yhi, -1, w) + 1) * static_cast<unsigned>(sizeof(RowPair<T>));
     }
+}
+
+// Box sums of one pixel column slot for both rows of the pair.
+template <class T, bool EXACT>
+__device__ __forceinline__ RowPair<T> sample_columns(const RowPair<T>* __restrict__ V, unsigned lo,
+                                                     unsigned hi, T fylo, T fyhi) {
+    const RowPair<T>* L = at_bytes(V, lo);
+    const RowPair<T>* H = at_bytes(V, hi);
+    const RowPair<T> l = L[1], r = H[0];
+    RowPair<T> la = l, ra = r;
+    if (EXACT) { la = L[0]; ra = H[1]; }
+    return {blend<T, EXACT>(la.r0, l.r0, r.r0, ra.r0, fylo, fyhi),
+            blend<T, EXACT>(la.r1, l.r1, r.r1, ra.r1, fylo, fyhi)};
 }
 
 template <class T>
@@ -146,9 +186,12 @@ __device__ __forceinline__ BoxOfWorkgroup<T> load_box(const BoxParams<T>& prm, i
     return {prm.xmin[k_par], prm.xmax[k_par], prm.ymin[k_par], prm.ymax[k_par]};
 }
 
+using Flip0 = std::integral_constant<int, 0>;
+using Flip1 = std::integral_constant<int, 1>;
+
 // ---------------------------------------------------------------------------------------------
 // Forward. Work item = (plane p, filter f, band). blockDim = nt, K >= ceil(w / nt).
-// LDS: [2 buffers][2 rows][w+3] T.
+// LDS: [2 buffers][w+3] RowPair<T>.
 template <class T, int K, bool EXACT, bool FULL>
 __global__ void __launch_bounds__(kMaxRowThreads) forward_rows_kernel(SampleArgs<T> a) {
     const int64_t vid = xcd_contiguous_id(a.per_xcd);
@@ -158,7 +201,8 @@ __global__ void __launch_bounds__(kMaxRowThreads) forward_rows_kernel(SampleArgs
     const int f = static_cast<int>(pf % a.F);
     const int64_t p = pf / a.F;
     const int k_par = static_cast<int>((a.plane0 + p) % a.C) * a.F + f;
-    const int h = a.h, w = a.w, nt = blockDim.x, q0 = 1 + threadIdx.x;
+    const int h = a.h, w = a.w, nt = blockDim.x;
+    const unsigned row_bytes = static_cast<unsigned>(w) * sizeof(T);
 
     const BoxOfWorkgroup<T> bx = load_box(a.prm, k_par);
     const BoxSplit<T> s = split_forward(bx.xmin, bx.xmax, bx.ymin, bx.ymax);
@@ -168,58 +212,53 @@ __global__ void __launch_bounds__(kMaxRowThreads) forward_rows_kernel(SampleArgs
     const int64_t pitch = w + 1;
     const T* plane = a.src + p * static_cast<int64_t>(h + 1) * pitch;
     T* out = a.dst + pf * static_cast<int64_t>(h) * w;
-    T* vbuf = reinterpret_cast<T*>(smem_raw);
+    RowPair<T>* vbuf = reinterpret_cast<RowPair<T>*>(smem_raw);
     const int vlen = w + 3;
+    clear_row_pads(vbuf, vlen);
 
     const int i0 = band * a.R;
     const int i1 = min(h, i0 + a.R);
 
-    int lo[K], hi[K];
-    column_taps<K>(lo, hi, s.ylo, s.yhi, w, nt);
+    unsigned qoff[K], lo[K], hi[K];
+    lane_columns<T, K>(qoff, nt);
+    column_taps<T, K>(lo, hi, s.ylo, s.yhi, w, nt);
 
     T ta[K], bc[K];                       // I[t(i-1)], I[b(i)]
     T t0[K], t1[K], b1[K], b2[K];         // I[t(i)], I[t(i+1)], I[b(i+1)], I[b(i+2)]
-    load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), w, q0, nt, ta);
-    load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xhi, 0, h), w, q0, nt, bc);
-    load_pair<T, K, FULL>(plane, pitch, i0, s.xlo, s.xhi, h, w, q0, nt, t0, t1, b1, b2);
+    load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), row_bytes, qoff, ta);
+    load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xhi, 0, h), row_bytes, qoff, bc);
+    load_pair<T, K, FULL>(plane, pitch, i0, s.xlo, s.xhi, h, row_bytes, qoff, t0, t1, b1, b2);
 
-    // One row pair. PREFETCH is a compile-time tag: the loop body always issues the next pair's
-    // loads and the last pair is peeled, so no branch joins a path with loads in flight to one
-    // without (the wait-count insertion would have to drain the prefetch at such a join).
-    int flip = 0;
-    auto row_pair = [&](int i, auto prefetch_tag) {
+    // One row pair. PREFETCH and the LDS buffer are compile-time tags: the loop body always
+    // issues the next pair's loads and the last pair is peeled, so no branch joins a path with
+    // loads in flight to one without (the wait-count insertion would have to drain the prefetch
+    // at such a join); the loop is unrolled over both buffers so that LDS addresses are lane
+    // constants plus immediates and the sliding rows rotate by renaming instead of moves.
+    auto row_pair = [&](int i, auto prefetch_tag, auto flip_tag) {
         constexpr bool PREFETCH = decltype(prefetch_tag)::value;
+        constexpr int FLIP = decltype(flip_tag)::value;
         T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {};
         if (PREFETCH)
-            load_pair<T, K, FULL>(plane, pitch, i + 2, s.xlo, s.xhi, h, w, q0, nt, n0, n1, n2, n3);
+            load_pair<T, K, FULL>(plane, pitch, i + 2, s.xlo, s.xhi, h, row_bytes, qoff, n0, n1, n2, n3);
 
-        T* V0 = vbuf + flip * 2 * vlen;
-        T* V1 = V0 + vlen;
-        flip ^= 1;
+        RowPair<T>* V = vbuf + (FLIP ? vlen : 0);
         T v0[K], v1[K];
 #pragma unroll
         for (int k = 0; k < K; ++k) {
             v0[k] = blend<T, EXACT>(ta[k], t0[k], bc[k], b1[k], s.fxlo, s.fxhi);
             v1[k] = blend<T, EXACT>(t0[k], t1[k], b1[k], b2[k], s.fxlo, s.fxhi);
         }
-        publish_row<T, K, FULL>(V0, v0, w, q0, nt);
-        publish_row<T, K, FULL>(V1, v1, w, q0, nt);
+        publish_rows<T, K, FULL>(V, v0, v1, w, row_bytes, qoff, nt);
         __syncthreads();
 
-        T* orow = out + static_cast<int64_t>(i) * w;
+        T* orow = out + static_cast<int64_t>(i) * w - 1;     // column q = j + 1 lands on pixel j
         const bool second = i + 1 < i1;
 #pragma unroll
         for (int k = 0; k < K; ++k) {
-            const int j = static_cast<int>(threadIdx.x) + nt * k;
-            if (FULL || j < w) {
-                const T o0 = blend<T, EXACT>(V0[lo[k]], V0[lo[k] + 1], V0[hi[k]], V0[hi[k] + 1],
-                                             s.fylo, s.fyhi);
-                __builtin_nontemporal_store(o0 * scale, orow + static_cast<unsigned>(j));
-                if (second) {
-                    const T o1 = blend<T, EXACT>(V1[lo[k]], V1[lo[k] + 1], V1[hi[k]],
-                                                 V1[hi[k] + 1], s.fylo, s.fyhi);
-                    __builtin_nontemporal_store(o1 * scale, orow + static_cast<unsigned>(w + j));
-                }
+            if (FULL || qoff[k] <= row_bytes) {
+                const RowPair<T> o = sample_columns<T, EXACT>(V, lo[k], hi[k], s.fylo, s.fyhi);
+                __builtin_nontemporal_store(o.r0 * scale, at_bytes(orow, qoff[k]));
+                if (second) __builtin_nontemporal_store(o.r1 * scale, at_bytes(orow + w, qoff[k]));
             }
         }
         if (PREFETCH) {
@@ -231,8 +270,16 @@ __global__ void __launch_bounds__(kMaxRowThreads) forward_rows_kernel(SampleArgs
         }
     };
     int i = i0;
-    for (; i + 2 < i1; i += 2) row_pair(i, std::true_type{});
-    row_pair(i, std::false_type{});
+    for (; i + 4 < i1; i += 4) {
+        row_pair(i, std::true_type{}, Flip0{});
+        row_pair(i + 2, std::true_type{}, Flip1{});
+    }
+    if (i + 2 < i1) {
+        row_pair(i, std::true_type{}, Flip0{});
+        row_pair(i + 2, std::false_type{}, Flip1{});
+    } else {
+        row_pair(i, std::false_type{}, Flip0{});
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -245,18 +292,23 @@ __global__ void __launch_bounds__(kMaxRowThreads) forward_rows_kernel(SampleArgs
 // it is ever added.
 template <class T, int K, int RB, bool EXACT, bool FULL, bool OFFS>
 __global__ void __launch_bounds__(kMaxRowThreads, BOXCONV_GI_WAVES) grad_input_rows_kernel(SampleArgs<T> a) {
-    static_assert(RB % 2 == 0, "rows are handled in pairs");
+    static_assert(RB % 4 == 0, "rows are handled in pairs, and pairs alternate between two LDS buffers");
     const int64_t vid = xcd_contiguous_id(a.per_xcd);
     if (vid >= a.total) return;
     const int band = static_cast<int>(vid % a.nb);
     const int64_t p = vid / a.nb;
     const int c_in = static_cast<int>((a.plane0 + p) % a.C);
-    const int h = a.h, w = a.w, nt = blockDim.x, q0 = 1 + threadIdx.x;
+    const int h = a.h, w = a.w, nt = blockDim.x;
+    const unsigned row_bytes = static_cast<unsigned>(w) * sizeof(T);
     const int64_t pitch = w + 1;
     const int64_t ipl = static_cast<int64_t>(h + 1) * pitch;
-    T* vbuf = reinterpret_cast<T*>(smem_raw);
+    RowPair<T>* vbuf = reinterpret_cast<RowPair<T>*>(smem_raw);
     const int vlen = w + 3;
+    clear_row_pads(vbuf, vlen);
     const int i0 = band * RB;
+
+    unsigned qoff[K];
+    lane_columns<T, K>(qoff, nt);
 
     T acc[RB][K];
 #pragma unroll
@@ -264,7 +316,6 @@ __global__ void __launch_bounds__(kMaxRowThreads, BOXCONV_GI_WAVES) grad_input_r
 #pragma unroll
         for (int k = 0; k < K; ++k) acc[r][k] = T(0);
 
-    int flip = 0;
     for (int f = 0; f < a.F; ++f) {
         const BoxOfWorkgroup<T> bx = load_box(a.prm, c_in * a.F + f);
         const BoxSplit<T> s = split_grad_input(bx.xmin, bx.xmax, bx.ymin, bx.ymax);
@@ -272,8 +323,8 @@ __global__ void __launch_bounds__(kMaxRowThreads, BOXCONV_GI_WAVES) grad_input_r
             ? inverse_extent(bx.xmin, bx.xmax, bx.ymin, bx.ymax, EXACT, true, true) : T(1);
         const T* plane = a.src + (p * a.F + f) * ipl;
 
-        int lo[K], hi[K];
-        column_taps<K>(lo, hi, s.ylo, s.yhi, w, nt);
+        unsigned lo[K], hi[K];
+        column_taps<T, K>(lo, hi, s.ylo, s.yhi, w, nt);
 
         // OFFS: `plane` holds a band-local integral (bands of off_R rows, each restarting at
         // zero). Integral row r (1..h) belongs to band (r-1)/off_R; row 0 counts as band 0. The
@@ -287,32 +338,32 @@ __global__ void __launch_bounds__(kMaxRowThreads, BOXCONV_GI_WAVES) grad_input_r
         T off_t[K], off_b[K];
 #pragma unroll
         for (int k = 0; k < K; ++k) { off_t[k] = T(0); off_b[k] = T(0); }
+        auto refresh = [&](int& cached_band, int& cached_last, int row_index, T (&cached)[K]) {
+            do { ++cached_band; cached_last += a.off_R; } while (row_index > cached_last);
+            double sum[K];
+#pragma unroll
+            for (int k = 0; k < K; ++k) sum[k] = 0.0;
+            for (int b = ref_band; b < cached_band; ++b) {
+                T bottom[K];
+                load_row<T, K, FULL>(plane, pitch, min(h, (b + 1) * a.off_R), row_bytes, qoff, bottom);
+#pragma unroll
+                for (int k = 0; k < K; ++k) sum[k] += static_cast<double>(bottom[k]);
+            }
+#pragma unroll
+            for (int k = 0; k < K; ++k) cached[k] = static_cast<T>(sum[k]);
+        };
         auto correct = [&](T (&row)[K], int row_index, int& cached_band, int& cached_last, T (&cached)[K]) {
             if (!OFFS) return;
-            if (row_index > cached_last) {                  // uniform: depends on the row only
-                do { ++cached_band; cached_last += a.off_R; } while (row_index > cached_last);
-                double sum[K];
-#pragma unroll
-                for (int k = 0; k < K; ++k) sum[k] = 0.0;
-                for (int b = ref_band; b < cached_band; ++b) {
-                    const T* bottom = plane + static_cast<int64_t>(min(h, (b + 1) * a.off_R)) * pitch;
-#pragma unroll
-                    for (int k = 0; k < K; ++k) {
-                        const int q = q0 + nt * k;
-                        if (FULL || q <= w) sum[k] += static_cast<double>(bottom[static_cast<unsigned>(q)]);
-                    }
-                }
-#pragma unroll
-                for (int k = 0; k < K; ++k) cached[k] = static_cast<T>(sum[k]);
-            }
+            if (row_index > cached_last)                    // uniform: depends on the row only
+                refresh(cached_band, cached_last, row_index, cached);
 #pragma unroll
             for (int k = 0; k < K; ++k) row[k] += cached[k];
         };
 
         T ta[K], bc[K], t0[K], t1[K], b1[K], b2[K];
-        load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), w, q0, nt, ta);
-        load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xhi, 0, h), w, q0, nt, bc);
-        load_pair<T, K, FULL>(plane, pitch, i0, s.xlo, s.xhi, h, w, q0, nt, t0, t1, b1, b2);
+        load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), row_bytes, qoff, ta);
+        load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xhi, 0, h), row_bytes, qoff, bc);
+        load_pair<T, K, FULL>(plane, pitch, i0, s.xlo, s.xhi, h, row_bytes, qoff, t0, t1, b1, b2);
         correct(ta, clampi(i0 + s.xlo - 1, 0, h), band_t, last_t, off_t);
         correct(t0, clampi(i0 + s.xlo, 0, h), band_t, last_t, off_t);
         correct(t1, clampi(i0 + 1 + s.xlo, 0, h), band_t, last_t, off_t);
@@ -326,67 +377,49 @@ __global__ void __launch_bounds__(kMaxRowThreads, BOXCONV_GI_WAVES) grad_input_r
 #pragma unroll
         for (int r = 0; r < RB; r += 2) {
             const int i = i0 + r;
-            {
-                T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {};
-                const bool more = kGradInputPrefetch && (r + 2 < RB);   // known after unrolling
-                if (more)
-                    load_pair<T, K, FULL>(plane, pitch, i + 2, s.xlo, s.xhi, h, w, q0, nt, n0, n1, n2, n3);
-                if (!kGradInputPrefetch && r > 0) {
-                    load_pair<T, K, FULL>(plane, pitch, i, s.xlo, s.xhi, h, w, q0, nt, t0, t1, b1, b2);
-                    if (OFFS) {
-                        correct(t0, clampi(i + s.xlo, 0, h), band_t, last_t, off_t);
-                        correct(t1, clampi(i + 1 + s.xlo, 0, h), band_t, last_t, off_t);
-                        correct(b1, clampi(i + 1 + s.xhi, 0, h), band_b, last_b, off_b);
-                        correct(b2, clampi(i + 2 + s.xhi, 0, h), band_b, last_b, off_b);
-                    }
-                }
-                T* V0 = vbuf + flip * 2 * vlen;
-                T* V1 = V0 + vlen;
-                flip ^= 1;
-                T v0[K], v1[K];
+            T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {};
+            const bool more = r + 2 < RB;                                // known after unrolling
+            if (more)
+                load_pair<T, K, FULL>(plane, pitch, i + 2, s.xlo, s.xhi, h, row_bytes, qoff, n0, n1, n2, n3);
+            RowPair<T>* V = vbuf + (((r >> 1) & 1) ? vlen : 0);
+            T v0[K], v1[K];
 #pragma unroll
-                for (int k = 0; k < K; ++k) {
-                    v0[k] = blend<T, EXACT>(ta[k], t0[k], bc[k], b1[k], s.fxlo, s.fxhi);
-                    v1[k] = blend<T, EXACT>(t0[k], t1[k], b1[k], b2[k], s.fxlo, s.fxhi);
-                }
-                publish_row<T, K, FULL>(V0, v0, w, q0, nt);
-                publish_row<T, K, FULL>(V1, v1, w, q0, nt);
-                __syncthreads();
+            for (int k = 0; k < K; ++k) {
+                v0[k] = blend<T, EXACT>(ta[k], t0[k], bc[k], b1[k], s.fxlo, s.fxhi);
+                v1[k] = blend<T, EXACT>(t0[k], t1[k], b1[k], b2[k], s.fxlo, s.fxhi);
+            }
+            publish_rows<T, K, FULL>(V, v0, v1, w, row_bytes, qoff, nt);
+            __syncthreads();
 #pragma unroll
-                for (int k = 0; k < K; ++k) {
-                    const int j = static_cast<int>(threadIdx.x) + nt * k;
-                    if (FULL || j < w) {
-                        acc[r][k] += scale * blend<T, EXACT>(V0[lo[k]], V0[lo[k] + 1], V0[hi[k]],
-                                                             V0[hi[k] + 1], s.fylo, s.fyhi);
-                        acc[r + 1][k] += scale * blend<T, EXACT>(V1[lo[k]], V1[lo[k] + 1], V1[hi[k]],
-                                                                 V1[hi[k] + 1], s.fylo, s.fyhi);
-                    }
+            for (int k = 0; k < K; ++k) {
+                if (FULL || qoff[k] <= row_bytes) {
+                    const RowPair<T> o = sample_columns<T, EXACT>(V, lo[k], hi[k], s.fylo, s.fyhi);
+                    acc[r][k] += scale * o.r0;
+                    acc[r + 1][k] += scale * o.r1;
                 }
+            }
+            if (more) {
 #pragma unroll
                 for (int k = 0; k < K; ++k) {
                     ta[k] = t1[k]; bc[k] = b2[k];
-                    if (more) { t0[k] = n0[k]; t1[k] = n1[k]; b1[k] = n2[k]; b2[k] = n3[k]; }
+                    t0[k] = n0[k]; t1[k] = n1[k]; b1[k] = n2[k]; b2[k] = n3[k];
                 }
-                if (OFFS && more) {
-                    correct(t0, clampi(i + 2 + s.xlo, 0, h), band_t, last_t, off_t);
-                    correct(t1, clampi(i + 3 + s.xlo, 0, h), band_t, last_t, off_t);
-                    correct(b1, clampi(i + 3 + s.xhi, 0, h), band_b, last_b, off_b);
-                    correct(b2, clampi(i + 4 + s.xhi, 0, h), band_b, last_b, off_b);
-                }
+                correct(t0, clampi(i + 2 + s.xlo, 0, h), band_t, last_t, off_t);
+                correct(t1, clampi(i + 3 + s.xlo, 0, h), band_t, last_t, off_t);
+                correct(b1, clampi(i + 3 + s.xhi, 0, h), band_b, last_b, off_b);
+                correct(b2, clampi(i + 4 + s.xhi, 0, h), band_b, last_b, off_b);
             }
         }
     }
 
-    T* out = a.dst + p * static_cast<int64_t>(h) * w;
+    T* out = a.dst + p * static_cast<int64_t>(h) * w - 1;    // column q = j + 1 lands on pixel j
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
         const int i = i0 + r;
         if (i < h) {
 #pragma unroll
-            for (int k = 0; k < K; ++k) {
-                const int j = static_cast<int>(threadIdx.x) + nt * k;
-                if (FULL || j < w) (out + static_cast<int64_t>(i) * w)[static_cast<unsigned>(j)] = acc[r][k];
-            }
+            for (int k = 0; k < K; ++k)
+                if (FULL || qoff[k] <= row_bytes) *at_bytes(out + static_cast<int64_t>(i) * w, qoff[k]) = acc[r][k];
         }
     }
 }
@@ -430,21 +463,21 @@ __device__ __forceinline__ void block_accumulate5(const double (&v)[5], double* 
 // (SCAN) the BAND-LOCAL integral image of grad_output: L[i+1][c+1] = sum of grad_output over rows
 // band_start..i and columns 0..c. Bands do not depend on each other, so nothing has to be known
 // about the rows above: the true integral is L plus the bottom rows of the bands above, which
-// the grad-input kernel adds when it loads a row. Column accumulators and the row prefix are
-// carried in double; lanes own K consecutive columns for this part (read back from the LDS row),
-// results go through an LDS stage so that global stores are lane-consecutive dwords.
+// the grad-input kernel adds when it loads a row. Lanes own K consecutive columns for this part
+// (read back from the LDS row), results go through an LDS stage so that global stores are
+// lane-consecutive dwords.
 //
-// LDS: [2 buffers][2 rows][K*nt + 8] grad_output rows (4 zeros in front, >= 4 behind),
-//      [2][2][4] X[w] triples, [2][K*nt] stage, [2][8] doubles wave totals, [8*5] doubles.
+// LDS: [2 buffers][K*nt + 8] RowPair grad_output rows (4 zero pairs in front, >= 4 behind),
+//      [2][2][4] X[w] triples, [K*nt] RowPair stage, [8*5] doubles, [2][8] wave totals.
 constexpr int kGPad = 4;
 
 template <class T>
 struct StreamLds {
-    T* grow;          // [2][2][glen]
-    T* xw;            // [2][2][4]
-    T* stage;         // [2][K*nt]
-    double* wave_tot; // [2][kMaxRowWaves]
-    double* red;      // [5 * kMaxRowWaves]
+    RowPair<T>* grow;   // [2][glen]
+    T* xw;              // [2][2][4]
+    RowPair<T>* stage;  // [K*nt]
+    double* red;        // [5 * kMaxRowWaves]
+    T* wave_tot;        // [2][kMaxRowWaves]
     int glen;
 };
 
@@ -459,13 +492,13 @@ template <class T>
 __device__ __forceinline__ StreamLds<T> carve_stream_lds(int K, int nt) {
     StreamLds<T> l;
     l.glen = K * nt + 8;
-    l.grow = reinterpret_cast<T*>(smem_raw);
-    l.xw = l.grow + 4 * l.glen;
-    l.stage = l.xw + 16;
+    l.grow = reinterpret_cast<RowPair<T>*>(smem_raw);
+    l.xw = reinterpret_cast<T*>(l.grow + 2 * l.glen);
+    l.stage = reinterpret_cast<RowPair<T>*>(l.xw + 16);
     size_t b = (4 * static_cast<size_t>(l.glen) + 16 + 2 * static_cast<size_t>(K) * nt) * sizeof(T);
     b = (b + 15) / 16 * 16;
-    l.wave_tot = reinterpret_cast<double*>(smem_raw + b);
-    l.red = l.wave_tot + 2 * kMaxRowWaves;
+    l.red = reinterpret_cast<double*>(smem_raw + b);
+    l.wave_tot = reinterpret_cast<T*>(l.red + 5 * kMaxRowWaves);
     return l;
 }
 
@@ -478,7 +511,8 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
     const int f = static_cast<int>(pf % a.F);
     const int64_t p = pf / a.F;
     const int k_par = static_cast<int>((a.plane0 + p) % a.C) * a.F + f;
-    const int h = a.h, w = a.w, nt = blockDim.x, tid = threadIdx.x, q0 = 1 + tid;
+    const int h = a.h, w = a.w, nt = blockDim.x, tid = threadIdx.x;
+    const unsigned row_bytes = static_cast<unsigned>(w) * sizeof(T);
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keep it scalar
 
@@ -496,22 +530,25 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
     const int i1 = min(h, i0 + a.R);
 
     // clear the grad_output rows once: pads and the columns beyond w stay zero for good
-    for (int e = tid; e < 4 * glen; e += nt) lds.grow[e] = T(0);
+    for (int e = tid; e < 2 * glen; e += nt) lds.grow[e] = RowPair<T>{T(0), T(0)};
     if (SCAN && band == 0)
         for (int c = tid; c <= w; c += nt) lrows[c] = T(0);                    // integral row 0
     __syncthreads();
 
-    // lane-constant LDS indices of the pairs (grA, gr) and (gl, glA), and the tail weights
-    int ir[K], il[K];
+    unsigned qoff[K];
+    lane_columns<T, K>(qoff, nt);
+
+    // lane-constant LDS byte offsets of the pairs (grA, gr) and (gl, glA), and the tail weights
+    unsigned ir[K], il[K];
     T delta[K];
-    int idx_ymax = 0, idx_ymin = 0;
+    unsigned idx_ymax = 0, idx_ymin = 0;
     if (PARAMS) {
 #pragma unroll
         for (int k = 0; k < K; ++k) {
             const int j = tid + nt * k;
             const int q = j + 1;
-            ir[k] = clampi(q - s.yhi - 1, -2, w) + kGPad;
-            il[k] = clampi(q - s.ylo, -2, w) + kGPad;
+            ir[k] = static_cast<unsigned>(clampi(q - s.yhi - 1, -2, w) + kGPad) * static_cast<unsigned>(sizeof(RowPair<T>));
+            il[k] = static_cast<unsigned>(clampi(q - s.ylo, -2, w) + kGPad) * static_cast<unsigned>(sizeof(RowPair<T>));
             T d = T(0);
             if (FULL || j < w) {
                 const T one = T(1);
@@ -528,55 +565,49 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
     }
 
     T sum[5] = {T(0), T(0), T(0), T(0), T(0)};
-    double colacc[K];                                 // SCAN: columns K*tid .. K*tid+K-1
+    T colacc[K];                                      // SCAN: columns K*tid .. K*tid+K-1
 #pragma unroll
-    for (int k = 0; k < K; ++k) colacc[k] = 0.0;
+    for (int k = 0; k < K; ++k) colacc[k] = T(0);
 
     T ta[K], bc[K], t0[K], t1[K], b1[K], b2[K], g0[K], g1[K];
     if (PARAMS) {
-        load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), w, q0, nt, ta);
-        load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xhi, 0, h), w, q0, nt, bc);
-        load_pair<T, K, FULL>(plane, pitch, i0, s.xlo, s.xhi, h, w, q0, nt, t0, t1, b1, b2);
+        load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), row_bytes, qoff, ta);
+        load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xhi, 0, h), row_bytes, qoff, bc);
+        load_pair<T, K, FULL>(plane, pitch, i0, s.xlo, s.xhi, h, row_bytes, qoff, t0, t1, b1, b2);
     }
     auto load_g = [&](int i, T (&dst)[K]) {
-        const T* grow = gout + static_cast<int64_t>(min(i, h - 1)) * w;
+        const T* grow = gout + static_cast<int64_t>(min(i, h - 1)) * w - 1;   // column q = j + 1 -> pixel j
         const bool valid = i < i1;
 #pragma unroll
-        for (int k = 0; k < K; ++k) {
-            const int j = tid + nt * k;
-            dst[k] = (valid && (FULL || j < w)) ? __builtin_nontemporal_load(grow + static_cast<unsigned>(j)) : T(0);
-        }
+        for (int k = 0; k < K; ++k)
+            dst[k] = (valid && (FULL || qoff[k] <= row_bytes))
+                         ? __builtin_nontemporal_load(at_bytes(grow, qoff[k])) : T(0);
     };
     load_g(i0, g0);
     load_g(i0 + 1, g1);
 
-    int flip = 0;
-    auto row_pair = [&](int i, auto prefetch_tag) {
+    auto row_pair = [&](int i, auto prefetch_tag, auto flip_tag) {
         constexpr bool PREFETCH = decltype(prefetch_tag)::value;   // see forward_rows_kernel
+        constexpr int FLIP = decltype(flip_tag)::value;
         T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {}, m0[K] = {}, m1[K] = {};
         if (PREFETCH) {
             if (PARAMS)
-                load_pair<T, K, FULL>(plane, pitch, i + 2, s.xlo, s.xhi, h, w, q0, nt, n0, n1, n2, n3);
+                load_pair<T, K, FULL>(plane, pitch, i + 2, s.xlo, s.xhi, h, row_bytes, qoff, n0, n1, n2, n3);
             load_g(i + 2, m0);
             load_g(i + 3, m1);
         }
 
-        T* G0 = lds.grow + flip * 2 * glen;
-        T* G1 = G0 + glen;
-        T* X0 = lds.xw + flip * 8;
+        RowPair<T>* G = lds.grow + (FLIP ? glen : 0);
+        T* X0 = lds.xw + FLIP * 8;
         T* X1 = X0 + 4;
-        flip ^= 1;
 
         T tail0 = T(0), tail1 = T(0);
 #pragma unroll
         for (int k = 0; k < K; ++k) {
-            const int j = tid + nt * k;
-            if (FULL || j < w) {
-                G0[j + kGPad] = g0[k];
-                G1[j + kGPad] = g1[k];
-            }
+            if (FULL || qoff[k] <= row_bytes)
+                *at_bytes(G + kGPad - 1, 2 * qoff[k]) = RowPair<T>{g0[k], g1[k]};
             if (PARAMS) { tail0 += delta[k] * g0[k]; tail1 += delta[k] * g1[k]; }
-            if (PARAMS && (FULL ? (k == K - 1 && tid == nt - 1) : (j == w - 1))) {   // owner of column q = w
+            if (PARAMS && (FULL ? (k == K - 1 && tid == nt - 1) : (qoff[k] == row_bytes))) {   // owner of column q = w
                 const T dt0 = t0[k] - ta[k], db0 = b1[k] - bc[k];
                 const T dt1 = t1[k] - t0[k], db1 = b2[k] - b1[k];
                 T v0 = bc[k] - t0[k], v1 = b1[k] - t1[k];
@@ -600,10 +631,12 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
                     v0 += s.fxhi * db0 + s.fxlo * dt0;
                     v1 += s.fxhi * db1 + s.fxlo * dt1;
                 }
+                const RowPair<T>* R = at_bytes(G, ir[k]);
+                const RowPair<T>* L = at_bytes(G, il[k]);
+                const RowPair<T> grA = R[0], gr = R[1], gl = L[0], glA = L[1];
                 {
-                    const T grA = G0[ir[k]], gr = G0[ir[k] + 1], gl = G0[il[k]], glA = G0[il[k] + 1];
-                    const T dr = grA - gr, dl = gl - glA;
-                    T wq = gr - gl;
+                    const T dr = grA.r0 - gr.r0, dl = gl.r0 - glA.r0;
+                    T wq = gr.r0 - gl.r0;
                     if (EXACT) wq += s.fyhi * dr + s.fylo * dl;
                     sum[4] += v0 * wq;
                     sum[1] += db0 * wq;
@@ -612,9 +645,8 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
                     sum[2] -= v0 * dl;
                 }
                 {
-                    const T grA = G1[ir[k]], gr = G1[ir[k] + 1], gl = G1[il[k]], glA = G1[il[k] + 1];
-                    const T dr = grA - gr, dl = gl - glA;
-                    T wq = gr - gl;
+                    const T dr = grA.r1 - gr.r1, dl = gl.r1 - glA.r1;
+                    T wq = gr.r1 - gl.r1;
                     if (EXACT) wq += s.fyhi * dr + s.fylo * dl;
                     sum[4] += v1 * wq;
                     sum[1] += db1 * wq;
@@ -629,32 +661,33 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
             sum[1] += dbw0 * tail0 + dbw1 * tail1;
             sum[0] -= dtw0 * tail0 + dtw1 * tail1;
             if (tid == 0) {
-                sum[3] += vw0 * G0[idx_ymax] + vw1 * G1[idx_ymax];
-                sum[2] -= vw0 * G0[idx_ymin] + vw1 * G1[idx_ymin];
+                const RowPair<T> gmax = G[idx_ymax], gmin = G[idx_ymin];
+                sum[3] += vw0 * gmax.r0 + vw1 * gmax.r1;
+                sum[2] -= vw0 * gmin.r0 + vw1 * gmin.r1;
             }
         }
 
         if (SCAN) {
-            // lane owns columns K*tid .. K*tid+K-1; two rows of the band-local integral.
-            // loc*: prefix inside the lane (small numbers, kept in T); carry*: everything to
-            // the left of the lane (double).
+            // lane owns columns K*tid .. K*tid+K-1; two rows of the band-local integral. A band
+            // restarts at zero and the row prefix is a tree (inside the lane, across the wave,
+            // across waves), so plain T arithmetic loses a few ulps of the band-local value only.
             T loc0[K], loc1[K];
-            double carry0, carry1;
+            T carry0, carry1;
             {
-                const T* r0 = G0 + kGPad + K * tid;
-                const T* r1 = G1 + kGPad + K * tid;
-                double run0 = 0.0, run1 = 0.0;
+                const RowPair<T>* r = G + kGPad + K * tid;
+                T run0 = T(0), run1 = T(0);
 #pragma unroll
                 for (int k = 0; k < K; ++k) {
-                    colacc[k] += static_cast<double>(r0[k]);
+                    const RowPair<T> g = r[k];
+                    colacc[k] += g.r0;
                     run0 += colacc[k];
-                    loc0[k] = static_cast<T>(run0);
-                    colacc[k] += static_cast<double>(r1[k]);
+                    loc0[k] = run0;
+                    colacc[k] += g.r1;
                     run1 += colacc[k];
-                    loc1[k] = static_cast<T>(run1);
+                    loc1[k] = run1;
                 }
-                const double inc0 = wave_inclusive_scan(run0);
-                const double inc1 = wave_inclusive_scan(run1);
+                const T inc0 = wave_inclusive_scan(run0);
+                const T inc1 = wave_inclusive_scan(run1);
                 carry0 = inc0 - run0;
                 carry1 = inc1 - run1;
                 if (lane == 63) { lds.wave_tot[wave] = inc0; lds.wave_tot[kMaxRowWaves + wave] = inc1; }
@@ -667,13 +700,9 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
                         carry0 += lds.wave_tot[wv];
                         carry1 += lds.wave_tot[kMaxRowWaves + wv];
                     }
-                T* s0 = lds.stage + K * tid;
-                T* s1 = lds.stage + K * nt + K * tid;
+                RowPair<T>* st = lds.stage + K * tid;
 #pragma unroll
-                for (int k = 0; k < K; ++k) {
-                    s0[k] = static_cast<T>(carry0 + static_cast<double>(loc0[k]));
-                    s1[k] = static_cast<T>(carry1 + static_cast<double>(loc1[k]));
-                }
+                for (int k = 0; k < K; ++k) st[k] = RowPair<T>{carry0 + loc0[k], carry1 + loc1[k]};
             }
             __syncthreads();                                                 // stage visible
             {
@@ -682,10 +711,10 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
                 const bool second = i + 1 < i1;
 #pragma unroll
                 for (int k = 0; k < K; ++k) {
-                    const int j = tid + nt * k;
-                    if (FULL || j < w) {
-                        __builtin_nontemporal_store(lds.stage[j], o0 + static_cast<unsigned>(j + 1));
-                        if (second) __builtin_nontemporal_store(lds.stage[K * nt + j], o1 + static_cast<unsigned>(j + 1));
+                    if (FULL || qoff[k] <= row_bytes) {
+                        const RowPair<T> v = *at_bytes(lds.stage - 1, 2 * qoff[k]);   // column j = q - 1
+                        __builtin_nontemporal_store(v.r0, at_bytes(o0, qoff[k]));
+                        if (second) __builtin_nontemporal_store(v.r1, at_bytes(o1, qoff[k]));
                     }
                 }
                 if (tid == 0) {
@@ -707,8 +736,16 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
         }
     };
     int i = i0;
-    for (; i + 2 < i1; i += 2) row_pair(i, std::true_type{});
-    row_pair(i, std::false_type{});
+    for (; i + 4 < i1; i += 4) {
+        row_pair(i, std::true_type{}, Flip0{});
+        row_pair(i + 2, std::true_type{}, Flip1{});
+    }
+    if (i + 2 < i1) {
+        row_pair(i, std::true_type{}, Flip0{});
+        row_pair(i + 2, std::false_type{}, Flip1{});
+    } else {
+        row_pair(i, std::false_type{}, Flip0{});
+    }
 
     if (PARAMS) {
         __syncthreads();

@@ -51,11 +51,8 @@ extern __shared__ __align__(16) unsigned char smem_raw[];
 // rather than more columns per lane: per-lane state (sliding rows, prefetched rows, accumulators)
 // scales with the columns per lane, and these kernels hide HBM latency with occupancy.
 constexpr int kMaxRowThreads = 512;
-#ifndef BOXCONV_GI_WAVES
-#define BOXCONV_GI_WAVES 1
-#endif
-#ifndef BOXCONV_GI_THREADS
-#define BOXCONV_GI_THREADS 256
+#ifndef BOXCONV_STREAM_UNROLL
+#define BOXCONV_STREAM_UNROLL 0
 #endif
 constexpr int kMaxRowWaves = kMaxRowThreads / 64;
 
@@ -90,38 +87,122 @@ __device__ __forceinline__ P* at_bytes(P* base, unsigned bytes) {
     return reinterpret_cast<P*>(reinterpret_cast<Byte*>(base) + bytes);
 }
 
-// Per-lane column slots. Lane `tid` owns integral columns q = 1 + tid + nt*k (pixel columns
-// j = q - 1), k < K. qoff[k] = q * sizeof(T) is the byte offset of column q in a row of T.
-// FULL: w == K * blockDim.x, so every (lane, k) slot is a valid column and no bounds checks are
-// compiled in; otherwise a slot is valid iff qoff[k] <= w * sizeof(T).
-template <class T, int K>
-__device__ __forceinline__ void lane_columns(unsigned (&qoff)[K], int nt) {
-#pragma unroll
-    for (int k = 0; k < K; ++k)
-        qoff[k] = static_cast<unsigned>(1 + static_cast<int>(threadIdx.x) + nt * k) *
-                  static_cast<unsigned>(sizeof(T));
+// One row of T in global memory addressed as a raw buffer: scalar descriptor (base, size in
+// bytes) plus one 32-bit VGPR byte offset per access, so no per-lane 64-bit address arithmetic.
+// The hardware checks the offset against the size: a load at or beyond `bytes` returns 0 and a
+// store there is dropped, which also masks column slots past the end of a row and whole rows
+// (bytes = 0) without branches. `row` must be wave-uniform.
+constexpr int kCacheDefault = 0, kCacheStream = 2;   // buffer cache policy bits: 2 = non-temporal
+template <class T>
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t row_buffer(const T* row, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(row), 0, static_cast<int>(bytes), 0x00020000);
+}
+template <int POLICY>
+__device__ __forceinline__ float buffer_load(__amdgpu_buffer_rsrc_t rs, unsigned off, float) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, off, 0, POLICY));
+}
+template <int POLICY>
+__device__ __forceinline__ double buffer_load(__amdgpu_buffer_rsrc_t rs, unsigned off, double) {
+    return __builtin_bit_cast(double, __builtin_amdgcn_raw_buffer_load_b64(rs, off, 0, POLICY));
+}
+template <int POLICY>
+__device__ __forceinline__ void buffer_store(float v, __amdgpu_buffer_rsrc_t rs, unsigned off) {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), rs, off, 0, POLICY);
+}
+template <int POLICY>
+__device__ __forceinline__ void buffer_store(double v, __amdgpu_buffer_rsrc_t rs, unsigned off) {
+    typedef unsigned v2u __attribute__((__vector_size__(8)));
+    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u, v), rs, off, 0, POLICY);
 }
 
-template <class T, int K, bool FULL>
-__device__ __forceinline__ void load_row(const T* __restrict__ plane, int64_t pitch, int row,
-                                         unsigned row_bytes, const unsigned (&qoff)[K], T (&dst)[K]) {
-    const T* r = plane + static_cast<int64_t>(row) * pitch;
+// K consecutive elements per lane. WHOLE: the run lies inside the buffer for every lane, so it
+// goes out as 16-byte pieces; otherwise element by element, each checked against the size.
+template <int POLICY, bool WHOLE, int K>
+__device__ __forceinline__ void buffer_store_run(const float (&v)[K], __amdgpu_buffer_rsrc_t rs, unsigned off) {
+    typedef unsigned v4u __attribute__((__vector_size__(16)));
+    if constexpr (WHOLE && K % 4 == 0) {
 #pragma unroll
-    for (int k = 0; k < K; ++k)
-        dst[k] = (FULL || qoff[k] <= row_bytes) ? *at_bytes(r, qoff[k]) : T(0);
+        for (int k = 0; k < K; k += 4) {
+            const v4u pack = {__builtin_bit_cast(unsigned, v[k]), __builtin_bit_cast(unsigned, v[k + 1]),
+                              __builtin_bit_cast(unsigned, v[k + 2]), __builtin_bit_cast(unsigned, v[k + 3])};
+            __builtin_amdgcn_raw_buffer_store_b128(pack, rs, off + 4u * k, 0, POLICY);
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < K; ++k) buffer_store<POLICY>(v[k], rs, off + 4u * k);
+    }
+}
+template <int POLICY, bool WHOLE, int K>
+__device__ __forceinline__ void buffer_store_run(const double (&v)[K], __amdgpu_buffer_rsrc_t rs, unsigned off) {
+#pragma unroll
+    for (int k = 0; k < K; ++k) buffer_store<POLICY>(v[k], rs, off + 8u * k);
+}
+
+// Per-lane column slots. Lane `tid` owns integral columns q = 1 + tid + NT*k (pixel columns
+// j = q - 1), k < K, NT = workgroup size. q1 = (1 + tid) * sizeof(T) is the byte offset of the
+// lane's first column in a row of T; the other slots are compile-time distances away, so one
+// register addresses all of them (instruction offsets for LDS, scalar offsets for buffers).
+// FULL: w == K * NT, so every (lane, k) slot is a valid column and no bounds checks are compiled
+// in; otherwise a slot is valid iff its byte offset is <= w * sizeof(T).
+template <class T>
+__device__ __forceinline__ unsigned lane_q1() {
+    return (1u + threadIdx.x) * static_cast<unsigned>(sizeof(T));
+}
+template <class T, int NT>
+__device__ __forceinline__ constexpr unsigned slot_bytes(int k) {
+    return static_cast<unsigned>(NT) * static_cast<unsigned>(k) * static_cast<unsigned>(sizeof(T));
+}
+template <class T, int NT, bool FULL>
+__device__ __forceinline__ bool slot_valid(unsigned q1, int k, unsigned row_bytes) {
+    return FULL || q1 + slot_bytes<T, NT>(k) <= row_bytes;
+}
+// Slot k of a row buffer. With FULL the slot distance rides in the scalar offset; otherwise it
+// is part of the checked per-lane offset, so slots past the end of the row read 0 / are dropped.
+template <class T, int NT, bool FULL, int POLICY>
+__device__ __forceinline__ T load_slot(__amdgpu_buffer_rsrc_t rs, unsigned q1, int k) {
+    if constexpr (FULL) {
+        if constexpr (sizeof(T) == 4)
+            return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b32(rs, q1, slot_bytes<T, NT>(k), POLICY));
+        else
+            return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b64(rs, q1, slot_bytes<T, NT>(k), POLICY));
+    } else {
+        return buffer_load<POLICY>(rs, q1 + slot_bytes<T, NT>(k), T());
+    }
+}
+template <class T, int NT, bool FULL, int POLICY>
+__device__ __forceinline__ void store_slot(T v, __amdgpu_buffer_rsrc_t rs, unsigned q1, int k) {
+    if constexpr (FULL) {
+        if constexpr (sizeof(T) == 4) {
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), rs, q1, slot_bytes<T, NT>(k), POLICY);
+        } else {
+            typedef unsigned v2u __attribute__((__vector_size__(8)));
+            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u, v), rs, q1, slot_bytes<T, NT>(k), POLICY);
+        }
+    } else {
+        buffer_store<POLICY>(v, rs, q1 + slot_bytes<T, NT>(k));
+    }
+}
+
+template <class T, int NT, int K, bool FULL>
+__device__ __forceinline__ void load_row(const T* __restrict__ plane, int64_t pitch, int row,
+                                         unsigned row_bytes, unsigned q1, T (&dst)[K]) {
+    // columns 0..w of the row; slots beyond w read 0
+    const __amdgpu_buffer_rsrc_t rs = row_buffer(plane + static_cast<int64_t>(row) * pitch,
+                                                 row_bytes + static_cast<unsigned>(sizeof(T)));
+#pragma unroll
+    for (int k = 0; k < K; ++k) dst[k] = load_slot<T, NT, FULL, kCacheDefault>(rs, q1, k);
 }
 
 // The four rows that become new when the window moves from output rows (i-2, i-1) to (i, i+1):
 // I[t(i)], I[t(i+1)], I[b(i+1)], I[b(i+2)].
-template <class T, int K, bool FULL>
+template <class T, int NT, int K, bool FULL>
 __device__ __forceinline__ void load_pair(const T* __restrict__ plane, int64_t pitch, int i,
-                                          int xlo, int xhi, int h, unsigned row_bytes,
-                                          const unsigned (&qoff)[K], T (&t0)[K], T (&t1)[K],
-                                          T (&b1)[K], T (&b2)[K]) {
-    load_row<T, K, FULL>(plane, pitch, clampi(i + xlo, 0, h), row_bytes, qoff, t0);
-    load_row<T, K, FULL>(plane, pitch, clampi(i + 1 + xlo, 0, h), row_bytes, qoff, t1);
-    load_row<T, K, FULL>(plane, pitch, clampi(i + 1 + xhi, 0, h), row_bytes, qoff, b1);
-    load_row<T, K, FULL>(plane, pitch, clampi(i + 2 + xhi, 0, h), row_bytes, qoff, b2);
+                                          int xlo, int xhi, int h, unsigned row_bytes, unsigned q1,
+                                          T (&t0)[K], T (&t1)[K], T (&b1)[K], T (&b2)[K]) {
+    load_row<T, NT, K, FULL>(plane, pitch, clampi(i + xlo, 0, h), row_bytes, q1, t0);
+    load_row<T, NT, K, FULL>(plane, pitch, clampi(i + 1 + xlo, 0, h), row_bytes, q1, t1);
+    load_row<T, NT, K, FULL>(plane, pitch, clampi(i + 1 + xhi, 0, h), row_bytes, q1, b1);
+    load_row<T, NT, K, FULL>(plane, pitch, clampi(i + 2 + xhi, 0, h), row_bytes, q1, b2);
 }
 
 template <class T, bool EXACT>
@@ -134,15 +215,15 @@ __device__ __forceinline__ T blend(T lo_adv, T lo, T hi, T hi_adv, T flo, T fhi)
 // Row vectors V(i), V(i+1) into LDS. Layout: V[q+1] for q = -1..w+1 with V(-1) = V(0) = 0 (written
 // once by clear_row_pads) and V(w+1) = V(w), so a clamped column pair is always two adjacent
 // entries.
-template <class T, int K, bool FULL>
+template <class T, int NT, int K, bool FULL>
 __device__ __forceinline__ void publish_rows(RowPair<T>* __restrict__ V, const T (&v0)[K],
-                                             const T (&v1)[K], int w, unsigned row_bytes,
-                                             const unsigned (&qoff)[K], int nt) {
+                                             const T (&v1)[K], int w, unsigned row_bytes, unsigned q1) {
 #pragma unroll
     for (int k = 0; k < K; ++k) {
         const RowPair<T> pr{v0[k], v1[k]};
-        if (FULL || qoff[k] <= row_bytes) *at_bytes(V + 1, 2 * qoff[k]) = pr;
-        if (FULL ? (k == K - 1 && static_cast<int>(threadIdx.x) == nt - 1) : (qoff[k] == row_bytes))
+        if (slot_valid<T, NT, FULL>(q1, k, row_bytes)) *at_bytes(V + 1 + NT * k, 2 * q1) = pr;
+        if (FULL ? (k == K - 1 && static_cast<int>(threadIdx.x) == NT - 1)
+                 : (q1 + slot_bytes<T, NT>(k) == row_bytes))
             V[w + 2] = pr;
     }
 }
@@ -153,12 +234,12 @@ __device__ __forceinline__ void clear_row_pads(RowPair<T>* vbuf, int vlen) {
 
 // LDS byte offsets of the column pairs (lAdv, l) = (lo, lo+1) and (r, rAdv) = (hi, hi+1) of the
 // lane's pixels.
-template <class T, int K>
+template <class T, int NT, int K>
 __device__ __forceinline__ void column_taps(unsigned (&lo)[K], unsigned (&hi)[K], int ylo, int yhi,
-                                            int w, int nt) {
+                                            int w) {
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-        const int j = static_cast<int>(threadIdx.x) + nt * k;
+        const int j = static_cast<int>(threadIdx.x) + NT * k;
         lo[k] = static_cast<unsigned>(clampi(j + ylo, 0, w + 1)) * static_cast<unsigned>(sizeof(RowPair<T>));
         hi[k] = static_cast<unsigned>(clampi(j + yhi, -1, w) + 1) * static_cast<unsigned>(sizeof(RowPair<T>));
     }
@@ -190,10 +271,10 @@ using Flip0 = std::integral_constant<int, 0>;
 using Flip1 = std::integral_constant<int, 1>;
 
 // ---------------------------------------------------------------------------------------------
-// Forward. Work item = (plane p, filter f, band). blockDim = nt, K >= ceil(w / nt).
+// Forward. Work item = (plane p, filter f, band). blockDim = NT, K >= ceil(w / NT).
 // LDS: [2 buffers][w+3] RowPair<T>.
-template <class T, int K, bool EXACT, bool FULL>
-__global__ void __launch_bounds__(kMaxRowThreads) forward_rows_kernel(SampleArgs<T> a) {
+template <class T, int NT, int K, bool EXACT, bool FULL>
+__global__ void __launch_bounds__(NT) forward_rows_kernel(SampleArgs<T> a) {
     const int64_t vid = xcd_contiguous_id(a.per_xcd);
     if (vid >= a.total) return;
     const int band = static_cast<int>(vid % a.nb);
@@ -201,7 +282,7 @@ __global__ void __launch_bounds__(kMaxRowThreads) forward_rows_kernel(SampleArgs
     const int f = static_cast<int>(pf % a.F);
     const int64_t p = pf / a.F;
     const int k_par = static_cast<int>((a.plane0 + p) % a.C) * a.F + f;
-    const int h = a.h, w = a.w, nt = blockDim.x;
+    const int h = a.h, w = a.w;
     const unsigned row_bytes = static_cast<unsigned>(w) * sizeof(T);
 
     const BoxOfWorkgroup<T> bx = load_box(a.prm, k_par);
@@ -219,15 +300,15 @@ __global__ void __launch_bounds__(kMaxRowThreads) forward_rows_kernel(SampleArgs
     const int i0 = band * a.R;
     const int i1 = min(h, i0 + a.R);
 
-    unsigned qoff[K], lo[K], hi[K];
-    lane_columns<T, K>(qoff, nt);
-    column_taps<T, K>(lo, hi, s.ylo, s.yhi, w, nt);
+    const unsigned q1 = lane_q1<T>();
+    unsigned lo[K], hi[K];
+    column_taps<T, NT, K>(lo, hi, s.ylo, s.yhi, w);
 
     T ta[K], bc[K];                       // I[t(i-1)], I[b(i)]
     T t0[K], t1[K], b1[K], b2[K];         // I[t(i)], I[t(i+1)], I[b(i+1)], I[b(i+2)]
-    load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), row_bytes, qoff, ta);
-    load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xhi, 0, h), row_bytes, qoff, bc);
-    load_pair<T, K, FULL>(plane, pitch, i0, s.xlo, s.xhi, h, row_bytes, qoff, t0, t1, b1, b2);
+    load_row<T, NT, K, FULL>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), row_bytes, q1, ta);
+    load_row<T, NT, K, FULL>(plane, pitch, clampi(i0 + s.xhi, 0, h), row_bytes, q1, bc);
+    load_pair<T, NT, K, FULL>(plane, pitch, i0, s.xlo, s.xhi, h, row_bytes, q1, t0, t1, b1, b2);
 
     // One row pair. PREFETCH and the LDS buffer are compile-time tags: the loop body always
     // issues the next pair's loads and the last pair is peeled, so no branch joins a path with
@@ -239,7 +320,7 @@ __global__ void __launch_bounds__(kMaxRowThreads) forward_rows_kernel(SampleArgs
         constexpr int FLIP = decltype(flip_tag)::value;
         T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {};
         if (PREFETCH)
-            load_pair<T, K, FULL>(plane, pitch, i + 2, s.xlo, s.xhi, h, row_bytes, qoff, n0, n1, n2, n3);
+            load_pair<T, NT, K, FULL>(plane, pitch, i + 2, s.xlo, s.xhi, h, row_bytes, q1, n0, n1, n2, n3);
 
         RowPair<T>* V = vbuf + (FLIP ? vlen : 0);
         T v0[K], v1[K];
@@ -248,17 +329,20 @@ __global__ void __launch_bounds__(kMaxRowThreads) forward_rows_kernel(SampleArgs
             v0[k] = blend<T, EXACT>(ta[k], t0[k], bc[k], b1[k], s.fxlo, s.fxhi);
             v1[k] = blend<T, EXACT>(t0[k], t1[k], b1[k], b2[k], s.fxlo, s.fxhi);
         }
-        publish_rows<T, K, FULL>(V, v0, v1, w, row_bytes, qoff, nt);
+        publish_rows<T, NT, K, FULL>(V, v0, v1, w, row_bytes, q1);
         __syncthreads();
 
-        T* orow = out + static_cast<int64_t>(i) * w - 1;     // column q = j + 1 lands on pixel j
-        const bool second = i + 1 < i1;
+        // column q = j + 1 lands on pixel j; the second row may lie past the band (size 0)
+        T* orow = out + static_cast<int64_t>(i) * w - 1;
+        const unsigned out_bytes = row_bytes + static_cast<unsigned>(sizeof(T));
+        const __amdgpu_buffer_rsrc_t ob0 = row_buffer(orow, out_bytes);
+        const __amdgpu_buffer_rsrc_t ob1 = row_buffer(orow + w, i + 1 < i1 ? out_bytes : 0u);
 #pragma unroll
         for (int k = 0; k < K; ++k) {
-            if (FULL || qoff[k] <= row_bytes) {
+            if (slot_valid<T, NT, FULL>(q1, k, row_bytes)) {
                 const RowPair<T> o = sample_columns<T, EXACT>(V, lo[k], hi[k], s.fylo, s.fyhi);
-                __builtin_nontemporal_store(o.r0 * scale, at_bytes(orow, qoff[k]));
-                if (second) __builtin_nontemporal_store(o.r1 * scale, at_bytes(orow + w, qoff[k]));
+                store_slot<T, NT, FULL, kCacheStream>(o.r0 * scale, ob0, q1, k);
+                store_slot<T, NT, FULL, kCacheStream>(o.r1 * scale, ob1, q1, k);
             }
         }
         if (PREFETCH) {
@@ -290,15 +374,15 @@ __global__ void __launch_bounds__(kMaxRowThreads) forward_rows_kernel(SampleArgs
 // involves differences between rows, so a row is corrected relative to a reference band (that of
 // the first row this workgroup touches for the filter): the bulk of the integral cancels before
 // it is ever added.
-template <class T, int K, int RB, bool EXACT, bool FULL, bool OFFS>
-__global__ void __launch_bounds__(kMaxRowThreads, BOXCONV_GI_WAVES) grad_input_rows_kernel(SampleArgs<T> a) {
+template <class T, int NT, int K, int RB, bool EXACT, bool FULL, bool OFFS>
+__global__ void __launch_bounds__(NT) grad_input_rows_kernel(SampleArgs<T> a) {
     static_assert(RB % 4 == 0, "rows are handled in pairs, and pairs alternate between two LDS buffers");
     const int64_t vid = xcd_contiguous_id(a.per_xcd);
     if (vid >= a.total) return;
     const int band = static_cast<int>(vid % a.nb);
     const int64_t p = vid / a.nb;
     const int c_in = static_cast<int>((a.plane0 + p) % a.C);
-    const int h = a.h, w = a.w, nt = blockDim.x;
+    const int h = a.h, w = a.w;
     const unsigned row_bytes = static_cast<unsigned>(w) * sizeof(T);
     const int64_t pitch = w + 1;
     const int64_t ipl = static_cast<int64_t>(h + 1) * pitch;
@@ -307,8 +391,7 @@ __global__ void __launch_bounds__(kMaxRowThreads, BOXCONV_GI_WAVES) grad_input_r
     clear_row_pads(vbuf, vlen);
     const int i0 = band * RB;
 
-    unsigned qoff[K];
-    lane_columns<T, K>(qoff, nt);
+    const unsigned q1 = lane_q1<T>();
 
     T acc[RB][K];
 #pragma unroll
@@ -324,7 +407,7 @@ __global__ void __launch_bounds__(kMaxRowThreads, BOXCONV_GI_WAVES) grad_input_r
         const T* plane = a.src + (p * a.F + f) * ipl;
 
         unsigned lo[K], hi[K];
-        column_taps<T, K>(lo, hi, s.ylo, s.yhi, w, nt);
+        column_taps<T, NT, K>(lo, hi, s.ylo, s.yhi, w);
 
         // OFFS: `plane` holds a band-local integral (bands of off_R rows, each restarting at
         // zero). Integral row r (1..h) belongs to band (r-1)/off_R; row 0 counts as band 0. The
@@ -345,7 +428,7 @@ __global__ void __launch_bounds__(kMaxRowThreads, BOXCONV_GI_WAVES) grad_input_r
             for (int k = 0; k < K; ++k) sum[k] = 0.0;
             for (int b = ref_band; b < cached_band; ++b) {
                 T bottom[K];
-                load_row<T, K, FULL>(plane, pitch, min(h, (b + 1) * a.off_R), row_bytes, qoff, bottom);
+                load_row<T, NT, K, FULL>(plane, pitch, min(h, (b + 1) * a.off_R), row_bytes, q1, bottom);
 #pragma unroll
                 for (int k = 0; k < K; ++k) sum[k] += static_cast<double>(bottom[k]);
             }
@@ -361,9 +444,9 @@ __global__ void __launch_bounds__(kMaxRowThreads, BOXCONV_GI_WAVES) grad_input_r
         };
 
         T ta[K], bc[K], t0[K], t1[K], b1[K], b2[K];
-        load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), row_bytes, qoff, ta);
-        load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xhi, 0, h), row_bytes, qoff, bc);
-        load_pair<T, K, FULL>(plane, pitch, i0, s.xlo, s.xhi, h, row_bytes, qoff, t0, t1, b1, b2);
+        load_row<T, NT, K, FULL>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), row_bytes, q1, ta);
+        load_row<T, NT, K, FULL>(plane, pitch, clampi(i0 + s.xhi, 0, h), row_bytes, q1, bc);
+        load_pair<T, NT, K, FULL>(plane, pitch, i0, s.xlo, s.xhi, h, row_bytes, q1, t0, t1, b1, b2);
         correct(ta, clampi(i0 + s.xlo - 1, 0, h), band_t, last_t, off_t);
         correct(t0, clampi(i0 + s.xlo, 0, h), band_t, last_t, off_t);
         correct(t1, clampi(i0 + 1 + s.xlo, 0, h), band_t, last_t, off_t);
@@ -380,7 +463,7 @@ __global__ void __launch_bounds__(kMaxRowThreads, BOXCONV_GI_WAVES) grad_input_r
             T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {};
             const bool more = r + 2 < RB;                                // known after unrolling
             if (more)
-                load_pair<T, K, FULL>(plane, pitch, i + 2, s.xlo, s.xhi, h, row_bytes, qoff, n0, n1, n2, n3);
+                load_pair<T, NT, K, FULL>(plane, pitch, i + 2, s.xlo, s.xhi, h, row_bytes, q1, n0, n1, n2, n3);
             RowPair<T>* V = vbuf + (((r >> 1) & 1) ? vlen : 0);
             T v0[K], v1[K];
 #pragma unroll
@@ -388,11 +471,11 @@ __global__ void __launch_bounds__(kMaxRowThreads, BOXCONV_GI_WAVES) grad_input_r
                 v0[k] = blend<T, EXACT>(ta[k], t0[k], bc[k], b1[k], s.fxlo, s.fxhi);
                 v1[k] = blend<T, EXACT>(t0[k], t1[k], b1[k], b2[k], s.fxlo, s.fxhi);
             }
-            publish_rows<T, K, FULL>(V, v0, v1, w, row_bytes, qoff, nt);
+            publish_rows<T, NT, K, FULL>(V, v0, v1, w, row_bytes, q1);
             __syncthreads();
 #pragma unroll
             for (int k = 0; k < K; ++k) {
-                if (FULL || qoff[k] <= row_bytes) {
+                if (slot_valid<T, NT, FULL>(q1, k, row_bytes)) {
                     const RowPair<T> o = sample_columns<T, EXACT>(V, lo[k], hi[k], s.fylo, s.fyhi);
                     acc[r][k] += scale * o.r0;
                     acc[r + 1][k] += scale * o.r1;
@@ -415,12 +498,11 @@ __global__ void __launch_bounds__(kMaxRowThreads, BOXCONV_GI_WAVES) grad_input_r
     T* out = a.dst + p * static_cast<int64_t>(h) * w - 1;    // column q = j + 1 lands on pixel j
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
-        const int i = i0 + r;
-        if (i < h) {
+        const int i = i0 + r;                                // rows past the image: size 0
+        const __amdgpu_buffer_rsrc_t ob = row_buffer(out + static_cast<int64_t>(min(i, h - 1)) * w,
+                                                     i < h ? row_bytes + static_cast<unsigned>(sizeof(T)) : 0u);
 #pragma unroll
-            for (int k = 0; k < K; ++k)
-                if (FULL || qoff[k] <= row_bytes) *at_bytes(out + static_cast<int64_t>(i) * w, qoff[k]) = acc[r][k];
-        }
+        for (int k = 0; k < K; ++k) store_slot<T, NT, FULL, kCacheDefault>(acc[r][k], ob, q1, k);
     }
 }
 
@@ -464,18 +546,18 @@ __device__ __forceinline__ void block_accumulate5(const double (&v)[5], double* 
 // band_start..i and columns 0..c. Bands do not depend on each other, so nothing has to be known
 // about the rows above: the true integral is L plus the bottom rows of the bands above, which
 // the grad-input kernel adds when it loads a row. Lanes own K consecutive columns for this part
-// (read back from the LDS row), results go through an LDS stage so that global stores are
-// lane-consecutive dwords.
+// (read back from the LDS row) and store them as one run, so a wave writes 64*K contiguous
+// elements per row.
 //
 // LDS: [2 buffers][K*nt + 8] RowPair grad_output rows (4 zero pairs in front, >= 4 behind),
-//      [2][2][4] X[w] triples, [K*nt] RowPair stage, [8*5] doubles, [2][8] wave totals.
+//      [2][2][4] X[w] triples, [K*nt] tail weights, [8*5] doubles, [2][8] wave totals.
 constexpr int kGPad = 4;
 
 template <class T>
 struct StreamLds {
     RowPair<T>* grow;   // [2][glen]
     T* xw;              // [2][2][4]
-    RowPair<T>* stage;  // [K*nt]
+    T* delta;           // [K*nt] tail weight of pixel column j
     double* red;        // [5 * kMaxRowWaves]
     T* wave_tot;        // [2][kMaxRowWaves]
     int glen;
@@ -483,7 +565,7 @@ struct StreamLds {
 
 __host__ __device__ inline size_t stream_lds_bytes(int K, int nt, size_t elem) {
     const size_t glen = static_cast<size_t>(K) * nt + 8;
-    size_t b = (4 * glen + 16 + 2 * static_cast<size_t>(K) * nt) * elem;
+    size_t b = (4 * glen + 16 + static_cast<size_t>(K) * nt) * elem;
     b = (b + 15) / 16 * 16;
     return b + (2 * kMaxRowWaves + 5 * kMaxRowWaves) * sizeof(double);
 }
@@ -494,16 +576,27 @@ __device__ __forceinline__ StreamLds<T> carve_stream_lds(int K, int nt) {
     l.glen = K * nt + 8;
     l.grow = reinterpret_cast<RowPair<T>*>(smem_raw);
     l.xw = reinterpret_cast<T*>(l.grow + 2 * l.glen);
-    l.stage = reinterpret_cast<RowPair<T>*>(l.xw + 16);
-    size_t b = (4 * static_cast<size_t>(l.glen) + 16 + 2 * static_cast<size_t>(K) * nt) * sizeof(T);
+    l.delta = l.xw + 16;
+    size_t b = (4 * static_cast<size_t>(l.glen) + 16 + static_cast<size_t>(K) * nt) * sizeof(T);
     b = (b + 15) / 16 * 16;
     l.red = reinterpret_cast<double*>(smem_raw + b);
     l.wave_tot = reinterpret_cast<T*>(l.red + 5 * kMaxRowWaves);
     return l;
 }
 
-template <class T, int K, bool EXACT, bool FULL, bool PARAMS, bool SCAN>
-__global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(SampleArgs<T> a) {
+template <class T, int WV>
+__device__ __forceinline__ void add_waves_left(const T* wave_tot, int wave, T& carry0, T& carry1) {
+    if constexpr (WV < kMaxRowWaves - 1) {
+        if (wave > WV) {
+            carry0 += wave_tot[WV];
+            carry1 += wave_tot[kMaxRowWaves + WV];
+            add_waves_left<T, WV + 1>(wave_tot, wave, carry0, carry1);
+        }
+    }
+}
+
+template <class T, int NT, int K, bool EXACT, bool FULL, bool PARAMS, bool SCAN>
+__global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a) {
     const int64_t vid = xcd_contiguous_id(a.per_xcd);
     if (vid >= a.total) return;                      // whole workgroup leaves together
     const int band = static_cast<int>(vid % a.nb);
@@ -511,7 +604,8 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
     const int f = static_cast<int>(pf % a.F);
     const int64_t p = pf / a.F;
     const int k_par = static_cast<int>((a.plane0 + p) % a.C) * a.F + f;
-    const int h = a.h, w = a.w, nt = blockDim.x, tid = threadIdx.x;
+    const int h = a.h, w = a.w, tid = threadIdx.x;
+    constexpr int nt = NT;
     const unsigned row_bytes = static_cast<unsigned>(w) * sizeof(T);
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keep it scalar
@@ -535,12 +629,11 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
         for (int c = tid; c <= w; c += nt) lrows[c] = T(0);                    // integral row 0
     __syncthreads();
 
-    unsigned qoff[K];
-    lane_columns<T, K>(qoff, nt);
+    const unsigned q1 = lane_q1<T>();
 
-    // lane-constant LDS byte offsets of the pairs (grA, gr) and (gl, glA), and the tail weights
+    // lane-constant LDS byte offsets of the pairs (grA, gr) and (gl, glA); the tail weights of the
+    // lane's columns go to LDS (read back once per row pair: cheaper than K live registers)
     unsigned ir[K], il[K];
-    T delta[K];
     unsigned idx_ymax = 0, idx_ymin = 0;
     if (PARAMS) {
 #pragma unroll
@@ -557,7 +650,7 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
                   - (EXACT ? (one - s.fylo) : one) * T(j > w - s.ylo)
                   - (EXACT ? s.fylo : T(0)) * T(j > w - s.ylo + 1);
             }
-            delta[k] = d;
+            lds.delta[j] = d;
         }
         const int j_ymax = w - s.yhi, j_ymin = w - s.ylo + 1;
         idx_ymax = (j_ymax >= 0 && j_ymax < w) ? j_ymax + kGPad : 0;          // index 0 holds a zero
@@ -571,28 +664,33 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
 
     T ta[K], bc[K], t0[K], t1[K], b1[K], b2[K], g0[K], g1[K];
     if (PARAMS) {
-        load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), row_bytes, qoff, ta);
-        load_row<T, K, FULL>(plane, pitch, clampi(i0 + s.xhi, 0, h), row_bytes, qoff, bc);
-        load_pair<T, K, FULL>(plane, pitch, i0, s.xlo, s.xhi, h, row_bytes, qoff, t0, t1, b1, b2);
+        load_row<T, NT, K, FULL>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), row_bytes, q1, ta);
+        load_row<T, NT, K, FULL>(plane, pitch, clampi(i0 + s.xhi, 0, h), row_bytes, q1, bc);
+        load_pair<T, NT, K, FULL>(plane, pitch, i0, s.xlo, s.xhi, h, row_bytes, q1, t0, t1, b1, b2);
     }
     auto load_g = [&](int i, T (&dst)[K]) {
-        const T* grow = gout + static_cast<int64_t>(min(i, h - 1)) * w - 1;   // column q = j + 1 -> pixel j
-        const bool valid = i < i1;
+        // column q = j + 1 -> pixel j; rows past the band read as zeros (size 0)
+        const __amdgpu_buffer_rsrc_t rs = row_buffer(gout + static_cast<int64_t>(min(i, h - 1)) * w - 1,
+                                                     i < i1 ? row_bytes + static_cast<unsigned>(sizeof(T)) : 0u);
 #pragma unroll
-        for (int k = 0; k < K; ++k)
-            dst[k] = (valid && (FULL || qoff[k] <= row_bytes))
-                         ? __builtin_nontemporal_load(at_bytes(grow, qoff[k])) : T(0);
+        for (int k = 0; k < K; ++k) dst[k] = load_slot<T, NT, FULL, kCacheStream>(rs, q1, k);
     };
     load_g(i0, g0);
     load_g(i0 + 1, g1);
 
+    int flip = 0;
     auto row_pair = [&](int i, auto prefetch_tag, auto flip_tag) {
         constexpr bool PREFETCH = decltype(prefetch_tag)::value;   // see forward_rows_kernel
+#if BOXCONV_STREAM_UNROLL
         constexpr int FLIP = decltype(flip_tag)::value;
+#else
+        const int FLIP = flip;
+        flip ^= 1;
+#endif
         T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {}, m0[K] = {}, m1[K] = {};
         if (PREFETCH) {
             if (PARAMS)
-                load_pair<T, K, FULL>(plane, pitch, i + 2, s.xlo, s.xhi, h, row_bytes, qoff, n0, n1, n2, n3);
+                load_pair<T, NT, K, FULL>(plane, pitch, i + 2, s.xlo, s.xhi, h, row_bytes, q1, n0, n1, n2, n3);
             load_g(i + 2, m0);
             load_g(i + 3, m1);
         }
@@ -604,10 +702,14 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
         T tail0 = T(0), tail1 = T(0);
 #pragma unroll
         for (int k = 0; k < K; ++k) {
-            if (FULL || qoff[k] <= row_bytes)
-                *at_bytes(G + kGPad - 1, 2 * qoff[k]) = RowPair<T>{g0[k], g1[k]};
-            if (PARAMS) { tail0 += delta[k] * g0[k]; tail1 += delta[k] * g1[k]; }
-            if (PARAMS && (FULL ? (k == K - 1 && tid == nt - 1) : (qoff[k] == row_bytes))) {   // owner of column q = w
+            if (slot_valid<T, NT, FULL>(q1, k, row_bytes))
+                *at_bytes(G + kGPad - 1 + NT * k, 2 * q1) = RowPair<T>{g0[k], g1[k]};
+            if (PARAMS) {
+                const T dlt = *at_bytes(lds.delta - 1 + NT * k, q1);
+                tail0 += dlt * g0[k];
+                tail1 += dlt * g1[k];
+            }
+            if (PARAMS && (FULL ? (k == K - 1 && tid == nt - 1) : (q1 + slot_bytes<T, NT>(k) == row_bytes))) {   // owner of column q = w
                 const T dt0 = t0[k] - ta[k], db0 = b1[k] - bc[k];
                 const T dt1 = t1[k] - t0[k], db1 = b2[k] - b1[k];
                 T v0 = bc[k] - t0[k], v1 = b1[k] - t1[k];
@@ -694,29 +796,22 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
             }
             __syncthreads();                                                 // wave totals visible
             {
-#pragma unroll
-                for (int wv = 0; wv < kMaxRowWaves - 1; ++wv)
-                    if (wv < wave) {                                         // scalar condition
-                        carry0 += lds.wave_tot[wv];
-                        carry1 += lds.wave_tot[kMaxRowWaves + wv];
-                    }
-                RowPair<T>* st = lds.stage + K * tid;
-#pragma unroll
-                for (int k = 0; k < K; ++k) st[k] = RowPair<T>{carry0 + loc0[k], carry1 + loc1[k]};
-            }
-            __syncthreads();                                                 // stage visible
-            {
+                // totals of the waves to the left; `wave` is scalar, so these are scalar branches
+                // and wave n takes n + 1 of them
+                add_waves_left<T, 0>(lds.wave_tot, wave, carry0, carry1);
+                // the lane's K consecutive columns K*tid+1 .. K*tid+K of integral rows i+1, i+2:
+                // a wave stores one contiguous run of 64*K elements per row
                 T* o0 = lrows + static_cast<int64_t>(i + 1) * pitch;
-                T* o1 = o0 + pitch;
                 const bool second = i + 1 < i1;
+                const unsigned out_bytes = row_bytes + static_cast<unsigned>(sizeof(T));
+                const __amdgpu_buffer_rsrc_t ob0 = row_buffer(o0, out_bytes);
+                const __amdgpu_buffer_rsrc_t ob1 = row_buffer(o0 + pitch, second ? out_bytes : 0u);
+                T out0[K], out1[K];
 #pragma unroll
-                for (int k = 0; k < K; ++k) {
-                    if (FULL || qoff[k] <= row_bytes) {
-                        const RowPair<T> v = *at_bytes(lds.stage - 1, 2 * qoff[k]);   // column j = q - 1
-                        __builtin_nontemporal_store(v.r0, at_bytes(o0, qoff[k]));
-                        if (second) __builtin_nontemporal_store(v.r1, at_bytes(o1, qoff[k]));
-                    }
-                }
+                for (int k = 0; k < K; ++k) { out0[k] = carry0 + loc0[k]; out1[k] = carry1 + loc1[k]; }
+                const unsigned first = static_cast<unsigned>(1 + K * tid) * static_cast<unsigned>(sizeof(T));
+                buffer_store_run<kCacheStream, FULL>(out0, ob0, first);
+                buffer_store_run<kCacheStream, FULL>(out1, ob1, first);
                 if (tid == 0) {
                     o0[0] = T(0);
                     if (second) o0[pitch] = T(0);
@@ -734,8 +829,12 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
                 g0[k] = m0[k]; g1[k] = m1[k];
             }
         }
+        // keep the two unrolled pairs apart: loads of the pair after next hoisted up here would
+        // only add live registers
+        __builtin_amdgcn_sched_barrier(0);
     };
     int i = i0;
+#if BOXCONV_STREAM_UNROLL
     for (; i + 4 < i1; i += 4) {
         row_pair(i, std::true_type{}, Flip0{});
         row_pair(i + 2, std::true_type{}, Flip1{});
@@ -746,6 +845,10 @@ __global__ void __launch_bounds__(kMaxRowThreads) grad_output_stream_kernel(Samp
     } else {
         row_pair(i, std::false_type{}, Flip0{});
     }
+#else
+    for (; i + 2 < i1; i += 2) row_pair(i, std::true_type{}, 0);
+    row_pair(i, std::false_type{}, 0);
+#endif
 
     if (PARAMS) {
         __syncthreads();
@@ -901,26 +1004,34 @@ __global__ void param_grad_finalize_kernel(const double* __restrict__ acc, BoxPa
 }
 
 // ---------------------------------------------------------------------------------------------
+// Workgroup shapes the row kernels are compiled for: (threads, columns per lane).
+//   (64,1) widths up to 64; (256,1|2|4) up to 256|512|1024; (512,1|2|4) up to 512|1024|2048.
+// Each kernel has a preferred size (measured at width 1024: 512 threads for forward and grad
+// input, 256 for the grad_output pass); rows too wide for 4 columns per lane at that size take
+// 512 threads, which bounds the register footprint and the length of the per-lane float
+// accumulation chains.
 struct RowConfig { int nt; int K; bool full; };
-inline int max_row_threads() {
-    static const int v = [] {
-        const char* e = std::getenv("BOXCONV_ROW_THREADS");
-        const int n = e ? std::atoi(e) : kMaxRowThreads;
-        return (n == 64 || n == 128 || n == 256 || n == 512) ? n : kMaxRowThreads;
-    }();
-    return v;
+inline int preferred_row_threads(const char* env_name, int fallback) {
+    const char* e = std::getenv(env_name);
+    const int n = e ? std::atoi(e) : fallback;
+    return (n == 256 || n == 512) ? n : fallback;
 }
-inline RowConfig row_config(int w, int cap = 256) {
+inline RowConfig row_config(int w, int prefer) {
     RowConfig c;
-    // `cap` threads are preferred (measured fastest at widths up to 1024); wider rows take the
-    // largest workgroup instead of more than 4 columns per lane, which keeps the register
-    // footprint and the length of the per-lane float accumulation chains bounded.
-    c.nt = std::min(std::min(max_row_threads(), cap), ((w + 63) / 64) * 64);
-    if ((w + c.nt - 1) / c.nt > 4) c.nt = std::min(max_row_threads(), ((w + 63) / 64) * 64);
-    const int k = (w + c.nt - 1) / c.nt;
-    c.K = k <= 1 ? 1 : k <= 2 ? 2 : k <= 4 ? 4 : 8;
+    if (w <= 64) {
+        c.nt = 64; c.K = 1;
+    } else {
+        c.nt = (w + prefer - 1) / prefer > 4 ? 512 : prefer;
+        const int k = (w + c.nt - 1) / c.nt;
+        c.K = k <= 1 ? 1 : k <= 2 ? 2 : 4;
+    }
     c.full = (c.K * c.nt == w);
     return c;
+}
+
+inline RowConfig stream_row_config(int w) {
+    static const int prefer = preferred_row_threads("BOXCONV_STREAM_THREADS", 256);
+    return row_config(w, prefer);
 }
 
 inline int bands_for(int64_t independent, int h, int min_rows, int64_t want) {
@@ -942,20 +1053,23 @@ void finish_args(SampleArgs<T>& a, int64_t total) {
     a.per_xcd = (total + kXcds - 1) / kXcds;
 }
 
-#define BOXCONV_DISPATCH_K(KERNEL, K, ...)                                           \
+#define BOXCONV_DISPATCH_K(KERNEL, NT, K, ...)                                       \
     switch (K) {                                                                     \
-        case 1: KERNEL(1, __VA_ARGS__); break;                                       \
-        case 2: KERNEL(2, __VA_ARGS__); break;                                       \
-        case 4: KERNEL(4, __VA_ARGS__); break;                                       \
-        default: KERNEL(8, __VA_ARGS__); break;                                      \
+        case 1: KERNEL(NT, 1, __VA_ARGS__); break;                                   \
+        case 2: KERNEL(NT, 2, __VA_ARGS__); break;                                   \
+        default: KERNEL(NT, 4, __VA_ARGS__); break;                                  \
     }
-#define BOXCONV_DISPATCH_K_EXACT_FULL(KERNEL, K, EXACT, FULL)                        \
+#define BOXCONV_DISPATCH_SHAPE(KERNEL, RC, ...)                                      \
+    if ((RC).nt == 64)       { KERNEL(64, 1, __VA_ARGS__); }                         \
+    else if ((RC).nt == 256) { BOXCONV_DISPATCH_K(KERNEL, 256, (RC).K, __VA_ARGS__) } \
+    else                     { BOXCONV_DISPATCH_K(KERNEL, 512, (RC).K, __VA_ARGS__) }
+#define BOXCONV_DISPATCH_SHAPE_EXACT_FULL(KERNEL, RC, EXACT)                         \
     if (EXACT) {                                                                     \
-        if (FULL) { BOXCONV_DISPATCH_K(KERNEL, K, true, true) }                      \
-        else      { BOXCONV_DISPATCH_K(KERNEL, K, true, false) }                     \
+        if ((RC).full) { BOXCONV_DISPATCH_SHAPE(KERNEL, RC, true, true) }            \
+        else           { BOXCONV_DISPATCH_SHAPE(KERNEL, RC, true, false) }           \
     } else {                                                                         \
-        if (FULL) { BOXCONV_DISPATCH_K(KERNEL, K, false, true) }                     \
-        else      { BOXCONV_DISPATCH_K(KERNEL, K, false, false) }                    \
+        if ((RC).full) { BOXCONV_DISPATCH_SHAPE(KERNEL, RC, false, true) }           \
+        else           { BOXCONV_DISPATCH_SHAPE(KERNEL, RC, false, false) }          \
     }
 
 }  // namespace
@@ -976,7 +1090,8 @@ hipError_t forward_launch(const T* integ, BoxParams<T> prm, T* out, Dims d, bool
         return hipGetLastError();
     }
 
-    const RowConfig rc = row_config(d.w);
+    static const int fwd_threads = preferred_row_threads("BOXCONV_FWD_THREADS", 512);
+    const RowConfig rc = row_config(d.w, fwd_threads);
     a.nb = bands_for(planes_f, d.h, 16, 4096);
     a.R = (d.h + a.nb - 1) / a.nb;
     a.R += a.R & 1;                                   // rows are handled in pairs
@@ -984,9 +1099,9 @@ hipError_t forward_launch(const T* integ, BoxParams<T> prm, T* out, Dims d, bool
     finish_args(a, planes_f * a.nb);
     const dim3 grid(static_cast<unsigned>(a.per_xcd * kXcds));
     const size_t lds = 4 * static_cast<size_t>(d.w + 3) * sizeof(T);
-#define LAUNCH_FWD(KK, EX, FU) \
-    BOXCONV_LAUNCH("forward_rows", (forward_rows_kernel<T, KK, EX, FU>), grid, dim3(rc.nt), lds, stream, a)
-    BOXCONV_DISPATCH_K_EXACT_FULL(LAUNCH_FWD, rc.K, exact, rc.full)
+#define LAUNCH_FWD(NT, KK, EX, FU) \
+    BOXCONV_LAUNCH("forward_rows", (forward_rows_kernel<T, NT, KK, EX, FU>), grid, dim3(NT), lds, stream, a)
+    BOXCONV_DISPATCH_SHAPE_EXACT_FULL(LAUNCH_FWD, rc, exact)
 #undef LAUNCH_FWD
     return hipGetLastError();
 }
@@ -1009,20 +1124,17 @@ hipError_t grad_input_launch(const T* gint, int band_rows, BoxParams<T> prm, T* 
     }
 
     constexpr int RB = 8;
-    static const int gi_threads = [] {
-        const char* e = std::getenv("BOXCONV_GI_THREADS");
-        return e ? std::atoi(e) : BOXCONV_GI_THREADS;
-    }();
+    static const int gi_threads = preferred_row_threads("BOXCONV_GI_THREADS", 512);
     const RowConfig rc = row_config(d.w, gi_threads);
     a.nb = (d.h + RB - 1) / RB;
     a.R = RB;
     finish_args(a, d.planes * a.nb);
     const dim3 grid(static_cast<unsigned>(a.per_xcd * kXcds));
     const size_t lds = 4 * static_cast<size_t>(d.w + 3) * sizeof(T);
-#define LAUNCH_GI(KK, EX, FU) \
-    if (band_rows > 0) BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, KK, RB, EX, FU, true>), grid, dim3(rc.nt), lds, stream, a); \
-    else BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, KK, RB, EX, FU, false>), grid, dim3(rc.nt), lds, stream, a)
-    BOXCONV_DISPATCH_K_EXACT_FULL(LAUNCH_GI, rc.K, exact, rc.full)
+#define LAUNCH_GI(NT, KK, EX, FU) \
+    if (band_rows > 0) BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, NT, KK, RB, EX, FU, true>), grid, dim3(NT), lds, stream, a); \
+    else BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, NT, KK, RB, EX, FU, false>), grid, dim3(NT), lds, stream, a)
+    BOXCONV_DISPATCH_SHAPE_EXACT_FULL(LAUNCH_GI, rc, exact)
 #undef LAUNCH_GI
     return hipGetLastError();
 }
@@ -1036,7 +1148,7 @@ hipError_t grad_params_begin(double* acc, int n_boxes, hipStream_t stream) {
 
 StreamPlan plan_grad_output_stream(int64_t planes_f, int h, int w, size_t elem_size) {
     StreamPlan sp{};
-    const RowConfig rc = row_config(std::max(w, 1));
+    const RowConfig rc = stream_row_config(std::max(w, 1));
     sp.usable = w <= kMaxRowStreamWidth && !force_gather_kernels() &&
                 stream_lds_bytes(rc.K, rc.nt, elem_size) <= kMaxDynamicLds;
     int nb = bands_for(std::max<int64_t>(planes_f, 1), h, 32, 2048);
@@ -1059,14 +1171,14 @@ hipError_t grad_output_stream_launch(const T* integ, const T* grad_out, BoxParam
     a.src = integ; a.grad_out = grad_out; a.acc = acc; a.dst = local_integral;
     a.nb = sp.nb; a.R = sp.R;
     finish_args(a, planes_f * a.nb);
-    const RowConfig rc = row_config(d.w);
+    const RowConfig rc = stream_row_config(d.w);
     const dim3 grid(static_cast<unsigned>(a.per_xcd * kXcds));
     const size_t lds = stream_lds_bytes(rc.K, rc.nt, sizeof(T));
-#define LAUNCH_GS(KK, EX, FU) \
-    if (params && scan) BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_kernel<T, KK, EX, FU, true, true>), grid, dim3(rc.nt), lds, stream, a); \
-    else if (params)    BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_kernel<T, KK, EX, FU, true, false>), grid, dim3(rc.nt), lds, stream, a); \
-    else                BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_kernel<T, KK, EX, FU, false, true>), grid, dim3(rc.nt), lds, stream, a)
-    BOXCONV_DISPATCH_K_EXACT_FULL(LAUNCH_GS, rc.K, exact, rc.full)
+#define LAUNCH_GS(NT, KK, EX, FU) \
+    if (params && scan) BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_kernel<T, NT, KK, EX, FU, true, true>), grid, dim3(NT), lds, stream, a); \
+    else if (params)    BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_kernel<T, NT, KK, EX, FU, true, false>), grid, dim3(NT), lds, stream, a); \
+    else                BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_kernel<T, NT, KK, EX, FU, false, true>), grid, dim3(NT), lds, stream, a)
+    BOXCONV_DISPATCH_SHAPE_EXACT_FULL(LAUNCH_GS, rc, exact)
 #undef LAUNCH_GS
     return hipGetLastError();
 }

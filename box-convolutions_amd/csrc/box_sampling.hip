@@ -87,122 +87,134 @@ __device__ __forceinline__ P* at_bytes(P* base, unsigned bytes) {
     return reinterpret_cast<P*>(reinterpret_cast<Byte*>(base) + bytes);
 }
 
-// One row of T in global memory addressed as a raw buffer: scalar descriptor (base, size in
-// bytes) plus one 32-bit VGPR byte offset per access, so no per-lane 64-bit address arithmetic.
-// The hardware checks the offset against the size: a load at or beyond `bytes` returns 0 and a
-// store there is dropped, which also masks column slots past the end of a row and whole rows
-// (bytes = 0) without branches. `row` must be wave-uniform.
+// Global memory is reached through raw buffer instructions: a scalar descriptor (base, size in
+// bytes), a scalar byte offset and one 32-bit VGPR byte offset per access, so there is no
+// per-lane 64-bit address arithmetic. The hardware checks the VGPR offset against the size: a
+// load at or beyond it returns 0 and a store there is dropped.
 constexpr int kCacheDefault = 0, kCacheStream = 2;   // buffer cache policy bits: 2 = non-temporal
 template <class T>
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t row_buffer(const T* row, unsigned bytes) {
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(row), 0, static_cast<int>(bytes), 0x00020000);
-}
-template <int POLICY>
-__device__ __forceinline__ float buffer_load(__amdgpu_buffer_rsrc_t rs, unsigned off, float) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs, off, 0, POLICY));
-}
-template <int POLICY>
-__device__ __forceinline__ double buffer_load(__amdgpu_buffer_rsrc_t rs, unsigned off, double) {
-    return __builtin_bit_cast(double, __builtin_amdgcn_raw_buffer_load_b64(rs, off, 0, POLICY));
-}
-template <int POLICY>
-__device__ __forceinline__ void buffer_store(float v, __amdgpu_buffer_rsrc_t rs, unsigned off) {
-    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), rs, off, 0, POLICY);
-}
-template <int POLICY>
-__device__ __forceinline__ void buffer_store(double v, __amdgpu_buffer_rsrc_t rs, unsigned off) {
-    typedef unsigned v2u __attribute__((__vector_size__(8)));
-    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u, v), rs, off, 0, POLICY);
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const T* base, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(base), 0, static_cast<int>(bytes), 0x00020000);
 }
 
-// K consecutive elements per lane. WHOLE: the run lies inside the buffer for every lane, so it
+// One row of a stack of rows: descriptor plus scalar offset. Must be wave-uniform.
+struct RowRef {
+    __amdgpu_buffer_rsrc_t rs;
+    int soff;
+};
+
+// A stack of equally long rows of T in global memory (`cols` elements of each row reachable,
+// rows `pitch` elements apart, the whole stack below 4 GiB).
+//   BY_OFFSET: one descriptor spans the stack and a row is selected by its scalar byte offset.
+//              Only for stacks where every column slot of every lane is a valid column (there
+//              is no per-row bounds check). Measured: good for stores, slower than per-row
+//              descriptors for loads, so loads never use it.
+//   else     : one descriptor per row, sized to the row, so that the bounds check masks the
+//              column slots past its end.
+// A row that does not `exist` gets size 0: loads give 0, stores vanish, no branch needed.
+template <class T, bool BY_OFFSET>
+struct Rows {
+    T* base;
+    unsigned pitch_bytes, row_bytes, stack_bytes;
+    __device__ __forceinline__ Rows(T* base_, int64_t pitch, int cols, int nrows)
+        : base(base_), pitch_bytes(static_cast<unsigned>(pitch * sizeof(T))),
+          row_bytes(static_cast<unsigned>(cols) * static_cast<unsigned>(sizeof(T))),
+          stack_bytes(static_cast<unsigned>(nrows - 1) * pitch_bytes + row_bytes) {}
+    __device__ __forceinline__ RowRef row(int r, bool exists = true) const {
+        const unsigned offset = static_cast<unsigned>(r) * pitch_bytes;
+        if constexpr (BY_OFFSET)
+            return {make_buffer(base, exists ? stack_bytes : 0u), static_cast<int>(offset)};
+        else
+            return {make_buffer(at_bytes(base, offset), exists ? row_bytes : 0u), 0};
+    }
+};
+template <class T> using LoadRows = Rows<const T, false>;
+
+template <int POLICY>
+__device__ __forceinline__ float buffer_load(const RowRef& r, int off, float) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r.rs, off, r.soff, POLICY));
+}
+template <int POLICY>
+__device__ __forceinline__ double buffer_load(const RowRef& r, int off, double) {
+    return __builtin_bit_cast(double, __builtin_amdgcn_raw_buffer_load_b64(r.rs, off, r.soff, POLICY));
+}
+template <int POLICY>
+__device__ __forceinline__ void buffer_store(float v, const RowRef& r, int off) {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r.rs, off, r.soff, POLICY);
+}
+template <int POLICY>
+__device__ __forceinline__ void buffer_store(double v, const RowRef& r, int off) {
+    typedef unsigned v2u __attribute__((__vector_size__(8)));
+    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u, v), r.rs, off, r.soff, POLICY);
+}
+
+// K consecutive elements per lane. WHOLE: the run lies inside the row for every lane, so it
 // goes out as 16-byte pieces; otherwise element by element, each checked against the size.
 template <int POLICY, bool WHOLE, int K>
-__device__ __forceinline__ void buffer_store_run(const float (&v)[K], __amdgpu_buffer_rsrc_t rs, unsigned off) {
+__device__ __forceinline__ void buffer_store_run(const float (&v)[K], const RowRef& r, int off) {
     typedef unsigned v4u __attribute__((__vector_size__(16)));
     if constexpr (WHOLE && K % 4 == 0) {
 #pragma unroll
         for (int k = 0; k < K; k += 4) {
             const v4u pack = {__builtin_bit_cast(unsigned, v[k]), __builtin_bit_cast(unsigned, v[k + 1]),
                               __builtin_bit_cast(unsigned, v[k + 2]), __builtin_bit_cast(unsigned, v[k + 3])};
-            __builtin_amdgcn_raw_buffer_store_b128(pack, rs, off + 4u * k, 0, POLICY);
+            __builtin_amdgcn_raw_buffer_store_b128(pack, r.rs, off + 4 * k, r.soff, POLICY);
         }
     } else {
 #pragma unroll
-        for (int k = 0; k < K; ++k) buffer_store<POLICY>(v[k], rs, off + 4u * k);
+        for (int k = 0; k < K; ++k) buffer_store<POLICY>(v[k], r, off + 4 * k);
     }
 }
 template <int POLICY, bool WHOLE, int K>
-__device__ __forceinline__ void buffer_store_run(const double (&v)[K], __amdgpu_buffer_rsrc_t rs, unsigned off) {
+__device__ __forceinline__ void buffer_store_run(const double (&v)[K], const RowRef& r, int off) {
 #pragma unroll
-    for (int k = 0; k < K; ++k) buffer_store<POLICY>(v[k], rs, off + 8u * k);
+    for (int k = 0; k < K; ++k) buffer_store<POLICY>(v[k], r, off + 8 * k);
 }
 
 // Per-lane column slots. Lane `tid` owns integral columns q = 1 + tid + NT*k (pixel columns
 // j = q - 1), k < K, NT = workgroup size. q1 = (1 + tid) * sizeof(T) is the byte offset of the
 // lane's first column in a row of T; the other slots are compile-time distances away, so one
-// register addresses all of them (instruction offsets for LDS, scalar offsets for buffers).
+// register addresses all of them (instruction offsets for LDS and for buffers).
 // FULL: w == K * NT, so every (lane, k) slot is a valid column and no bounds checks are compiled
 // in; otherwise a slot is valid iff its byte offset is <= w * sizeof(T).
 template <class T>
-__device__ __forceinline__ unsigned lane_q1() {
-    return (1u + threadIdx.x) * static_cast<unsigned>(sizeof(T));
+__device__ __forceinline__ int lane_q1() {
+    return (1 + static_cast<int>(threadIdx.x)) * static_cast<int>(sizeof(T));
 }
 template <class T, int NT>
-__device__ __forceinline__ constexpr unsigned slot_bytes(int k) {
-    return static_cast<unsigned>(NT) * static_cast<unsigned>(k) * static_cast<unsigned>(sizeof(T));
+__device__ __forceinline__ constexpr int slot_bytes(int k) {
+    return NT * k * static_cast<int>(sizeof(T));
 }
 template <class T, int NT, bool FULL>
-__device__ __forceinline__ bool slot_valid(unsigned q1, int k, unsigned row_bytes) {
-    return FULL || q1 + slot_bytes<T, NT>(k) <= row_bytes;
+__device__ __forceinline__ bool slot_valid(int q1, int k, unsigned row_bytes) {
+    return FULL || static_cast<unsigned>(q1 + slot_bytes<T, NT>(k)) <= row_bytes;
 }
-// Slot k of a row buffer. With FULL the slot distance rides in the scalar offset; otherwise it
-// is part of the checked per-lane offset, so slots past the end of the row read 0 / are dropped.
-template <class T, int NT, bool FULL, int POLICY>
-__device__ __forceinline__ T load_slot(__amdgpu_buffer_rsrc_t rs, unsigned q1, int k) {
-    if constexpr (FULL) {
-        if constexpr (sizeof(T) == 4)
-            return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b32(rs, q1, slot_bytes<T, NT>(k), POLICY));
-        else
-            return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b64(rs, q1, slot_bytes<T, NT>(k), POLICY));
-    } else {
-        return buffer_load<POLICY>(rs, q1 + slot_bytes<T, NT>(k), T());
-    }
+template <class T, int NT, int POLICY>
+__device__ __forceinline__ T load_slot(const RowRef& r, int q1, int k) {
+    return buffer_load<POLICY>(r, q1 + slot_bytes<T, NT>(k), T());
 }
-template <class T, int NT, bool FULL, int POLICY>
-__device__ __forceinline__ void store_slot(T v, __amdgpu_buffer_rsrc_t rs, unsigned q1, int k) {
-    if constexpr (FULL) {
-        if constexpr (sizeof(T) == 4) {
-            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), rs, q1, slot_bytes<T, NT>(k), POLICY);
-        } else {
-            typedef unsigned v2u __attribute__((__vector_size__(8)));
-            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u, v), rs, q1, slot_bytes<T, NT>(k), POLICY);
-        }
-    } else {
-        buffer_store<POLICY>(v, rs, q1 + slot_bytes<T, NT>(k));
-    }
+template <class T, int NT, int POLICY>
+__device__ __forceinline__ void store_slot(T v, const RowRef& r, int q1, int k) {
+    buffer_store<POLICY>(v, r, q1 + slot_bytes<T, NT>(k));
 }
 
-template <class T, int NT, int K, bool FULL>
-__device__ __forceinline__ void load_row(const T* __restrict__ plane, int64_t pitch, int row,
-                                         unsigned row_bytes, unsigned q1, T (&dst)[K]) {
-    // columns 0..w of the row; slots beyond w read 0
-    const __amdgpu_buffer_rsrc_t rs = row_buffer(plane + static_cast<int64_t>(row) * pitch,
-                                                 row_bytes + static_cast<unsigned>(sizeof(T)));
+// Columns 1.. of one row into the lane's slots; slots past the end of the row read 0.
+template <class T, int NT, int K>
+__device__ __forceinline__ void load_row(const RowRef& r, int q1, T (&dst)[K]) {
 #pragma unroll
-    for (int k = 0; k < K; ++k) dst[k] = load_slot<T, NT, FULL, kCacheDefault>(rs, q1, k);
+    for (int k = 0; k < K; ++k) dst[k] = load_slot<T, NT, kCacheDefault>(r, q1, k);
 }
 
 // The four rows that become new when the window moves from output rows (i-2, i-1) to (i, i+1):
 // I[t(i)], I[t(i+1)], I[b(i+1)], I[b(i+2)].
 template <class T, int NT, int K, bool FULL>
-__device__ __forceinline__ void load_pair(const T* __restrict__ plane, int64_t pitch, int i,
-                                          int xlo, int xhi, int h, unsigned row_bytes, unsigned q1,
-                                          T (&t0)[K], T (&t1)[K], T (&b1)[K], T (&b2)[K]) {
-    load_row<T, NT, K, FULL>(plane, pitch, clampi(i + xlo, 0, h), row_bytes, q1, t0);
-    load_row<T, NT, K, FULL>(plane, pitch, clampi(i + 1 + xlo, 0, h), row_bytes, q1, t1);
-    load_row<T, NT, K, FULL>(plane, pitch, clampi(i + 1 + xhi, 0, h), row_bytes, q1, b1);
-    load_row<T, NT, K, FULL>(plane, pitch, clampi(i + 2 + xhi, 0, h), row_bytes, q1, b2);
+__device__ __forceinline__ void load_pair(const LoadRows<T>& rows, int i, int xlo, int xhi,
+                                          int h, int q1, T (&t0)[K], T (&t1)[K], T (&b1)[K],
+                                          T (&b2)[K]) {
+    load_row<T, NT, K>(rows.row(clampi(i + xlo, 0, h)), q1, t0);
+    load_row<T, NT, K>(rows.row(clampi(i + 1 + xlo, 0, h)), q1, t1);
+    load_row<T, NT, K>(rows.row(clampi(i + 1 + xhi, 0, h)), q1, b1);
+    load_row<T, NT, K>(rows.row(clampi(i + 2 + xhi, 0, h)), q1, b2);
 }
 
 template <class T, bool EXACT>
@@ -217,13 +229,13 @@ __device__ __forceinline__ T blend(T lo_adv, T lo, T hi, T hi_adv, T flo, T fhi)
 // entries.
 template <class T, int NT, int K, bool FULL>
 __device__ __forceinline__ void publish_rows(RowPair<T>* __restrict__ V, const T (&v0)[K],
-                                             const T (&v1)[K], int w, unsigned row_bytes, unsigned q1) {
+                                             const T (&v1)[K], int w, unsigned row_bytes, int q1) {
 #pragma unroll
     for (int k = 0; k < K; ++k) {
         const RowPair<T> pr{v0[k], v1[k]};
         if (slot_valid<T, NT, FULL>(q1, k, row_bytes)) *at_bytes(V + 1 + NT * k, 2 * q1) = pr;
         if (FULL ? (k == K - 1 && static_cast<int>(threadIdx.x) == NT - 1)
-                 : (q1 + slot_bytes<T, NT>(k) == row_bytes))
+                 : (static_cast<unsigned>(q1 + slot_bytes<T, NT>(k)) == row_bytes))
             V[w + 2] = pr;
     }
 }
@@ -292,7 +304,9 @@ __global__ void __launch_bounds__(NT) forward_rows_kernel(SampleArgs<T> a) {
 
     const int64_t pitch = w + 1;
     const T* plane = a.src + p * static_cast<int64_t>(h + 1) * pitch;
-    T* out = a.dst + pf * static_cast<int64_t>(h) * w;
+    // output rows start one element early so that column slot q = j + 1 lands on pixel j
+    const LoadRows<T> irows(plane, pitch, w + 1, h + 1);
+    const Rows<T, FULL> orows(a.dst + pf * static_cast<int64_t>(h) * w - 1, w, w + 1, h);
     RowPair<T>* vbuf = reinterpret_cast<RowPair<T>*>(smem_raw);
     const int vlen = w + 3;
     clear_row_pads(vbuf, vlen);
@@ -300,15 +314,15 @@ __global__ void __launch_bounds__(NT) forward_rows_kernel(SampleArgs<T> a) {
     const int i0 = band * a.R;
     const int i1 = min(h, i0 + a.R);
 
-    const unsigned q1 = lane_q1<T>();
+    const int q1 = lane_q1<T>();
     unsigned lo[K], hi[K];
     column_taps<T, NT, K>(lo, hi, s.ylo, s.yhi, w);
 
     T ta[K], bc[K];                       // I[t(i-1)], I[b(i)]
     T t0[K], t1[K], b1[K], b2[K];         // I[t(i)], I[t(i+1)], I[b(i+1)], I[b(i+2)]
-    load_row<T, NT, K, FULL>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), row_bytes, q1, ta);
-    load_row<T, NT, K, FULL>(plane, pitch, clampi(i0 + s.xhi, 0, h), row_bytes, q1, bc);
-    load_pair<T, NT, K, FULL>(plane, pitch, i0, s.xlo, s.xhi, h, row_bytes, q1, t0, t1, b1, b2);
+    load_row<T, NT, K>(irows.row(clampi(i0 + s.xlo - 1, 0, h)), q1, ta);
+    load_row<T, NT, K>(irows.row(clampi(i0 + s.xhi, 0, h)), q1, bc);
+    load_pair<T, NT, K, FULL>(irows, i0, s.xlo, s.xhi, h, q1, t0, t1, b1, b2);
 
     // One row pair. PREFETCH and the LDS buffer are compile-time tags: the loop body always
     // issues the next pair's loads and the last pair is peeled, so no branch joins a path with
@@ -320,7 +334,7 @@ __global__ void __launch_bounds__(NT) forward_rows_kernel(SampleArgs<T> a) {
         constexpr int FLIP = decltype(flip_tag)::value;
         T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {};
         if (PREFETCH)
-            load_pair<T, NT, K, FULL>(plane, pitch, i + 2, s.xlo, s.xhi, h, row_bytes, q1, n0, n1, n2, n3);
+            load_pair<T, NT, K, FULL>(irows, i + 2, s.xlo, s.xhi, h, q1, n0, n1, n2, n3);
 
         RowPair<T>* V = vbuf + (FLIP ? vlen : 0);
         T v0[K], v1[K];
@@ -332,17 +346,14 @@ __global__ void __launch_bounds__(NT) forward_rows_kernel(SampleArgs<T> a) {
         publish_rows<T, NT, K, FULL>(V, v0, v1, w, row_bytes, q1);
         __syncthreads();
 
-        // column q = j + 1 lands on pixel j; the second row may lie past the band (size 0)
-        T* orow = out + static_cast<int64_t>(i) * w - 1;
-        const unsigned out_bytes = row_bytes + static_cast<unsigned>(sizeof(T));
-        const __amdgpu_buffer_rsrc_t ob0 = row_buffer(orow, out_bytes);
-        const __amdgpu_buffer_rsrc_t ob1 = row_buffer(orow + w, i + 1 < i1 ? out_bytes : 0u);
+        const RowRef ob0 = orows.row(i);
+        const RowRef ob1 = orows.row(min(i + 1, h - 1), i + 1 < i1);   // may lie past the band
 #pragma unroll
         for (int k = 0; k < K; ++k) {
             if (slot_valid<T, NT, FULL>(q1, k, row_bytes)) {
                 const RowPair<T> o = sample_columns<T, EXACT>(V, lo[k], hi[k], s.fylo, s.fyhi);
-                store_slot<T, NT, FULL, kCacheStream>(o.r0 * scale, ob0, q1, k);
-                store_slot<T, NT, FULL, kCacheStream>(o.r1 * scale, ob1, q1, k);
+                store_slot<T, NT, kCacheStream>(o.r0 * scale, ob0, q1, k);
+                store_slot<T, NT, kCacheStream>(o.r1 * scale, ob1, q1, k);
             }
         }
         if (PREFETCH) {
@@ -391,7 +402,7 @@ __global__ void __launch_bounds__(NT) grad_input_rows_kernel(SampleArgs<T> a) {
     clear_row_pads(vbuf, vlen);
     const int i0 = band * RB;
 
-    const unsigned q1 = lane_q1<T>();
+    const int q1 = lane_q1<T>();
 
     T acc[RB][K];
 #pragma unroll
@@ -404,105 +415,138 @@ __global__ void __launch_bounds__(NT) grad_input_rows_kernel(SampleArgs<T> a) {
         const BoxSplit<T> s = split_grad_input(bx.xmin, bx.xmax, bx.ymin, bx.ymax);
         const T scale = a.normalize
             ? inverse_extent(bx.xmin, bx.xmax, bx.ymin, bx.ymax, EXACT, true, true) : T(1);
-        const T* plane = a.src + (p * a.F + f) * ipl;
+        const LoadRows<T> irows(a.src + (p * a.F + f) * ipl, pitch, w + 1, h + 1);
 
         unsigned lo[K], hi[K];
         column_taps<T, NT, K>(lo, hi, s.ylo, s.yhi, w);
 
-        // OFFS: `plane` holds a band-local integral (bands of off_R rows, each restarting at
+        // OFFS: the plane holds a band-local integral (bands of off_R rows, each restarting at
         // zero). Integral row r (1..h) belongs to band (r-1)/off_R; row 0 counts as band 0. The
         // true integral is the stored row plus the bottom rows of all bands above it; relative to
         // the reference band (that of the first row touched) only the bottom rows of the bands in
-        // between remain, summed in double. Rows only move down, so each side tracks the last row
-        // of its current band instead of dividing.
-        const int ref_band = OFFS ? max(clampi(i0 + s.xlo - 1, 0, h) - 1, 0) / a.off_R : 0;
-        int band_t = ref_band, band_b = ref_band;
-        int last_t = (ref_band + 1) * a.off_R, last_b = last_t;     // last row of the cached band
-        T off_t[K], off_b[K];
-#pragma unroll
-        for (int k = 0; k < K; ++k) { off_t[k] = T(0); off_b[k] = T(0); }
-        auto refresh = [&](int& cached_band, int& cached_last, int row_index, T (&cached)[K]) {
-            do { ++cached_band; cached_last += a.off_R; } while (row_index > cached_last);
+        // between remain, summed in double.
+        //   Usual case: the RB+2 top rows lie in one band and so do the RB+2 bottom rows. Then
+        //   the top rows need nothing, the bottom rows share one offset vector, and since V only
+        //   contains differences, that vector is added to V once.
+        //   Otherwise (CROSS) every loaded row is corrected on its own; rows only move down, so
+        //   each side tracks the last row of its current band instead of dividing.
+        const int first_t = clampi(i0 + s.xlo - 1, 0, h), final_t = clampi(i0 + RB - 1 + s.xlo, 0, h);
+        const int first_b = clampi(i0 + s.xhi, 0, h), final_b = clampi(i0 + RB + s.xhi, 0, h);
+        // reference band: that of the topmost row touched (a box given with min > max has its
+        // "bottom" rows above its "top" rows)
+        const int ref_band = OFFS ? max(min(first_t, first_b) - 1, 0) / a.off_R : 0;
+        const int ref_last = (ref_band + 1) * a.off_R;              // last row of the reference band
+        auto bottoms_between = [&](int from_band, int to_band, T (&dst)[K]) {
             double sum[K];
 #pragma unroll
             for (int k = 0; k < K; ++k) sum[k] = 0.0;
-            for (int b = ref_band; b < cached_band; ++b) {
+            for (int b = from_band; b < to_band; ++b) {
                 T bottom[K];
-                load_row<T, NT, K, FULL>(plane, pitch, min(h, (b + 1) * a.off_R), row_bytes, q1, bottom);
+                load_row<T, NT, K>(irows.row(min(h, (b + 1) * a.off_R)), q1, bottom);
 #pragma unroll
                 for (int k = 0; k < K; ++k) sum[k] += static_cast<double>(bottom[k]);
             }
 #pragma unroll
-            for (int k = 0; k < K; ++k) cached[k] = static_cast<T>(sum[k]);
+            for (int k = 0; k < K; ++k) dst[k] = static_cast<T>(sum[k]);
         };
-        auto correct = [&](T (&row)[K], int row_index, int& cached_band, int& cached_last, T (&cached)[K]) {
-            if (!OFFS) return;
-            if (row_index > cached_last)                    // uniform: depends on the row only
-                refresh(cached_band, cached_last, row_index, cached);
+        bool cross = false;
+        T off_b[K];                                 // usual case: offset of bottom minus top rows
 #pragma unroll
-            for (int k = 0; k < K; ++k) row[k] += cached[k];
-        };
-
-        T ta[K], bc[K], t0[K], t1[K], b1[K], b2[K];
-        load_row<T, NT, K, FULL>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), row_bytes, q1, ta);
-        load_row<T, NT, K, FULL>(plane, pitch, clampi(i0 + s.xhi, 0, h), row_bytes, q1, bc);
-        load_pair<T, NT, K, FULL>(plane, pitch, i0, s.xlo, s.xhi, h, row_bytes, q1, t0, t1, b1, b2);
-        correct(ta, clampi(i0 + s.xlo - 1, 0, h), band_t, last_t, off_t);
-        correct(t0, clampi(i0 + s.xlo, 0, h), band_t, last_t, off_t);
-        correct(t1, clampi(i0 + 1 + s.xlo, 0, h), band_t, last_t, off_t);
-        correct(bc, clampi(i0 + s.xhi, 0, h), band_b, last_b, off_b);
-        correct(b1, clampi(i0 + 1 + s.xhi, 0, h), band_b, last_b, off_b);
-        correct(b2, clampi(i0 + 2 + s.xhi, 0, h), band_b, last_b, off_b);
-
-        // All RB rows are always computed (rows past the image read clamped, valid rows and are
-        // not stored) and the prefetch of the next pair is decided at compile time: straight-line
-        // code, so loads stay in flight across the barrier.
+        for (int k = 0; k < K; ++k) off_b[k] = T(0);
+        if (OFFS) {
+            int band_t = ref_band, last_t = ref_last, band_b = ref_band, last_b = ref_last;
+            while (first_t > last_t) { ++band_t; last_t += a.off_R; }
+            while (first_b > last_b) { ++band_b; last_b += a.off_R; }
+            cross = final_t > last_t || final_b > last_b;
+            if (!cross && band_b > band_t) bottoms_between(band_t, band_b, off_b);
+            if (!cross && band_b < band_t) {
+                bottoms_between(band_b, band_t, off_b);
 #pragma unroll
-        for (int r = 0; r < RB; r += 2) {
-            const int i = i0 + r;
-            T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {};
-            const bool more = r + 2 < RB;                                // known after unrolling
-            if (more)
-                load_pair<T, NT, K, FULL>(plane, pitch, i + 2, s.xlo, s.xhi, h, row_bytes, q1, n0, n1, n2, n3);
-            RowPair<T>* V = vbuf + (((r >> 1) & 1) ? vlen : 0);
-            T v0[K], v1[K];
-#pragma unroll
-            for (int k = 0; k < K; ++k) {
-                v0[k] = blend<T, EXACT>(ta[k], t0[k], bc[k], b1[k], s.fxlo, s.fxhi);
-                v1[k] = blend<T, EXACT>(t0[k], t1[k], b1[k], b2[k], s.fxlo, s.fxhi);
-            }
-            publish_rows<T, NT, K, FULL>(V, v0, v1, w, row_bytes, q1);
-            __syncthreads();
-#pragma unroll
-            for (int k = 0; k < K; ++k) {
-                if (slot_valid<T, NT, FULL>(q1, k, row_bytes)) {
-                    const RowPair<T> o = sample_columns<T, EXACT>(V, lo[k], hi[k], s.fylo, s.fyhi);
-                    acc[r][k] += scale * o.r0;
-                    acc[r + 1][k] += scale * o.r1;
-                }
-            }
-            if (more) {
-#pragma unroll
-                for (int k = 0; k < K; ++k) {
-                    ta[k] = t1[k]; bc[k] = b2[k];
-                    t0[k] = n0[k]; t1[k] = n1[k]; b1[k] = n2[k]; b2[k] = n3[k];
-                }
-                correct(t0, clampi(i + 2 + s.xlo, 0, h), band_t, last_t, off_t);
-                correct(t1, clampi(i + 3 + s.xlo, 0, h), band_t, last_t, off_t);
-                correct(b1, clampi(i + 3 + s.xhi, 0, h), band_b, last_b, off_b);
-                correct(b2, clampi(i + 4 + s.xhi, 0, h), band_b, last_b, off_b);
+                for (int k = 0; k < K; ++k) off_b[k] = -off_b[k];
             }
         }
+
+        auto pass = [&](auto cross_tag) {
+            constexpr bool CROSS = decltype(cross_tag)::value;
+            int band_t = ref_band, band_b = ref_band, last_t = ref_last, last_b = ref_last;
+            T off_t[K];
+#pragma unroll
+            for (int k = 0; k < K; ++k) off_t[k] = T(0);
+            auto correct = [&](T (&row)[K], int row_index, int& cached_band, int& cached_last, T (&cached)[K]) {
+                if constexpr (CROSS) {
+                    if (row_index > cached_last) {              // uniform: depends on the row only
+                        do { ++cached_band; cached_last += a.off_R; } while (row_index > cached_last);
+                        bottoms_between(ref_band, cached_band, cached);
+                    }
+#pragma unroll
+                    for (int k = 0; k < K; ++k) row[k] += cached[k];
+                }
+            };
+
+            T ta[K], bc[K], t0[K], t1[K], b1[K], b2[K];
+            load_row<T, NT, K>(irows.row(first_t), q1, ta);
+            load_row<T, NT, K>(irows.row(first_b), q1, bc);
+            load_pair<T, NT, K, FULL>(irows, i0, s.xlo, s.xhi, h, q1, t0, t1, b1, b2);
+            correct(ta, first_t, band_t, last_t, off_t);
+            correct(t0, clampi(i0 + s.xlo, 0, h), band_t, last_t, off_t);
+            correct(t1, clampi(i0 + 1 + s.xlo, 0, h), band_t, last_t, off_t);
+            correct(bc, first_b, band_b, last_b, off_b);
+            correct(b1, clampi(i0 + 1 + s.xhi, 0, h), band_b, last_b, off_b);
+            correct(b2, clampi(i0 + 2 + s.xhi, 0, h), band_b, last_b, off_b);
+
+            // All RB rows are always computed (rows past the image read clamped, valid rows and
+            // are not stored) and the prefetch of the next pair is decided at compile time:
+            // straight-line code, so loads stay in flight across the barrier.
+#pragma unroll
+            for (int r = 0; r < RB; r += 2) {
+                const int i = i0 + r;
+                T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {};
+                const bool more = r + 2 < RB;                            // known after unrolling
+                if (more)
+                    load_pair<T, NT, K, FULL>(irows, i + 2, s.xlo, s.xhi, h, q1, n0, n1, n2, n3);
+                RowPair<T>* V = vbuf + (((r >> 1) & 1) ? vlen : 0);
+                T v0[K], v1[K];
+#pragma unroll
+                for (int k = 0; k < K; ++k) {
+                    v0[k] = blend<T, EXACT>(ta[k], t0[k], bc[k], b1[k], s.fxlo, s.fxhi);
+                    v1[k] = blend<T, EXACT>(t0[k], t1[k], b1[k], b2[k], s.fxlo, s.fxhi);
+                    if (OFFS && !CROSS) { v0[k] += off_b[k]; v1[k] += off_b[k]; }
+                }
+                publish_rows<T, NT, K, FULL>(V, v0, v1, w, row_bytes, q1);
+                __syncthreads();
+#pragma unroll
+                for (int k = 0; k < K; ++k) {
+                    if (slot_valid<T, NT, FULL>(q1, k, row_bytes)) {
+                        const RowPair<T> o = sample_columns<T, EXACT>(V, lo[k], hi[k], s.fylo, s.fyhi);
+                        acc[r][k] += scale * o.r0;
+                        acc[r + 1][k] += scale * o.r1;
+                    }
+                }
+                if (more) {
+#pragma unroll
+                    for (int k = 0; k < K; ++k) {
+                        ta[k] = t1[k]; bc[k] = b2[k];
+                        t0[k] = n0[k]; t1[k] = n1[k]; b1[k] = n2[k]; b2[k] = n3[k];
+                    }
+                    correct(t0, clampi(i + 2 + s.xlo, 0, h), band_t, last_t, off_t);
+                    correct(t1, clampi(i + 3 + s.xlo, 0, h), band_t, last_t, off_t);
+                    correct(b1, clampi(i + 3 + s.xhi, 0, h), band_b, last_b, off_b);
+                    correct(b2, clampi(i + 4 + s.xhi, 0, h), band_b, last_b, off_b);
+                }
+            }
+        };
+        if (OFFS && cross) pass(std::true_type{});
+        else pass(std::false_type{});
     }
 
-    T* out = a.dst + p * static_cast<int64_t>(h) * w - 1;    // column q = j + 1 lands on pixel j
+    // column slot q = j + 1 lands on pixel j; rows past the image get size 0
+    const Rows<T, FULL> orows(a.dst + p * static_cast<int64_t>(h) * w - 1, w, w + 1, h);
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
-        const int i = i0 + r;                                // rows past the image: size 0
-        const __amdgpu_buffer_rsrc_t ob = row_buffer(out + static_cast<int64_t>(min(i, h - 1)) * w,
-                                                     i < h ? row_bytes + static_cast<unsigned>(sizeof(T)) : 0u);
+        const int i = i0 + r;
+        const RowRef ob = orows.row(min(i, h - 1), i < h);
 #pragma unroll
-        for (int k = 0; k < K; ++k) store_slot<T, NT, FULL, kCacheDefault>(acc[r][k], ob, q1, k);
+        for (int k = 0; k < K; ++k) store_slot<T, NT, kCacheDefault>(acc[r][k], ob, q1, k);
     }
 }
 
@@ -614,9 +658,12 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
     const BoxSplit<T> s = split_grad_params(bx.xmin, bx.xmax, bx.ymin, bx.ymax);
 
     const int64_t pitch = w + 1;
-    const T* plane = a.src + p * static_cast<int64_t>(h + 1) * pitch;          // integral of input
-    const T* gout = a.grad_out + pf * static_cast<int64_t>(h) * w;
-    T* lrows = SCAN ? a.dst + pf * static_cast<int64_t>(h + 1) * pitch : nullptr; // band-local integral
+    // integral of the input; grad_output (one element early: column slot q = j + 1 is pixel j);
+    // band-local integral of grad_output
+    const LoadRows<T> irows(a.src + p * static_cast<int64_t>(h + 1) * pitch, pitch, w + 1, h + 1);
+    const LoadRows<T> grows(a.grad_out + pf * static_cast<int64_t>(h) * w - 1, w, w + 1, h);
+    T* lrows = SCAN ? a.dst + pf * static_cast<int64_t>(h + 1) * pitch : nullptr;
+    const Rows<T, FULL> lout(lrows, pitch, w + 1, h + 1);
     const StreamLds<T> lds = carve_stream_lds<T>(K, nt);
     const int glen = lds.glen;
 
@@ -629,7 +676,7 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
         for (int c = tid; c <= w; c += nt) lrows[c] = T(0);                    // integral row 0
     __syncthreads();
 
-    const unsigned q1 = lane_q1<T>();
+    const int q1 = lane_q1<T>();
 
     // lane-constant LDS byte offsets of the pairs (grA, gr) and (gl, glA); the tail weights of the
     // lane's columns go to LDS (read back once per row pair: cheaper than K live registers)
@@ -664,16 +711,14 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
 
     T ta[K], bc[K], t0[K], t1[K], b1[K], b2[K], g0[K], g1[K];
     if (PARAMS) {
-        load_row<T, NT, K, FULL>(plane, pitch, clampi(i0 + s.xlo - 1, 0, h), row_bytes, q1, ta);
-        load_row<T, NT, K, FULL>(plane, pitch, clampi(i0 + s.xhi, 0, h), row_bytes, q1, bc);
-        load_pair<T, NT, K, FULL>(plane, pitch, i0, s.xlo, s.xhi, h, row_bytes, q1, t0, t1, b1, b2);
+        load_row<T, NT, K>(irows.row(clampi(i0 + s.xlo - 1, 0, h)), q1, ta);
+        load_row<T, NT, K>(irows.row(clampi(i0 + s.xhi, 0, h)), q1, bc);
+        load_pair<T, NT, K, FULL>(irows, i0, s.xlo, s.xhi, h, q1, t0, t1, b1, b2);
     }
     auto load_g = [&](int i, T (&dst)[K]) {
-        // column q = j + 1 -> pixel j; rows past the band read as zeros (size 0)
-        const __amdgpu_buffer_rsrc_t rs = row_buffer(gout + static_cast<int64_t>(min(i, h - 1)) * w - 1,
-                                                     i < i1 ? row_bytes + static_cast<unsigned>(sizeof(T)) : 0u);
+        const RowRef r = grows.row(min(i, h - 1), i < i1);     // rows past the band read as zeros
 #pragma unroll
-        for (int k = 0; k < K; ++k) dst[k] = load_slot<T, NT, FULL, kCacheStream>(rs, q1, k);
+        for (int k = 0; k < K; ++k) dst[k] = load_slot<T, NT, kCacheStream>(r, q1, k);
     };
     load_g(i0, g0);
     load_g(i0 + 1, g1);
@@ -690,7 +735,7 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
         T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {}, m0[K] = {}, m1[K] = {};
         if (PREFETCH) {
             if (PARAMS)
-                load_pair<T, NT, K, FULL>(plane, pitch, i + 2, s.xlo, s.xhi, h, row_bytes, q1, n0, n1, n2, n3);
+                load_pair<T, NT, K, FULL>(irows, i + 2, s.xlo, s.xhi, h, q1, n0, n1, n2, n3);
             load_g(i + 2, m0);
             load_g(i + 3, m1);
         }
@@ -803,13 +848,12 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
                 // a wave stores one contiguous run of 64*K elements per row
                 T* o0 = lrows + static_cast<int64_t>(i + 1) * pitch;
                 const bool second = i + 1 < i1;
-                const unsigned out_bytes = row_bytes + static_cast<unsigned>(sizeof(T));
-                const __amdgpu_buffer_rsrc_t ob0 = row_buffer(o0, out_bytes);
-                const __amdgpu_buffer_rsrc_t ob1 = row_buffer(o0 + pitch, second ? out_bytes : 0u);
+                const RowRef ob0 = lout.row(i + 1);
+                const RowRef ob1 = lout.row(min(i + 2, h), second);
                 T out0[K], out1[K];
 #pragma unroll
                 for (int k = 0; k < K; ++k) { out0[k] = carry0 + loc0[k]; out1[k] = carry1 + loc1[k]; }
-                const unsigned first = static_cast<unsigned>(1 + K * tid) * static_cast<unsigned>(sizeof(T));
+                const int first = (1 + K * tid) * static_cast<int>(sizeof(T));
                 buffer_store_run<kCacheStream, FULL>(out0, ob0, first);
                 buffer_store_run<kCacheStream, FULL>(out1, ob1, first);
                 if (tid == 0) {
@@ -1029,6 +1073,12 @@ inline RowConfig row_config(int w, int prefer) {
     return c;
 }
 
+// The row kernels address a plane with 32-bit byte offsets and hold a full row per workgroup.
+inline bool row_kernels_apply(int h, int w, size_t elem_size) {
+    const uint64_t plane_bytes = (static_cast<uint64_t>(h) + 1) * (static_cast<uint64_t>(w) + 1) * elem_size;
+    return w <= kMaxRowStreamWidth && plane_bytes < (1ull << 31) && !force_gather_kernels();
+}
+
 inline RowConfig stream_row_config(int w) {
     static const int prefer = preferred_row_threads("BOXCONV_STREAM_THREADS", 256);
     return row_config(w, prefer);
@@ -1082,7 +1132,7 @@ hipError_t forward_launch(const T* integ, BoxParams<T> prm, T* out, Dims d, bool
     SampleArgs<T> a = base_args(prm, d);
     a.src = integ; a.dst = out; a.normalize = normalize ? 1 : 0;
 
-    if (d.w > kMaxRowStreamWidth || force_gather_kernels()) {
+    if (!row_kernels_apply(d.h, d.w, sizeof(T))) {
         finish_args(a, planes_f * d.hw());
         const dim3 grid(static_cast<unsigned>((a.total + 255) / 256));
         if (exact) BOXCONV_LAUNCH("forward_gather", (forward_gather_kernel<T, true>), grid, dim3(256), 0, stream, a);
@@ -1114,7 +1164,7 @@ hipError_t grad_input_launch(const T* gint, int band_rows, BoxParams<T> prm, T* 
     a.src = gint; a.dst = grad_in; a.normalize = normalize ? 1 : 0;
     a.off_R = band_rows;
 
-    if (d.w > kMaxRowStreamWidth || force_gather_kernels()) {
+    if (!row_kernels_apply(d.h, d.w, sizeof(T))) {
         if (band_rows > 0) return hipErrorInvalidValue;         // the gather kernel needs a true integral
         finish_args(a, d.planes * d.hw());
         const dim3 grid(static_cast<unsigned>((a.total + 255) / 256));
@@ -1149,7 +1199,7 @@ hipError_t grad_params_begin(double* acc, int n_boxes, hipStream_t stream) {
 StreamPlan plan_grad_output_stream(int64_t planes_f, int h, int w, size_t elem_size) {
     StreamPlan sp{};
     const RowConfig rc = stream_row_config(std::max(w, 1));
-    sp.usable = w <= kMaxRowStreamWidth && !force_gather_kernels() &&
+    sp.usable = row_kernels_apply(h, w, elem_size) &&
                 stream_lds_bytes(rc.K, rc.nt, elem_size) <= kMaxDynamicLds;
     int nb = bands_for(std::max<int64_t>(planes_f, 1), h, 32, 2048);
     int R = (h + nb - 1) / nb;

@@ -137,6 +137,26 @@ def test_forward_backward_small(hip, oracle, B, C, F, h, w, kind, dtype):
             assert_parity(cpu, gpu, dtype, "%s normalize=%s exact=%s" % (kind, normalize, exact), **sc)
 
 
+@pytest.mark.parametrize("kind", ["inside", "hanging", "inverted"])
+@pytest.mark.parametrize("h,w", [(150, 90), (257, 256), (97, 520)])
+def test_backward_across_row_bands(hip, oracle, h, w, kind):
+    """Images tall enough that the backward pass cuts grad_output into several row bands, with
+    boxes whose top and bottom rows fall into different bands; 'inverted' boxes have min > max
+    along the rows (their bottom rows lie above their top rows)."""
+    rng = np.random.default_rng(h * 1000 + w + len(kind))
+    B, C, F = 1, 2, 3
+    x = rng.standard_normal((B, C, h, w)).astype(np.float32)
+    g = (rng.standard_normal((B, C * F, h, w)) + 0.5).astype(np.float32)
+    boxes = list(make_boxes(rng, C, F, h, w, "hanging" if kind == "inverted" else kind,
+                            away_from_integers=0.05))
+    if kind == "inverted":
+        lo = rng.uniform(-0.6 * h, 0.6 * h, (C, F))
+        boxes[0] = lo.astype(np.float32)                                  # x_min
+        boxes[1] = (lo - rng.uniform(3.3, 0.5 * h, (C, F))).astype(np.float32)   # x_max < x_min
+    cpu, gpu, sc = run_both(hip, oracle, x, tuple(boxes), 3.5 * h, 2.25 * w, False, True, g)
+    assert_parity(cpu, gpu, np.float32, "%s %dx%d" % (kind, h, w), **sc)
+
+
 def test_unit_box_is_identity(hip):
     x = torch.randn(2, 3, 13, 31, device="cuda")
     z = torch.zeros(3, 2, device="cuda")

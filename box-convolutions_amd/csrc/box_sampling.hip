@@ -79,98 +79,6 @@ struct alignas(2 * sizeof(T)) RowPair {
     T r0, r1;
 };
 
-// Pointer plus a byte offset held in a 32-bit register. Global accesses written this way use a
-// scalar base and one VGPR offset, LDS accesses an immediate base; no per-access address math.
-template <class P>
-__device__ __forceinline__ P* at_bytes(P* base, unsigned bytes) {
-    using Byte = std::conditional_t<std::is_const<P>::value, const char, char>;
-    return reinterpret_cast<P*>(reinterpret_cast<Byte*>(base) + bytes);
-}
-
-// Global memory is reached through raw buffer instructions: a scalar descriptor (base, size in
-// bytes), a scalar byte offset and one 32-bit VGPR byte offset per access, so there is no
-// per-lane 64-bit address arithmetic. The hardware checks the VGPR offset against the size: a
-// load at or beyond it returns 0 and a store there is dropped.
-constexpr int kCacheDefault = 0, kCacheStream = 2;   // buffer cache policy bits: 2 = non-temporal
-template <class T>
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const T* base, unsigned bytes) {
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(base), 0, static_cast<int>(bytes), 0x00020000);
-}
-
-// One row of a stack of rows: descriptor plus scalar offset. Must be wave-uniform.
-struct RowRef {
-    __amdgpu_buffer_rsrc_t rs;
-    int soff;
-};
-
-// A stack of equally long rows of T in global memory (`cols` elements of each row reachable,
-// rows `pitch` elements apart, the whole stack below 4 GiB).
-//   BY_OFFSET: one descriptor spans the stack and a row is selected by its scalar byte offset.
-//              Only for stacks where every column slot of every lane is a valid column (there
-//              is no per-row bounds check). Measured: good for stores, slower than per-row
-//              descriptors for loads, so loads never use it.
-//   else     : one descriptor per row, sized to the row, so that the bounds check masks the
-//              column slots past its end.
-// A row that does not `exist` gets size 0: loads give 0, stores vanish, no branch needed.
-template <class T, bool BY_OFFSET>
-struct Rows {
-    T* base;
-    unsigned pitch_bytes, row_bytes, stack_bytes;
-    __device__ __forceinline__ Rows(T* base_, int64_t pitch, int cols, int nrows)
-        : base(base_), pitch_bytes(static_cast<unsigned>(pitch * sizeof(T))),
-          row_bytes(static_cast<unsigned>(cols) * static_cast<unsigned>(sizeof(T))),
-          stack_bytes(static_cast<unsigned>(nrows - 1) * pitch_bytes + row_bytes) {}
-    __device__ __forceinline__ RowRef row(int r, bool exists = true) const {
-        const unsigned offset = static_cast<unsigned>(r) * pitch_bytes;
-        if constexpr (BY_OFFSET)
-            return {make_buffer(base, exists ? stack_bytes : 0u), static_cast<int>(offset)};
-        else
-            return {make_buffer(at_bytes(base, offset), exists ? row_bytes : 0u), 0};
-    }
-};
-template <class T> using LoadRows = Rows<const T, false>;
-
-template <int POLICY>
-__device__ __forceinline__ float buffer_load(const RowRef& r, int off, float) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r.rs, off, r.soff, POLICY));
-}
-template <int POLICY>
-__device__ __forceinline__ double buffer_load(const RowRef& r, int off, double) {
-    return __builtin_bit_cast(double, __builtin_amdgcn_raw_buffer_load_b64(r.rs, off, r.soff, POLICY));
-}
-template <int POLICY>
-__device__ __forceinline__ void buffer_store(float v, const RowRef& r, int off) {
-    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r.rs, off, r.soff, POLICY);
-}
-template <int POLICY>
-__device__ __forceinline__ void buffer_store(double v, const RowRef& r, int off) {
-    typedef unsigned v2u __attribute__((__vector_size__(8)));
-    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u, v), r.rs, off, r.soff, POLICY);
-}
-
-// K consecutive elements per lane. WHOLE: the run lies inside the row for every lane, so it
-// goes out as 16-byte pieces; otherwise element by element, each checked against the size.
-template <int POLICY, bool WHOLE, int K>
-__device__ __forceinline__ void buffer_store_run(const float (&v)[K], const RowRef& r, int off) {
-    typedef unsigned v4u __attribute__((__vector_size__(16)));
-    if constexpr (WHOLE && K % 4 == 0) {
-#pragma unroll
-        for (int k = 0; k < K; k += 4) {
-            const v4u pack = {__builtin_bit_cast(unsigned, v[k]), __builtin_bit_cast(unsigned, v[k + 1]),
-                              __builtin_bit_cast(unsigned, v[k + 2]), __builtin_bit_cast(unsigned, v[k + 3])};
-            __builtin_amdgcn_raw_buffer_store_b128(pack, r.rs, off + 4 * k, r.soff, POLICY);
-        }
-    } else {
-#pragma unroll
-        for (int k = 0; k < K; ++k) buffer_store<POLICY>(v[k], r, off + 4 * k);
-    }
-}
-template <int POLICY, bool WHOLE, int K>
-__device__ __forceinline__ void buffer_store_run(const double (&v)[K], const RowRef& r, int off) {
-#pragma unroll
-    for (int k = 0; k < K; ++k) buffer_store<POLICY>(v[k], r, off + 8 * k);
-}
-
 // Per-lane column slots. Lane `tid` owns integral columns q = 1 + tid + NT*k (pixel columns
 // j = q - 1), k < K, NT = workgroup size. q1 = (1 + tid) * sizeof(T) is the byte offset of the
 // lane's first column in a row of T; the other slots are compile-time distances away, so one
@@ -287,13 +195,14 @@ using Flip1 = std::integral_constant<int, 1>;
 // LDS: [2 buffers][w+3] RowPair<T>.
 template <class T, int NT, int K, bool EXACT, bool FULL>
 __global__ void __launch_bounds__(NT) forward_rows_kernel(SampleArgs<T> a) {
-    const int64_t vid = xcd_contiguous_id(a.per_xcd);
+    const unsigned vid = xcd_contiguous_id(a.per_xcd);
     if (vid >= a.total) return;
-    const int band = static_cast<int>(vid % a.nb);
-    const int64_t pf = vid / a.nb;
-    const int f = static_cast<int>(pf % a.F);
-    const int64_t p = pf / a.F;
-    const int k_par = static_cast<int>((a.plane0 + p) % a.C) * a.F + f;
+    const unsigned nbands = a.nb, nfilt = a.F;
+    const int band = static_cast<int>(vid % nbands);
+    const unsigned pf32 = vid / nbands;
+    const int f = static_cast<int>(pf32 % nfilt);
+    const int64_t pf = pf32, p = pf32 / nfilt;
+    const int k_par = static_cast<int>(static_cast<unsigned>(a.plane0 + p) % static_cast<unsigned>(a.C)) * a.F + f;
     const int h = a.h, w = a.w;
     const unsigned row_bytes = static_cast<unsigned>(w) * sizeof(T);
 
@@ -388,11 +297,12 @@ __global__ void __launch_bounds__(NT) forward_rows_kernel(SampleArgs<T> a) {
 template <class T, int NT, int K, int RB, bool EXACT, bool FULL, bool OFFS>
 __global__ void __launch_bounds__(NT) grad_input_rows_kernel(SampleArgs<T> a) {
     static_assert(RB % 4 == 0, "rows are handled in pairs, and pairs alternate between two LDS buffers");
-    const int64_t vid = xcd_contiguous_id(a.per_xcd);
+    const unsigned vid = xcd_contiguous_id(a.per_xcd);
     if (vid >= a.total) return;
-    const int band = static_cast<int>(vid % a.nb);
-    const int64_t p = vid / a.nb;
-    const int c_in = static_cast<int>((a.plane0 + p) % a.C);
+    const unsigned nbands = a.nb;
+    const int band = static_cast<int>(vid % nbands);
+    const int64_t p = vid / nbands;
+    const int c_in = static_cast<int>(static_cast<unsigned>(a.plane0 + p) % static_cast<unsigned>(a.C));
     const int h = a.h, w = a.w;
     const unsigned row_bytes = static_cast<unsigned>(w) * sizeof(T);
     const int64_t pitch = w + 1;
@@ -641,13 +551,14 @@ __device__ __forceinline__ void add_waves_left(const T* wave_tot, int wave, T& c
 
 template <class T, int NT, int K, bool EXACT, bool FULL, bool PARAMS, bool SCAN>
 __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a) {
-    const int64_t vid = xcd_contiguous_id(a.per_xcd);
+    const unsigned vid = xcd_contiguous_id(a.per_xcd);
     if (vid >= a.total) return;                      // whole workgroup leaves together
-    const int band = static_cast<int>(vid % a.nb);
-    const int64_t pf = vid / a.nb;
-    const int f = static_cast<int>(pf % a.F);
-    const int64_t p = pf / a.F;
-    const int k_par = static_cast<int>((a.plane0 + p) % a.C) * a.F + f;
+    const unsigned nbands = a.nb, nfilt = a.F;
+    const int band = static_cast<int>(vid % nbands);
+    const unsigned pf32 = vid / nbands;
+    const int f = static_cast<int>(pf32 % nfilt);
+    const int64_t pf = pf32, p = pf32 / nfilt;
+    const int k_par = static_cast<int>(static_cast<unsigned>(a.plane0 + p) % static_cast<unsigned>(a.C)) * a.F + f;
     const int h = a.h, w = a.w, tid = threadIdx.x;
     constexpr int nt = NT;
     const unsigned row_bytes = static_cast<unsigned>(w) * sizeof(T);
@@ -942,7 +853,7 @@ __global__ void __launch_bounds__(256) forward_gather_kernel(SampleArgs<T> a) {
     const int pix = static_cast<int>(idx % hw);
     const int i = pix / a.w, j = pix % a.w;
     const int64_t p = pf / a.F;
-    const int k_par = static_cast<int>((a.plane0 + p) % a.C) * a.F + static_cast<int>(pf % a.F);
+    const int k_par = static_cast<int>(static_cast<unsigned>(a.plane0 + p) % static_cast<unsigned>(a.C)) * a.F + static_cast<int>(pf % a.F);
     const BoxOfWorkgroup<T> bx = load_box(a.prm, k_par);
     const BoxSplit<T> s = split_forward(bx.xmin, bx.xmax, bx.ymin, bx.ymax);
     const T scale = a.normalize
@@ -959,7 +870,7 @@ __global__ void __launch_bounds__(256) grad_input_gather_kernel(SampleArgs<T> a)
     const int64_t p = idx / hw;
     const int pix = static_cast<int>(idx % hw);
     const int i = pix / a.w, j = pix % a.w;
-    const int c_in = static_cast<int>((a.plane0 + p) % a.C);
+    const int c_in = static_cast<int>(static_cast<unsigned>(a.plane0 + p) % static_cast<unsigned>(a.C));
     const int64_t ipl = static_cast<int64_t>(a.h + 1) * (a.w + 1);
     T acc = T(0);
     for (int f = 0; f < a.F; ++f) {
@@ -980,7 +891,7 @@ __global__ void __launch_bounds__(256) grad_params_gather_kernel(SampleArgs<T> a
     const int64_t pf = blockIdx.x / blocks_per_plane;
     const int pix = static_cast<int>(blockIdx.x % blocks_per_plane) * blockDim.x + threadIdx.x;
     const int64_t p = pf / a.F;
-    const int k_par = static_cast<int>((a.plane0 + p) % a.C) * a.F + static_cast<int>(pf % a.F);
+    const int k_par = static_cast<int>(static_cast<unsigned>(a.plane0 + p) % static_cast<unsigned>(a.C)) * a.F + static_cast<int>(pf % a.F);
     double v[5] = {0, 0, 0, 0, 0};
     if (pix < h * w) {
         const int i = pix / w, j = pix % w;

@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace boxconv {
 
 constexpr int kWave = 64;
@@ -135,15 +137,133 @@ __device__ __forceinline__ float read_lane<float>(float v, int lane) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
 }
 
+// ---------------------------------------------------------------------------------------------
+// Pointer plus a byte offset held in a 32-bit register. Global accesses written this way use a
+// scalar base and one VGPR offset, LDS accesses an immediate base; no per-access address math.
+template <class P>
+__device__ __forceinline__ P* at_bytes(P* base, unsigned bytes) {
+    using Byte = std::conditional_t<std::is_const<P>::value, const char, char>;
+    return reinterpret_cast<P*>(reinterpret_cast<Byte*>(base) + bytes);
+}
+
+// Global memory is reached through raw buffer instructions: a scalar descriptor (base, size in
+// bytes), a scalar byte offset and one 32-bit VGPR byte offset per access, so there is no
+// per-lane 64-bit address arithmetic. The hardware checks the VGPR offset against the size: a
+// load at or beyond it returns 0 and a store there is dropped.
+constexpr int kCacheDefault = 0, kCacheStream = 2;   // buffer cache policy bits: 2 = non-temporal
+template <class T>
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const T* base, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(base), 0, static_cast<int>(bytes), 0x00020000);
+}
+
+// One row of a stack of rows: descriptor plus scalar offset. Must be wave-uniform.
+struct RowRef {
+    __amdgpu_buffer_rsrc_t rs;
+    int soff;
+};
+
+// A stack of equally long rows of T in global memory (`cols` elements of each row reachable,
+// rows `pitch` elements apart, the whole stack below 4 GiB).
+//   BY_OFFSET: one descriptor spans the stack and a row is selected by its scalar byte offset.
+//              Only for stacks where every column slot of every lane is a valid column (there
+//              is no per-row bounds check). Measured: good for stores, slower than per-row
+//              descriptors for loads, so loads never use it.
+//   else     : one descriptor per row, sized to the row, so that the bounds check masks the
+//              column slots past its end.
+// A row that does not `exist` gets size 0: loads give 0, stores vanish, no branch needed.
+template <class T, bool BY_OFFSET>
+struct Rows {
+    T* base;
+    unsigned pitch_bytes, row_bytes, stack_bytes;
+    __device__ __forceinline__ Rows(T* base_, int64_t pitch, int cols, int nrows)
+        : base(base_), pitch_bytes(static_cast<unsigned>(pitch * sizeof(T))),
+          row_bytes(static_cast<unsigned>(cols) * static_cast<unsigned>(sizeof(T))),
+          stack_bytes(static_cast<unsigned>(nrows - 1) * pitch_bytes + row_bytes) {}
+    __device__ __forceinline__ RowRef row(int r, bool exists = true) const {
+        const unsigned offset = static_cast<unsigned>(r) * pitch_bytes;
+        if constexpr (BY_OFFSET)
+            return {make_buffer(base, exists ? stack_bytes : 0u), static_cast<int>(offset)};
+        else
+            return {make_buffer(at_bytes(base, offset), exists ? row_bytes : 0u), 0};
+    }
+};
+template <class T> using LoadRows = Rows<const T, false>;
+
+template <int POLICY>
+__device__ __forceinline__ float buffer_load(const RowRef& r, int off, float) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r.rs, off, r.soff, POLICY));
+}
+template <int POLICY>
+__device__ __forceinline__ double buffer_load(const RowRef& r, int off, double) {
+    return __builtin_bit_cast(double, __builtin_amdgcn_raw_buffer_load_b64(r.rs, off, r.soff, POLICY));
+}
+template <int POLICY>
+__device__ __forceinline__ void buffer_store(float v, const RowRef& r, int off) {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r.rs, off, r.soff, POLICY);
+}
+template <int POLICY>
+__device__ __forceinline__ void buffer_store(double v, const RowRef& r, int off) {
+    typedef unsigned v2u __attribute__((__vector_size__(8)));
+    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u, v), r.rs, off, r.soff, POLICY);
+}
+
+// K consecutive elements per lane. WHOLE: the run lies inside the row for every lane, so it
+// goes out as 16-byte pieces; otherwise element by element, each checked against the size.
+template <int POLICY, bool WHOLE, int K>
+__device__ __forceinline__ void buffer_store_run(const float (&v)[K], const RowRef& r, int off) {
+    typedef unsigned v4u __attribute__((__vector_size__(16)));
+    if constexpr (WHOLE && K % 4 == 0) {
+#pragma unroll
+        for (int k = 0; k < K; k += 4) {
+            const v4u pack = {__builtin_bit_cast(unsigned, v[k]), __builtin_bit_cast(unsigned, v[k + 1]),
+                              __builtin_bit_cast(unsigned, v[k + 2]), __builtin_bit_cast(unsigned, v[k + 3])};
+            __builtin_amdgcn_raw_buffer_store_b128(pack, r.rs, off + 4 * k, r.soff, POLICY);
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < K; ++k) buffer_store<POLICY>(v[k], r, off + 4 * k);
+    }
+}
+template <int POLICY, bool WHOLE, int K>
+__device__ __forceinline__ void buffer_store_run(const double (&v)[K], const RowRef& r, int off) {
+#pragma unroll
+    for (int k = 0; k < K; ++k) buffer_store<POLICY>(v[k], r, off + 8 * k);
+}
+
+// K consecutive elements per lane, element by element, each checked against the row size.
+// (There is deliberately no 16-byte variant: this toolchain lowers the 128-bit raw buffer LOAD
+// builtin to a 32-bit load. 16-byte loads go through load_quad below.)
+template <int POLICY, class T, int K>
+__device__ __forceinline__ void buffer_load_run(T (&v)[K], const RowRef& r, int off) {
+#pragma unroll
+    for (int k = 0; k < K; ++k) v[k] = buffer_load<POLICY>(r, off + static_cast<int>(sizeof(T)) * k, T());
+}
+
+// Four consecutive elements from a 16-byte aligned address with one (float) or two (double)
+// 16-byte non-temporal global loads.
+__device__ __forceinline__ void load_quad(const float* p, float (&v)[4]) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    const f4 q = __builtin_nontemporal_load(reinterpret_cast<const f4*>(p));
+    v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+}
+__device__ __forceinline__ void load_quad(const double* p, double (&v)[4]) {
+    typedef double d2 __attribute__((ext_vector_type(2)));
+    const d2 q0 = __builtin_nontemporal_load(reinterpret_cast<const d2*>(p));
+    const d2 q1 = __builtin_nontemporal_load(reinterpret_cast<const d2*>(p) + 1);
+    v[0] = q0.x; v[1] = q0.y; v[2] = q1.x; v[3] = q1.y;
+}
+
 // Workgroup index remapped so that a contiguous range of work items lands on one XCD.
 // Hardware hands consecutive workgroup ids to the 8 XCDs in turn; item ids are decoded with the
 // slowest-varying coordinate first, so giving XCD x the range [x*per, (x+1)*per) keeps all the
 // work that shares one integral plane inside one XCD's L2. Launch with 8*per workgroups,
 // per = ceil(total/8); ids >= total must exit.
 constexpr int kXcds = 8;
-__device__ __forceinline__ int64_t xcd_contiguous_id(int64_t per_xcd) {
-    const int64_t id = blockIdx.x;
-    return (id % kXcds) * per_xcd + id / kXcds;
+// A grid has fewer than 2^31 workgroups, so 32-bit arithmetic is exact (and much cheaper than
+// 64-bit division in scalar code).
+__device__ __forceinline__ unsigned xcd_contiguous_id(int64_t per_xcd) {
+    const unsigned id = blockIdx.x;
+    return (id % kXcds) * static_cast<unsigned>(per_xcd) + id / kXcds;
 }
 
 }  // namespace boxconv

@@ -32,30 +32,47 @@ template <class T>
 struct alignas(4 * sizeof(T)) Vec4 { T v[4]; };
 
 // ---- pass 1 -----------------------------------------------------------------------------------
-template <class T>
+// One workgroup per (plane, band, strip of 1024 columns); lane `tid` owns 4 consecutive columns
+// and keeps 8 row loads in flight. VEC: rows are 16-byte aligned and w is a multiple of 4.
+template <class T, bool VEC>
 __global__ void __launch_bounds__(256)
 band_colsum_kernel(const T* __restrict__ in, double* __restrict__ aux, int h, int w, int nb,
-                   int R) {
-    const int64_t blk = blockIdx.x;                 // p * (nb-1) + band, band < nb-1
-    const int band = static_cast<int>(blk % (nb - 1));
-    const int64_t p = blk / (nb - 1);
+                   int R, int strips) {
+    constexpr int U = 8;
+    unsigned blk = blockIdx.x;                      // (p * (nb-1) + band) * strips + strip
+    const int strip = static_cast<int>(blk % static_cast<unsigned>(strips));
+    blk /= static_cast<unsigned>(strips);
+    const int band = static_cast<int>(blk % static_cast<unsigned>(nb - 1));
+    const int64_t p = blk / static_cast<unsigned>(nb - 1);
     const int r0 = band * R;
     const int r1 = min(h, r0 + R);
+    const int c0 = strip * 1024 + 4 * static_cast<int>(threadIdx.x);
     const T* src = in + p * static_cast<int64_t>(h) * w;
-    double* dst = aux + blk * static_cast<int64_t>(w);
-    for (int c = threadIdx.x; c < w; c += blockDim.x) {
-        double a0 = 0, a1 = 0, a2 = 0, a3 = 0;
-        int r = r0;
-        for (; r + 3 < r1; r += 4) {
-            const T x0 = src[static_cast<int64_t>(r) * w + c];
-            const T x1 = src[static_cast<int64_t>(r + 1) * w + c];
-            const T x2 = src[static_cast<int64_t>(r + 2) * w + c];
-            const T x3 = src[static_cast<int64_t>(r + 3) * w + c];
-            a0 += x0; a1 += x1; a2 += x2; a3 += x3;
+    const Rows<const T, false> irows(src, w, w, h);
+    const int off = c0 * static_cast<int>(sizeof(T));
+
+    double acc[4] = {0.0, 0.0, 0.0, 0.0};
+    for (int r = r0; r < r1; r += U) {
+        T x[U][4];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (VEC) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) x[u][v] = T(0);
+                if (r + u < r1 && c0 < w) load_quad(src + static_cast<int64_t>(r + u) * w + c0, x[u]);
+            } else {
+                buffer_load_run<kCacheDefault>(x[u], irows.row(min(r + u, h - 1), r + u < r1), off);
+            }
         }
-        for (; r < r1; ++r) a0 += src[static_cast<int64_t>(r) * w + c];
-        dst[c] = (a0 + a1) + (a2 + a3);
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) acc[v] += static_cast<double>(x[u][v]);
     }
+    double* dst = aux + static_cast<int64_t>(blk) * w;
+#pragma unroll
+    for (int v = 0; v < 4; ++v)
+        if (c0 + v < w) dst[c0 + v] = acc[v];
 }
 
 // ---- pass 2 -----------------------------------------------------------------------------------
@@ -88,11 +105,11 @@ band_scan_kernel(const T* __restrict__ in, T* __restrict__ out, const double* __
     __shared__ __align__(32) T stage[RB][TW];
     __shared__ double row_carry[256];   // prefix of each band row up to the current tile; R <= 256
 
-    int64_t blk = xcd_contiguous_id(per_xcd);     // p * nb + band
+    unsigned blk = xcd_contiguous_id(per_xcd);    // p * nb + band
     if (blk >= total) return;
-    if (reverse) blk = total - 1 - blk;
-    const int band = static_cast<int>(blk % nb);
-    const int64_t p = blk / nb;
+    if (reverse) blk = static_cast<unsigned>(total) - 1u - blk;
+    const int band = static_cast<int>(blk % static_cast<unsigned>(nb));
+    const int64_t p = blk / static_cast<unsigned>(nb);
     const int r0 = band * R;
     const int r1 = min(h, r0 + R);
     const int tid = threadIdx.x;
@@ -212,6 +229,113 @@ band_scan_kernel(const T* __restrict__ in, T* __restrict__ out, const double* __
     }
 }
 
+// ---- pass 3, rows no wider than one tile --------------------------------------------------------
+// WAVES*64 threads, lane `tid` owns the 4 consecutive columns 4*tid .. 4*tid+3, so a row of up to
+// WAVES*256 columns is one tile. Differences to band_scan_kernel: `aux` holds the plain per-band
+// column sums (the sum over the bands above is formed here, no band_prefix pass); the loads of the
+// next RB rows are in flight while the current ones are scanned; there is one barrier per RB rows
+// (wave totals, double-buffered) and results are stored straight from registers, 4 consecutive
+// elements per lane. VEC: rows are 16-byte aligned and w is a multiple of 4. FULL: w == 4 * threads.
+template <class T, int WAVES, int RB, bool VEC, bool FULL>
+__global__ void __launch_bounds__(WAVES * 64)
+band_scan_rows_kernel(const T* __restrict__ in, T* __restrict__ out, const double* __restrict__ aux,
+                      int h, int w, int nb, int R, int64_t total, int64_t per_xcd, int reverse) {
+    constexpr int NT = WAVES * 64;
+    __shared__ double wave_tot[2][RB][WAVES];
+
+    unsigned blk = xcd_contiguous_id(per_xcd);    // p * nb + band
+    if (blk >= total) return;
+    if (reverse) blk = static_cast<unsigned>(total) - 1u - blk;
+    const int band = static_cast<int>(blk % static_cast<unsigned>(nb));
+    const int64_t p = blk / static_cast<unsigned>(nb);
+    const int r0 = band * R;
+    const int r1 = min(h, r0 + R);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keep it scalar
+    const int64_t W1 = static_cast<int64_t>(w) + 1;
+    const int c0 = 4 * tid;                       // first of the lane's columns
+
+    const T* src = in + p * static_cast<int64_t>(h) * w;
+    const Rows<const T, false> irows(src, w, w, h);
+    T* dst = out + p * static_cast<int64_t>(h + 1) * W1;
+    const Rows<T, FULL> orows(dst, W1, w + 1, h + 1);
+    const int in_off = c0 * static_cast<int>(sizeof(T));
+    const int out_off = (c0 + 1) * static_cast<int>(sizeof(T));
+
+    if (band == 0)
+        for (int c = tid; c <= w; c += NT) dst[c] = T(0);
+
+    // column accumulators start at the sum of all bands above
+    double colacc[4] = {0.0, 0.0, 0.0, 0.0};
+    {
+        const Rows<const double, false> arows(aux + p * static_cast<int64_t>(nb - 1) * w, w, w, max(nb - 1, 1));
+        for (int b = 0; b < band; ++b) {
+            double part[4];
+            buffer_load_run<kCacheDefault>(part, arows.row(b), c0 * 8);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) colacc[v] += part[v];
+        }
+    }
+
+    auto load_batch = [&](int rbase, T (&x)[RB][4]) {
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            const int row = rbase + rb;
+            if (VEC) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) x[rb][v] = T(0);
+                if (row < r1 && c0 < w) load_quad(src + static_cast<int64_t>(row) * w + c0, x[rb]);
+            } else {
+                buffer_load_run<kCacheStream>(x[rb], irows.row(min(row, h - 1), row < r1), in_off);
+            }
+        }
+    };
+
+    T x[RB][4];
+    load_batch(r0, x);
+    int buf = 0;
+    for (int rbase = r0; rbase < r1; rbase += RB) {
+        T nx[RB][4];
+        load_batch(rbase + RB, nx);               // rows past the band come back as zeros, unread
+
+        double pre[RB][4], excl[RB];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            double run = 0.0;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                colacc[v] += static_cast<double>(x[rb][v]);
+                run += colacc[v];
+                pre[rb][v] = run;                 // inclusive within the lane
+            }
+            const double incl = wave_inclusive_scan(run);
+            excl[rb] = incl - run;                // lanes to the left, this wave
+            if (lane == 63) wave_tot[buf][rb][wave] = incl;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            const int row = rbase + rb;
+            double left = excl[rb];
+#pragma unroll
+            for (int wv = 0; wv < WAVES - 1; ++wv)
+                if (wv < wave) left += wave_tot[buf][rb][wv];      // scalar condition
+            T res[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) res[v] = static_cast<T>(left + pre[rb][v]);
+            const RowRef orow = orows.row(min(row + 1, h), row < r1);
+            buffer_store_run<kCacheDefault, FULL>(res, orow, out_off);
+            if (tid == 0 && row < r1) dst[static_cast<int64_t>(row + 1) * W1] = T(0);
+        }
+        buf ^= 1;
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) x[rb][v] = nx[rb][v];
+    }
+}
+
 template <class T>
 bool aligned_for_vec4(const T* p, int w) {
     return (w % 4 == 0) && (reinterpret_cast<uintptr_t>(p) % (4 * sizeof(T)) == 0);
@@ -232,6 +356,33 @@ hipError_t launch_scan(const T* in, T* out, const double* aux, int64_t planes, i
         BOXCONV_LAUNCH("band_scan", (band_scan_kernel<T, WAVES, M, RB, false>), grid, block, 0, stream,
                        in, out, aux, h, w, nb, R, total, per_xcd, rev);
     return hipGetLastError();
+}
+
+template <class T, int WAVES, int RB>
+hipError_t launch_scan_rows(const T* in, T* out, const double* aux, int64_t planes, int h, int w,
+                            int nb, int R, bool reverse, hipStream_t stream) {
+    const int64_t total = planes * nb;
+    const int64_t per_xcd = (total + kXcds - 1) / kXcds;
+    const int rev = reverse ? 1 : 0;
+    const dim3 grid(static_cast<unsigned>(per_xcd * kXcds));
+    const dim3 block(WAVES * 64);
+    const bool vec = aligned_for_vec4(in, w), full = (w == WAVES * 256);
+#define LAUNCH_ROWS(VEC, FULL)                                                                     \
+    BOXCONV_LAUNCH("band_scan", (band_scan_rows_kernel<T, WAVES, RB, VEC, FULL>), grid, block, 0,  \
+                   stream, in, out, aux, h, w, nb, R, total, per_xcd, rev)
+    if (vec && full) LAUNCH_ROWS(true, true);
+    else if (vec)    LAUNCH_ROWS(true, false);
+    else             LAUNCH_ROWS(false, false);
+#undef LAUNCH_ROWS
+    return hipGetLastError();
+}
+
+// Rows this narrow are scanned by band_scan_rows_kernel, which sums the band column sums itself;
+// the bands above a workgroup are few (nb <= h/32), so re-reading them is cheaper than a pass.
+constexpr int kMaxScanRowsWidth = 2048;
+inline bool scan_by_rows(int h, int w, size_t elem) {
+    const uint64_t plane_bytes = (static_cast<uint64_t>(h) + 1) * (static_cast<uint64_t>(w) + 1) * elem;
+    return w <= kMaxScanRowsWidth && plane_bytes < (1ull << 31);
 }
 
 }  // namespace
@@ -262,19 +413,31 @@ hipError_t integral_image_launch(const T* in, T* out, int64_t planes, int h, int
     if (planes == 0) return hipSuccess;
     const int nb = pl.nb, R = pl.R;
     if (nb > 1 && !colsums_ready) {
-        BOXCONV_LAUNCH("band_colsum", (band_colsum_kernel<T>),
-                       dim3(static_cast<unsigned>(planes * (nb - 1))), dim3(256), 0, stream, in, aux,
-                       h, w, nb, R);
+        const int strips = (w + 1023) / 1024;
+        const dim3 grid(static_cast<unsigned>(planes * (nb - 1) * strips));
+        if (aligned_for_vec4(in, w))
+            BOXCONV_LAUNCH("band_colsum", (band_colsum_kernel<T, true>), grid, dim3(256), 0, stream,
+                           in, aux, h, w, nb, R, strips);
+        else
+            BOXCONV_LAUNCH("band_colsum", (band_colsum_kernel<T, false>), grid, dim3(256), 0, stream,
+                           in, aux, h, w, nb, R, strips);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
-    if (nb > 2) {
+    const bool by_rows = scan_by_rows(h, w, sizeof(T));
+    if (nb > 2 && !by_rows) {
         const int64_t n = planes * w;
         BOXCONV_LAUNCH("band_prefix", band_prefix_kernel,
                        dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, stream, aux,
                        planes, w, nb);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
+    }
+    if (by_rows) {
+        if (w <= 256)       return launch_scan_rows<T, 1, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
+        else if (w <= 512)  return launch_scan_rows<T, 2, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
+        else if (w <= 1024) return launch_scan_rows<T, 4, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
+        else                return launch_scan_rows<T, 8, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
     }
     // Tile width: one wave covers 256 columns per chunk, four waves 1024.
     if (w <= 256)        return launch_scan<T, 1, 1, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);

@@ -62,7 +62,8 @@ struct SampleArgs {
     BoxParams<T> prm;
     T* dst;               // forward: [planes,F,h,w]; grad input: [planes,h,w]
     const T* grad_out;    // param grads only: [planes,F,h,w]
-    double* acc;          // param grads only: [C*F*5]
+    double* acc;          // param grads only: [C*F*5], or [planes*F*acc_slots*5] workgroup slots
+    int acc_slots;        // param grads only: slots per (plane, filter), 0 = atomics on [C*F*5]
     int off_R;                // grad input only: rows per band of a band-local integral, 0 = true integral
     int C, F, h, w;
     int nb, R;            // bands per plane and rows per band
@@ -461,9 +462,11 @@ __global__ void __launch_bounds__(NT) grad_input_rows_kernel(SampleArgs<T> a) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Sum of 5 per-lane values over the workgroup, then one atomic per value.
+// Sum of 5 per-lane values over the workgroup; the totals are added to dst atomically or, when
+// dst is a slot that only this workgroup writes, simply stored.
 __device__ __forceinline__ void block_accumulate5(const double (&v)[5], double* __restrict__ dst,
-                                                  double* __restrict__ lds /* [waves*5] */) {
+                                                  double* __restrict__ lds /* [waves*5] */,
+                                                  bool atomic = true) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = (blockDim.x + 63) >> 6;
 #pragma unroll
     for (int n = 0; n < 5; ++n) {
@@ -474,7 +477,8 @@ __device__ __forceinline__ void block_accumulate5(const double (&v)[5], double* 
     if (threadIdx.x < 5) {
         double tot = 0.0;
         for (int wv = 0; wv < waves; ++wv) tot += lds[wv * 5 + threadIdx.x];
-        unsafeAtomicAdd(dst + threadIdx.x, tot);
+        if (atomic) unsafeAtomicAdd(dst + threadIdx.x, tot);
+        else dst[threadIdx.x] = tot;
     }
 }
 
@@ -810,7 +814,13 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
         const double v[5] = {static_cast<double>(sum[0]), static_cast<double>(sum[1]),
                              static_cast<double>(sum[2]), static_cast<double>(sum[3]),
                              static_cast<double>(sum[4])};
-        block_accumulate5(v, a.acc + static_cast<int64_t>(k_par) * 5, lds.red);
+        // slots > 0: one slot per workgroup, summed by the finalize kernel in a fixed order
+        // (no clearing pass, no atomics, bit-reproducible); else atomics into the box's five sums
+        if (a.acc_slots > 0)
+            block_accumulate5(v, a.acc + ((static_cast<int64_t>(a.plane0 + p) * a.F + f) * a.acc_slots + band) * 5,
+                              lds.red, false);
+        else
+            block_accumulate5(v, a.acc + static_cast<int64_t>(k_par) * 5, lds.red);
     }
 }
 
@@ -931,21 +941,41 @@ __global__ void fill_zero_kernel(double* __restrict__ p, int n) {
 // Turns the five sums per box into the four gradients (reference:
 // src/box_convolution_interface.cpp:345-391): optional 1/area, the d(1/area) term
 // sum(g*out) * (+-1)/(extent along the parameter's axis), and the reparametrization scale.
+// One wave per box. slots == 0: acc holds the five sums per box. Otherwise acc holds one slot of
+// five partial sums per (batch item b, box, band): [(b*n + box)*slots + band][5]; the wave adds
+// them in a fixed order.
 template <class T>
-__global__ void param_grad_finalize_kernel(const double* __restrict__ acc, BoxParams<T> prm,
-                                           T* g0, T* g1, T* g2, T* g3, int n, float reparam_h,
-                                           float reparam_w, int normalize, int exact) {
-    const int k = blockIdx.x * blockDim.x + threadIdx.x;
-    if (k >= n) return;
+__global__ void __launch_bounds__(64)
+param_grad_finalize_kernel(const double* __restrict__ acc, int batch, int slots, BoxParams<T> prm,
+                           T* g0, T* g1, T* g2, T* g3, int n, float reparam_h, float reparam_w,
+                           int normalize, int exact) {
+    const int k = blockIdx.x;
+    const int lane = threadIdx.x;
+    double sum[5] = {0.0, 0.0, 0.0, 0.0, 0.0};
+    if (slots > 0) {
+        const int per_box = batch * slots;
+        for (int e = lane; e < per_box; e += 64) {
+            const int b = e / slots, band = e % slots;
+            const double* part = acc + ((static_cast<int64_t>(b) * n + k) * slots + band) * 5;
+#pragma unroll
+            for (int m = 0; m < 5; ++m) sum[m] += part[m];
+        }
+#pragma unroll
+        for (int m = 0; m < 5; ++m) sum[m] = wave_sum_to_last(sum[m]);
+    } else {
+#pragma unroll
+        for (int m = 0; m < 5; ++m) sum[m] = acc[k * 5 + m];
+    }
+    if (lane != 63) return;
     const T xmin = prm.xmin[k], xmax = prm.xmax[k], ymin = prm.ymin[k], ymax = prm.ymax[k];
     const bool ex = exact != 0;
     const T inv_area = normalize ? inverse_extent(xmin, xmax, ymin, ymax, ex, true, true) : T(1);
-    const T s = normalize ? static_cast<T>(acc[k * 5 + 4]) * inv_area : T(0);   // sum(g * output)
+    const T s = normalize ? static_cast<T>(sum[4]) * inv_area : T(0);   // sum(g * output)
     T* outp[4] = {g0, g1, g2, g3};
 #pragma unroll
     for (int which = 0; which < 4; ++which) {
         if (outp[which] == nullptr) continue;
-        T g = static_cast<T>(acc[k * 5 + which]);
+        T g = static_cast<T>(sum[which]);
         if (normalize) {
             g *= inv_area;
             const bool is_x = which < 2;
@@ -1122,14 +1152,15 @@ StreamPlan plan_grad_output_stream(int64_t planes_f, int h, int w, size_t elem_s
 
 template <class T>
 hipError_t grad_output_stream_launch(const T* integ, const T* grad_out, BoxParams<T> prm,
-                                     double* acc, T* local_integral, const StreamPlan& sp, Dims d,
-                                     bool exact, hipStream_t stream) {
+                                     double* acc, int acc_slots, T* local_integral,
+                                     const StreamPlan& sp, Dims d, bool exact, hipStream_t stream) {
     const int64_t planes_f = d.planes * d.F;
     if (planes_f == 0 || d.hw() == 0) return hipSuccess;
     const bool params = acc != nullptr, scan = local_integral != nullptr;
     if (!sp.usable || (!params && !scan)) return hipErrorInvalidValue;
     SampleArgs<T> a = base_args(prm, d);
-    a.src = integ; a.grad_out = grad_out; a.acc = acc; a.dst = local_integral;
+    a.src = integ; a.grad_out = grad_out; a.acc = acc; a.acc_slots = acc_slots; a.dst = local_integral;
+    if (acc_slots != 0 && acc_slots != sp.nb) return hipErrorInvalidValue;
     a.nb = sp.nb; a.R = sp.R;
     finish_args(a, planes_f * a.nb);
     const RowConfig rc = stream_row_config(d.w);
@@ -1161,12 +1192,12 @@ hipError_t grad_params_gather_launch(const T* integ, const T* grad_out, BoxParam
 }
 
 template <class T>
-hipError_t grad_params_finish(const double* acc, BoxParams<T> prm, T* gxmin, T* gxmax, T* gymin,
-                              T* gymax, int n_boxes, float reparam_h, float reparam_w,
-                              bool normalize, bool exact, hipStream_t stream) {
+hipError_t grad_params_finish(const double* acc, int batch, int acc_slots, BoxParams<T> prm,
+                              T* gxmin, T* gxmax, T* gymin, T* gymax, int n_boxes, float reparam_h,
+                              float reparam_w, bool normalize, bool exact, hipStream_t stream) {
     if (n_boxes == 0) return hipSuccess;
-    BOXCONV_LAUNCH("param_grad_finalize", (param_grad_finalize_kernel<T>), dim3((n_boxes + 127) / 128),
-                   dim3(128), 0, stream, acc, prm, gxmin, gxmax, gymin, gymax, n_boxes, reparam_h,
+    BOXCONV_LAUNCH("param_grad_finalize", (param_grad_finalize_kernel<T>), dim3(n_boxes), dim3(64), 0,
+                   stream, acc, batch, acc_slots, prm, gxmin, gxmax, gymin, gymax, n_boxes, reparam_h,
                    reparam_w, normalize ? 1 : 0, exact ? 1 : 0);
     return hipGetLastError();
 }
@@ -1175,12 +1206,13 @@ hipError_t grad_params_finish(const double* acc, BoxParams<T> prm, T* gxmin, T* 
     template hipError_t forward_launch<T>(const T*, BoxParams<T>, T*, Dims, bool, bool, hipStream_t); \
     template hipError_t grad_input_launch<T>(const T*, int, BoxParams<T>, T*, Dims, bool, bool,    \
                                              hipStream_t);                                         \
-    template hipError_t grad_output_stream_launch<T>(const T*, const T*, BoxParams<T>, double*, T*, \
-                                                     const StreamPlan&, Dims, bool, hipStream_t);  \
+    template hipError_t grad_output_stream_launch<T>(const T*, const T*, BoxParams<T>, double*, int, \
+                                                     T*, const StreamPlan&, Dims, bool,            \
+                                                     hipStream_t);                                 \
     template hipError_t grad_params_gather_launch<T>(const T*, const T*, BoxParams<T>, double*,    \
                                                      Dims, bool, hipStream_t);                     \
-    template hipError_t grad_params_finish<T>(const double*, BoxParams<T>, T*, T*, T*, T*, int,    \
-                                              float, float, bool, bool, hipStream_t);
+    template hipError_t grad_params_finish<T>(const double*, int, int, BoxParams<T>, T*, T*, T*,   \
+                                              T*, int, float, float, bool, bool, hipStream_t);
 
 BOXCONV_INSTANTIATE(float)
 BOXCONV_INSTANTIATE(double)

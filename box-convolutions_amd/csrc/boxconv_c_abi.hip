@@ -108,10 +108,12 @@ bool reverse_second_pass() {
 // Workspace of the backward pass:
 //   [integral of grad_output: chunk*F planes of (h+1)(w+1)]   only if grad_input is wanted
 //   [aux doubles: band column sums, three-pass fallback only]
-//   [acc: C*F*5 doubles]                                       only if parameter gradients are wanted
+//   [acc: C*F*5 doubles, times batch*bands when every streaming workgroup has its own slot]
+//                                                              only if parameter gradients are wanted
 struct BackwardLayout {
     size_t gint_off, aux_off, acc_off, total;
     int64_t chunk;        // planes per chunk
+    int acc_slots;        // > 0: per-workgroup accumulation slots per (plane, filter), see grad_output_stream_launch
     bool streaming;       // grad_output_stream_kernel usable for this shape
 };
 
@@ -142,7 +144,13 @@ BackwardLayout backward_layout(int batch, int in_planes, int num_filters, int h,
         off += align_up(static_cast<size_t>(aux) * 8, 256);
     }
     L.acc_off = off;
-    if (need_params) off += align_up(static_cast<size_t>(in_planes) * num_filters * 5 * 8, 256);
+    // one accumulation slot per streaming workgroup when the whole batch goes in one chunk
+    L.acc_slots = 0;
+    if (need_params && L.streaming && L.chunk >= planes)
+        L.acc_slots = boxconv::plan_grad_output_stream(planes * num_filters, h, w, elem_size).nb;
+    if (need_params)
+        off += align_up(static_cast<size_t>(in_planes) * num_filters * 5 * 8 *
+                        (L.acc_slots > 0 ? static_cast<size_t>(batch) * L.acc_slots : 1), 256);
     L.total = off;
     return L;
 }
@@ -217,7 +225,7 @@ int backward_impl(const T* integ, const T* x_min, const T* x_max, const T* y_min
 
     if (need_input && nout == 0)
         return fail(BOXCONV_E_INVALID_ARGUMENT, "backward: grad_input requested with zero filters");
-    if (need_params)
+    if (need_params && L.acc_slots == 0)
         if (int rc = hip_result(boxconv::grad_params_begin(acc, n_boxes, s), "accumulator clear"))
             return rc;
 
@@ -235,7 +243,7 @@ int backward_impl(const T* integ, const T* x_min, const T* x_max, const T* y_min
             const boxconv::StreamPlan sp =
                 boxconv::plan_grad_output_stream(np * num_filters, h, w, sizeof(T));
             if (int rc = hip_result(boxconv::grad_output_stream_launch<T>(
-                    integ_chunk, go_chunk, prm, acc, gint, sp, d, exact != 0, s),
+                    integ_chunk, go_chunk, prm, acc, L.acc_slots, gint, sp, d, exact != 0, s),
                     "grad_output streaming launch"))
                 return rc;
             if (need_input)
@@ -266,7 +274,7 @@ int backward_impl(const T* integ, const T* x_min, const T* x_max, const T* y_min
     }
     if (need_params)
         if (int rc = hip_result(boxconv::grad_params_finish<T>(
-                acc, prm, gx_min, gx_max, gy_min, gy_max, n_boxes, reparam_h, reparam_w,
+                acc, batch, L.acc_slots, prm, gx_min, gx_max, gy_min, gy_max, n_boxes, reparam_h, reparam_w,
                 normalize != 0, exact != 0, s), "parameter-gradient finish"))
             return rc;
     return 0;

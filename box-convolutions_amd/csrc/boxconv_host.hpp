@@ -62,22 +62,25 @@ struct StreamPlan {
 };
 StreamPlan plan_grad_output_stream(int64_t planes_f, int h, int w, size_t elem_size);
 
-// acc ([C*F*5] doubles, cleared by grad_params_begin) may be null: no parameter sums.
+// acc may be null: no parameter sums. With acc_slots == sp.nb it is [all planes*F][nb][5] doubles
+// and every workgroup stores its five partial sums in its own slot (nothing to clear, no atomics,
+// results reproducible bit for bit); with acc_slots == 0 it is [C*F*5] doubles, cleared by
+// grad_params_begin, and workgroups add atomically. grad_params_finish takes the same two values.
 // local_integral ([planes*F, h+1, w+1]) may be null: no integral. At least one of the two must
 // be given.
 template <class T>
 hipError_t grad_output_stream_launch(const T* integ, const T* grad_out, BoxParams<T> prm,
-                                     double* acc, T* local_integral, const StreamPlan& sp, Dims d,
-                                     bool exact, hipStream_t stream);
+                                     double* acc, int acc_slots, T* local_integral,
+                                     const StreamPlan& sp, Dims d, bool exact, hipStream_t stream);
 
 hipError_t grad_params_begin(double* acc, int n_boxes, hipStream_t stream);
 template <class T>
 hipError_t grad_params_gather_launch(const T* integ, const T* grad_out, BoxParams<T> prm,
                                      double* acc, Dims d, bool exact, hipStream_t stream);
 template <class T>
-hipError_t grad_params_finish(const double* acc, BoxParams<T> prm, T* gxmin, T* gxmax, T* gymin,
-                              T* gymax, int n_boxes, float reparam_h, float reparam_w,
-                              bool normalize, bool exact, hipStream_t stream);
+hipError_t grad_params_finish(const double* acc, int batch, int acc_slots, BoxParams<T> prm,
+                              T* gxmin, T* gxmax, T* gymin, T* gymax, int n_boxes, float reparam_h,
+                              float reparam_w, bool normalize, bool exact, hipStream_t stream);
 
 template <class T>
 hipError_t clip_launch(T* xmin, T* xmax, T* ymin, T* ymax, int n, double reparam_h,

@@ -157,6 +157,24 @@ def test_backward_across_row_bands(hip, oracle, h, w, kind):
     assert_parity(cpu, gpu, np.float32, "%s %dx%d" % (kind, h, w), **sc)
 
 
+def test_parameter_gradients_are_reproducible(hip):
+    """The streaming backward adds the per-workgroup partial sums in a fixed order (no atomics),
+    so repeated calls agree bit for bit."""
+    rng = np.random.default_rng(5)
+    B, C, F, h, w = 3, 2, 3, 130, 200
+    x = dev(rng.standard_normal((B, C, h, w)).astype(np.float32))
+    g = dev(rng.standard_normal((B, C * F, h, w)).astype(np.float32))
+    boxes = [dev(b) for b in make_boxes(rng, C, F, h, w, "hanging")]
+    integ = hip.integral_image(x)
+    out = hip.box_convolution_forward(integ, *boxes, True, True)
+    runs = [hip.box_convolution_backward(integ, *boxes, g, out, 11.0, 7.0, True, True,
+                                         True, True, True, True, True) for _ in range(3)]
+    torch.cuda.synchronize()
+    for other in runs[1:]:
+        for a, b in zip(runs[0], other):
+            assert torch.equal(a, b)
+
+
 def test_unit_box_is_identity(hip):
     x = torch.randn(2, 3, 13, 31, device="cuda")
     z = torch.zeros(3, 2, device="cuda")

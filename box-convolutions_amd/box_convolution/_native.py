@@ -38,6 +38,7 @@ for _s in ("f32", "f64"):
     _SIGNATURES["boxconv_backward_" + _s] = (
         _i, [_vp] * 7 + [_f, _f, _i, _i] + [_vp] * 5 + [_i] * 5 + [_vp, _sz, _vp])
     _SIGNATURES["boxconv_clip_parameters_" + _s] = (_i, [_vp] * 4 + [_i] + [_d] * 4 + [_i, _vp])
+    _SIGNATURES["boxconv_clip_reparametrize_" + _s] = (_i, [_vp] * 5 + [_i] + [_d] * 4 + [_i, _vp])
 
 EXPORTED_SYMBOLS = tuple(sorted(_SIGNATURES))
 
@@ -265,6 +266,31 @@ def clip_parameters(x_min, x_max, y_min, y_max, reparametrization_h, reparametri
             float(reparametrization_h), float(reparametrization_w), float(max_input_h),
             float(max_input_w), int(bool(exact)), _stream(x_min.device))
     _check(rc, "clip_parameters")
+
+
+def clip_reparametrize(x_min, x_max, y_min, y_max, reparametrization_h, reparametrization_w,
+                       max_input_h, max_input_w, exact):
+    """``clip_parameters`` followed by ``reparametrize(..., inverse=True)`` in one launch: clips the
+    stored parameters in place and returns the four clipped tensors in real pixel units (new
+    tensors, views of one allocation). Device tensors only."""
+    params = (x_min, x_max, y_min, y_max)
+    for p in params:
+        if (not p.is_cuda or p.shape != x_min.shape or p.dtype != x_min.dtype
+                or p.device != x_min.device or not p.is_contiguous()):
+            raise RuntimeError("box_convolution: clip_reparametrize needs four contiguous device "
+                               "tensors of one shape, dtype and device")
+    sfx = _suffix(x_min, "parameters")
+    n = x_min.numel()
+    real = torch.empty((4,) + tuple(x_min.shape), dtype=x_min.dtype, device=x_min.device)
+    if n > 0:
+        lib = load()
+        with torch.cuda.device(x_min.device):
+            rc = getattr(lib, "boxconv_clip_reparametrize_" + sfx)(
+                _ptr(x_min), _ptr(x_max), _ptr(y_min), _ptr(y_max), _ptr(real), n,
+                float(reparametrization_h), float(reparametrization_w), float(max_input_h),
+                float(max_input_w), int(bool(exact)), _stream(x_min.device))
+        _check(rc, "clip_reparametrize")
+    return real[0], real[1], real[2], real[3]
 
 
 KERNEL_NAMES = ("band_colsum", "band_prefix", "band_scan", "forward_rows", "grad_output_stream",

@@ -37,18 +37,26 @@ class BoxConvolutionFunction(torch.autograd.Function):
     """``apply(input, x_min, x_max, y_min, y_max, reparametrization_h, reparametrization_w,
     normalize, exact) -> output [B, C*F, h, w]``; parameters in stored units.
     (reference box_convolution_function.py:30-65)
+
+    One optional trailing argument that the reference does not have: ``real_parameters``, the four
+    parameters already in real pixel units (what ``reparametrize(..., inverse=True)`` would
+    return for the stored ones). ``BoxConv2d`` passes it in training mode, where the clip kernel
+    produces them on the side.
     """
 
     @staticmethod
     def forward(ctx, input, x_min, x_max, y_min, y_max,
-                reparametrization_h, reparametrization_w, normalize, exact):
+                reparametrization_h, reparametrization_w, normalize, exact, real_parameters=None):
         ctx.normalize = normalize
         ctx.reparametrization_h = reparametrization_h
         ctx.reparametrization_w = reparametrization_w
         ctx.exact = exact
 
-        x_min, x_max, y_min, y_max = reparametrize(
-            x_min, x_max, y_min, y_max, reparametrization_h, reparametrization_w, inverse=True)
+        if real_parameters is not None:
+            x_min, x_max, y_min, y_max = real_parameters
+        else:
+            x_min, x_max, y_min, y_max = reparametrize(
+                x_min, x_max, y_min, y_max, reparametrization_h, reparametrization_w, inverse=True)
 
         input_integrated = _native.integral_image(input)
         output = _native.box_convolution_forward(
@@ -67,5 +75,6 @@ class BoxConvolutionFunction(torch.autograd.Function):
             input_integrated, x_min, x_max, y_min, y_max, grad_output, None,
             ctx.reparametrization_h, ctx.reparametrization_w,
             ctx.normalize, ctx.exact, *ctx.needs_input_grad[:5])
-        # no gradients for reparametrization_h, reparametrization_w, normalize, exact
-        return tuple(grads) + (None,) * 4
+        # no gradients for reparametrization_h, reparametrization_w, normalize, exact,
+        # real_parameters
+        return tuple(grads) + (None,) * 5

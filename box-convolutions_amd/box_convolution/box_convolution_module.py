@@ -99,9 +99,18 @@ class BoxConv2d(torch.nn.Module):
         return self
 
     def forward(self, input):
+        real_parameters = None
         if self.training:
-            self._clip_parameters()
+            if self.x_min.is_cuda:
+                # the projection and the stored -> real conversion in one launch
+                real_parameters = _native.clip_reparametrize(
+                    self.x_min.detach(), self.x_max.detach(), self.y_min.detach(), self.y_max.detach(),
+                    self.reparametrization_h, self.reparametrization_w,
+                    self.max_input_h, self.max_input_w, self.exact)
+            else:
+                self._clip_parameters()
 
         return BoxConvolutionFunction.apply(
             input, self.x_min, self.x_max, self.y_min, self.y_max,
-            self.reparametrization_h, self.reparametrization_w, self.normalize, self.exact)
+            self.reparametrization_h, self.reparametrization_w, self.normalize, self.exact,
+            real_parameters)

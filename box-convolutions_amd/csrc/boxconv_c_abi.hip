@@ -281,7 +281,7 @@ int backward_impl(const T* integ, const T* x_min, const T* x_max, const T* y_min
 }
 
 template <class T>
-int clip_impl(T* x_min, T* x_max, T* y_min, T* y_max, int n, double reparam_h, double reparam_w,
+int clip_impl(T* x_min, T* x_max, T* y_min, T* y_max, T* real, int n, double reparam_h, double reparam_w,
               double max_h, double max_w, int exact, void* stream) {
     if (n < 0) return fail(BOXCONV_E_INVALID_ARGUMENT, "clip: negative element count");
     if (n == 0) return 0;
@@ -289,7 +289,7 @@ int clip_impl(T* x_min, T* x_max, T* y_min, T* y_max, int n, double reparam_h, d
         return fail(BOXCONV_E_INVALID_ARGUMENT, "clip: null parameter pointer");
     if (!(reparam_h != 0.0) || !(reparam_w != 0.0))
         return fail(BOXCONV_E_INVALID_ARGUMENT, "clip: reparametrization factor is zero");
-    return hip_result(boxconv::clip_launch<T>(x_min, x_max, y_min, y_max, n, reparam_h, reparam_w,
+    return hip_result(boxconv::clip_launch<T>(x_min, x_max, y_min, y_max, real, n, reparam_h, reparam_w,
                                               max_h, max_w, exact != 0,
                                               static_cast<hipStream_t>(stream)),
                       "clip launch");
@@ -401,13 +401,32 @@ int boxconv_backward_f64(const double* input_integrated, const double* x_min, co
 int boxconv_clip_parameters_f32(float* x_min, float* x_max, float* y_min, float* y_max, int n,
                                 double reparametrization_h, double reparametrization_w,
                                 double max_input_h, double max_input_w, int exact, void* stream) {
-    return clip_impl<float>(x_min, x_max, y_min, y_max, n, reparametrization_h,
+    return clip_impl<float>(x_min, x_max, y_min, y_max, nullptr, n, reparametrization_h,
                             reparametrization_w, max_input_h, max_input_w, exact, stream);
 }
 int boxconv_clip_parameters_f64(double* x_min, double* x_max, double* y_min, double* y_max, int n,
                                 double reparametrization_h, double reparametrization_w,
                                 double max_input_h, double max_input_w, int exact, void* stream) {
-    return clip_impl<double>(x_min, x_max, y_min, y_max, n, reparametrization_h,
+    return clip_impl<double>(x_min, x_max, y_min, y_max, nullptr, n, reparametrization_h,
+                             reparametrization_w, max_input_h, max_input_w, exact, stream);
+}
+
+int boxconv_clip_reparametrize_f32(float* x_min, float* x_max, float* y_min, float* y_max,
+                                   float* real_parameters, int n, double reparametrization_h,
+                                   double reparametrization_w, double max_input_h,
+                                   double max_input_w, int exact, void* stream) {
+    if (n > 0 && real_parameters == nullptr)
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "clip_reparametrize: null output pointer");
+    return clip_impl<float>(x_min, x_max, y_min, y_max, real_parameters, n, reparametrization_h,
+                            reparametrization_w, max_input_h, max_input_w, exact, stream);
+}
+int boxconv_clip_reparametrize_f64(double* x_min, double* x_max, double* y_min, double* y_max,
+                                   double* real_parameters, int n, double reparametrization_h,
+                                   double reparametrization_w, double max_input_h,
+                                   double max_input_w, int exact, void* stream) {
+    if (n > 0 && real_parameters == nullptr)
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "clip_reparametrize: null output pointer");
+    return clip_impl<double>(x_min, x_max, y_min, y_max, real_parameters, n, reparametrization_h,
                              reparametrization_w, max_input_h, max_input_w, exact, stream);
 }
 

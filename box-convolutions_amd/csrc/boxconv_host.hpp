@@ -82,8 +82,9 @@ hipError_t grad_params_finish(const double* acc, int batch, int acc_slots, BoxPa
                               T* gxmin, T* gxmax, T* gymin, T* gymax, int n_boxes, float reparam_h,
                               float reparam_w, bool normalize, bool exact, hipStream_t stream);
 
+// real: null, or [4][n] receiving the clipped bounds times their reparametrization factor.
 template <class T>
-hipError_t clip_launch(T* xmin, T* xmax, T* ymin, T* ymax, int n, double reparam_h,
+hipError_t clip_launch(T* xmin, T* xmax, T* ymin, T* ymax, T* real, int n, double reparam_h,
                        double reparam_w, double max_h, double max_w, bool exact,
                        hipStream_t stream);
 

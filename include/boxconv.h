@@ -125,6 +125,24 @@ int boxconv_clip_parameters_f64(double* x_min, double* x_max, double* y_min, dou
                                 double reparametrization_h, double reparametrization_w,
                                 double max_input_h, double max_input_w, int exact, void* stream);
 
+/* ---- clip + stored -> real units in one launch ------------------------------------------------
+ * What a training-mode forward of the reference does with the parameters before anything else:
+ * `clip_parameters(...)` (as above; reference box_convolution/box_convolution_module.py:203-206)
+ * followed by `reparametrize(..., inverse=True)` (reference
+ * box_convolution/box_convolution_function.py:5-27, called at :41-43), i.e. four more element-wise
+ * multiplications. The stored parameters are clipped in place exactly as by
+ * boxconv_clip_parameters_*; real_parameters ([4][n]: x_min, x_max, y_min, y_max) receives
+ * clipped * reparametrization, the factor rounded to the element type first (a tensor times a
+ * Python float). */
+int boxconv_clip_reparametrize_f32(float* x_min, float* x_max, float* y_min, float* y_max,
+                                   float* real_parameters, int n, double reparametrization_h,
+                                   double reparametrization_w, double max_input_h,
+                                   double max_input_w, int exact, void* stream);
+int boxconv_clip_reparametrize_f64(double* x_min, double* x_max, double* y_min, double* y_max,
+                                   double* real_parameters, int n, double reparametrization_h,
+                                   double reparametrization_w, double max_input_h,
+                                   double max_input_w, int exact, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

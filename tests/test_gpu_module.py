@@ -249,3 +249,33 @@ def test_noncontiguous_input_and_dtype_errors(hip):
         hip.box_convolution_forward(torch.zeros(1, 3, 5, 5, device=DEV), z, z, z, z, True, True)
     with pytest.raises(RuntimeError, match="different devices"):
         hip.box_convolution_forward(torch.zeros(1, 2, 5, 5, device=DEV), z.cpu(), z, z, z, True, True)
+
+
+def test_training_forward_fuses_clip_and_reparametrize():
+    """In training mode the module clips and converts to real units in one launch; the result
+    must equal clip_parameters followed by reparametrize(..., inverse=True) bit for bit."""
+    from box_convolution import BoxConv2d, _native
+    from box_convolution.box_convolution_function import reparametrize
+    torch.manual_seed(3)
+    for dtype in (torch.float32, torch.float64):
+        m = BoxConv2d(3, 4, 20, 30).to("cuda", dtype)
+        with torch.no_grad():      # push some boxes out of bounds / make some too thin
+            m.x_min.mul_(3.0); m.y_max.add_(0.5); m.x_max.copy_(m.x_min + 1e-4)
+        stored = [p.detach().clone() for p in (m.x_min, m.x_max, m.y_min, m.y_max)]
+        _native.clip_parameters(*stored, m.reparametrization_h, m.reparametrization_w, 20, 30, True)
+        want_real = reparametrize(*stored, m.reparametrization_h, m.reparametrization_w, inverse=True)
+        live = [p.detach() for p in (m.x_min, m.x_max, m.y_min, m.y_max)]
+        got_real = _native.clip_reparametrize(*live, m.reparametrization_h, m.reparametrization_w, 20, 30, True)
+        for a, b in zip(live, stored):
+            assert torch.equal(a, b)
+        for a, b in zip(got_real, want_real):
+            assert torch.equal(a, b)
+        # and through the module: same output as the two-step path
+        x = torch.randn(2, 3, 20, 30, device="cuda", dtype=dtype)
+        m.train()
+        out = m(x)
+        from box_convolution.box_convolution_function import BoxConvolutionFunction
+        # (the forward clipped once more; compare with the parameters as they are now)
+        now = [p.detach() for p in (m.x_min, m.x_max, m.y_min, m.y_max)]
+        ref = BoxConvolutionFunction.apply(x, *now, m.reparametrization_h, m.reparametrization_w, True, True)
+        assert torch.equal(out, ref)

@@ -95,7 +95,8 @@ def test_train_and_forward_clip_hooks(monkeypatch):
     m.train()
     n = len(calls)
     assert m(torch.zeros(1, 1, 8, 8)) == "out" and len(calls) == n + 1
-    assert seen[0][5:] == (m.reparametrization_h, m.reparametrization_w, True, False)
+    # (parameters on the host: separate clip, no pre-scaled parameters handed over)
+    assert seen[0][5:] == (m.reparametrization_h, m.reparametrization_w, True, False, None)
     m.training = False
     m(torch.zeros(1, 1, 8, 8))
     assert len(calls) == n + 1                 # no clip in eval mode

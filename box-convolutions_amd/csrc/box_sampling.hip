@@ -769,8 +769,8 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
 #pragma unroll
                 for (int k = 0; k < K; ++k) { out0[k] = carry0 + loc0[k]; out1[k] = carry1 + loc1[k]; }
                 const int first = (1 + K * tid) * static_cast<int>(sizeof(T));
-                buffer_store_run<kCacheStream, FULL>(out0, ob0, first);
-                buffer_store_run<kCacheStream, FULL>(out1, ob1, first);
+                buffer_store_run<kCacheStream, FULL>(out0, ob0, first, static_cast<int>(row_bytes + sizeof(T)));
+                buffer_store_run<kCacheStream, FULL>(out1, ob1, first, static_cast<int>(row_bytes + sizeof(T)));
                 if (tid == 0) {
                     o0[0] = T(0);
                     if (second) o0[pitch] = T(0);
@@ -990,7 +990,7 @@ param_grad_finalize_kernel(const double* __restrict__ acc, int batch, int slots,
 
 // ---------------------------------------------------------------------------------------------
 // Workgroup shapes the row kernels are compiled for: (threads, columns per lane).
-//   (64,1) widths up to 64; (256,1|2|4) up to 256|512|1024; (512,1|2|4) up to 512|1024|2048.
+//   (64,1) widths up to 64; (256,1..4) up to 256..1024; (512,1..4) up to 512..2048.
 // Each kernel has a preferred size (measured at width 1024: 512 threads for forward and grad
 // input, 256 for the grad_output pass); rows too wide for 4 columns per lane at that size take
 // 512 threads, which bounds the register footprint and the length of the per-lane float
@@ -1006,9 +1006,12 @@ inline RowConfig row_config(int w, int prefer) {
     if (w <= 64) {
         c.nt = 64; c.K = 1;
     } else {
-        c.nt = (w + prefer - 1) / prefer > 4 ? 512 : prefer;
-        const int k = (w + c.nt - 1) / c.nt;
-        c.K = k <= 1 ? 1 : k <= 2 ? 2 : 4;
+        // fewest column slots (K * threads) that cover the row; the preferred size wins ties
+        const int other = prefer == 256 ? 512 : 256;
+        const int kp = (w + prefer - 1) / prefer, ko = (w + other - 1) / other;
+        const bool use_other = kp > 4 || (ko <= 4 && ko * other < kp * prefer);
+        c.nt = use_other ? other : prefer;
+        c.K = std::min(std::max(use_other ? ko : kp, 1), 4);
     }
     c.full = (c.K * c.nt == w);
     return c;
@@ -1048,6 +1051,7 @@ void finish_args(SampleArgs<T>& a, int64_t total) {
     switch (K) {                                                                     \
         case 1: KERNEL(NT, 1, __VA_ARGS__); break;                                   \
         case 2: KERNEL(NT, 2, __VA_ARGS__); break;                                   \
+        case 3: KERNEL(NT, 3, __VA_ARGS__); break;                                   \
         default: KERNEL(NT, 4, __VA_ARGS__); break;                                  \
     }
 #define BOXCONV_DISPATCH_SHAPE(KERNEL, RC, ...)                                      \

@@ -207,25 +207,47 @@ __device__ __forceinline__ void buffer_store(double v, const RowRef& r, int off)
     __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u, v), r.rs, off, r.soff, POLICY);
 }
 
-// K consecutive elements per lane. WHOLE: the run lies inside the row for every lane, so it
-// goes out as 16-byte pieces; otherwise element by element, each checked against the size.
-template <int POLICY, bool WHOLE, int K>
-__device__ __forceinline__ void buffer_store_run(const float (&v)[K], const RowRef& r, int off) {
+// K consecutive elements per lane starting at byte offset `off` of a row of `limit` bytes. A
+// lane whose run lies inside the row stores it with one wide instruction (16, 12 or 8 bytes;
+// dword alignment suffices); the at most one lane per row whose run straddles the end goes
+// element by element, each store checked against the row size. WHOLE: every lane's run lies
+// inside the row, nothing to test.
+template <int POLICY, int K>
+__device__ __forceinline__ void buffer_store_wide(const float (&v)[K], const RowRef& r, int off) {
     typedef unsigned v4u __attribute__((__vector_size__(16)));
-    if constexpr (WHOLE && K % 4 == 0) {
+    typedef unsigned v3u __attribute__((__vector_size__(12)));
+    typedef unsigned v2u __attribute__((__vector_size__(8)));
+    if constexpr (K % 4 == 0) {
 #pragma unroll
         for (int k = 0; k < K; k += 4) {
             const v4u pack = {__builtin_bit_cast(unsigned, v[k]), __builtin_bit_cast(unsigned, v[k + 1]),
                               __builtin_bit_cast(unsigned, v[k + 2]), __builtin_bit_cast(unsigned, v[k + 3])};
             __builtin_amdgcn_raw_buffer_store_b128(pack, r.rs, off + 4 * k, r.soff, POLICY);
         }
+    } else if constexpr (K == 3) {
+        const v3u pack = {__builtin_bit_cast(unsigned, v[0]), __builtin_bit_cast(unsigned, v[1]),
+                          __builtin_bit_cast(unsigned, v[2])};
+        __builtin_amdgcn_raw_buffer_store_b96(pack, r.rs, off, r.soff, POLICY);
+    } else if constexpr (K == 2) {
+        const v2u pack = {__builtin_bit_cast(unsigned, v[0]), __builtin_bit_cast(unsigned, v[1])};
+        __builtin_amdgcn_raw_buffer_store_b64(pack, r.rs, off, r.soff, POLICY);
     } else {
 #pragma unroll
         for (int k = 0; k < K; ++k) buffer_store<POLICY>(v[k], r, off + 4 * k);
     }
 }
 template <int POLICY, bool WHOLE, int K>
-__device__ __forceinline__ void buffer_store_run(const double (&v)[K], const RowRef& r, int off) {
+__device__ __forceinline__ void buffer_store_run(const float (&v)[K], const RowRef& r, int off, int limit) {
+    if (WHOLE || off + 4 * K <= limit) {
+        buffer_store_wide<POLICY, K>(v, r, off);
+    } else {
+#pragma unroll
+        for (int k = 0; k < K; ++k) buffer_store<POLICY>(v[k], r, off + 4 * k);
+    }
+}
+template <int POLICY, bool WHOLE, int K>
+__device__ __forceinline__ void buffer_store_run(const double (&v)[K], const RowRef& r, int off, int limit) {
+    (void)limit;
 #pragma unroll
     for (int k = 0; k < K; ++k) buffer_store<POLICY>(v[k], r, off + 8 * k);
 }

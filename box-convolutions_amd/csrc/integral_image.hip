@@ -325,7 +325,7 @@ band_scan_rows_kernel(const T* __restrict__ in, T* __restrict__ out, const doubl
 #pragma unroll
             for (int v = 0; v < 4; ++v) res[v] = static_cast<T>(left + pre[rb][v]);
             const RowRef orow = orows.row(min(row + 1, h), row < r1);
-            buffer_store_run<kCacheDefault, FULL>(res, orow, out_off);
+            buffer_store_run<kCacheDefault, FULL>(res, orow, out_off, (w + 1) * static_cast<int>(sizeof(T)));
             if (tid == 0 && row < r1) dst[static_cast<int64_t>(row + 1) * W1] = T(0);
         }
         buf ^= 1;

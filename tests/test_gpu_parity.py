@@ -77,17 +77,26 @@ def run_both(hip, oracle, x, boxes, reparam_h, reparam_w, normalize, exact, grad
                                         normalize, exact, *needs)
     torch.cuda.synchronize()
     scales = dict(i_max=float(np.abs(integ_cpu).max()),
-                  gi_max=float(np.abs(oracle.integral_image(grad_out)).max()))
+                  gi_max=float(np.abs(oracle.integral_image(grad_out)).max()),
+                  pg_scale=float(np.abs(integ_cpu).max() * np.abs(grad_out).max()
+                                 * max(abs(reparam_h), abs(reparam_w))
+                                 * np.sqrt(grad_out.shape[-1] * grad_out.shape[-2])) if grad_out.size else 0.0)
     return (out_cpu, back_cpu), (host(out), [None if g is None else host(g) for g in back]), scales
 
 
-def assert_parity(cpu, gpu, dtype, what="", i_max=0.0, gi_max=0.0):
+def assert_parity(cpu, gpu, dtype, what="", i_max=0.0, gi_max=0.0, pg_scale=0.0):
     """max|gpu-cpu| <= tol * max|cpu| + 8 eps * (largest integral-image entry).
 
     The additive term is the rounding noise both implementations carry: every output is a
     difference of integral-image entries, each known to half a unit in its last place. It only
     matters for tensors that are (nearly) zero, e.g. a box that misses the image entirely.
-    i_max / gi_max: largest |entry| of the integral image of the input / of grad_output."""
+    i_max / gi_max: largest |entry| of the integral image of the input / of grad_output.
+    Parameter gradients are sums of grad_output times differences of integral-image entries,
+    scaled by the reparametrization factor; when every box of a tensor misses the image the true
+    gradients are zero and the float32 CPU result is rounding noise of the order eps * pg_scale
+    (pg_scale = i_max * max|grad_output| * reparametrization * sqrt(h*w): a random walk over the
+    pixels; the float64 oracle gives exact zeros there), which then is the scale they are compared
+    on. For boxes that do touch the image the gradients are of the order pg_scale itself."""
     tol_f, tol_p = TOL[dtype]
     eps = float(np.finfo(dtype).eps)
     (out_c, back_c), (out_g, back_g) = cpu, gpu
@@ -100,7 +109,7 @@ def assert_parity(cpu, gpu, dtype, what="", i_max=0.0, gi_max=0.0):
     assert close(out_g, out_c, tol_f, 8 * eps * i_max), what + " forward"
     if back_c[0] is not None:
         assert close(back_g[0], back_c[0], tol_f, 8 * eps * gi_max), what + " grad_input"
-    floor = param_grad_floor(back_c[1:])
+    floor = max(param_grad_floor(back_c[1:]), 8 * eps * pg_scale)
     for k, name in enumerate(("x_min", "x_max", "y_min", "y_max")):
         if back_c[1 + k] is not None:
             assert rel_err(back_g[1 + k], back_c[1 + k], floor) <= tol_p, what + " grad_" + name
@@ -111,6 +120,7 @@ SMALL_CASES = [
     (1, 1, 1, 2, 2), (1, 1, 1, 5, 9), (2, 3, 2, 7, 6), (1, 2, 3, 10, 10), (2, 1, 5, 28, 28),
     (1, 2, 2, 17, 65), (1, 1, 3, 40, 130), (1, 2, 2, 33, 300), (1, 1, 2, 20, 600),
     (1, 1, 2, 12, 1100), (1, 1, 1, 9, 2100), (1, 1, 2, 1, 1), (1, 1, 2, 1, 70), (1, 1, 2, 70, 1),
+    (1, 1, 2, 12, 700), (1, 2, 1, 10, 768), (1, 1, 2, 11, 1300), (1, 1, 1, 9, 1536),   # three columns per lane
 ]
 
 

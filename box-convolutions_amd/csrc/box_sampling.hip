@@ -20,12 +20,16 @@
 //
 // Row streaming. Column 0 of I is zero, so V(i) has w interesting entries. A workgroup owns a
 // band of output rows at full width: each lane keeps I[t(i-1)] and I[b(i)] of its columns in
-// registers and loads only the new rows I[t(i)], I[b(i+1)] per output row (coalesced). Two output
-// rows are handled per barrier, and the loads of the next two are issued before the barrier.
-//   forward / grad input: V(i) goes to LDS; every output pixel reads its four V entries.
-//   parameter gradients : the row of grad_output goes to LDS instead and every column q reads
+// registers and loads only the new rows I[t(i)], I[b(i+1)] per output row (coalesced raw buffer
+// loads: scalar row descriptor, one offset register per lane). Two output rows are handled per
+// barrier, and the loads of the next two are issued before the barrier. The two rows of a pair
+// sit interleaved in LDS, so one LDS access serves both.
+//   forward / grad input: V(i), V(i+1) go to LDS; every output pixel reads its four V entries.
+//   parameter gradients : the rows of grad_output go to LDS instead and every column q reads
 //       the four grad_output entries whose box edges fall on q (the transposed access), so V and
 //       the two row differences never leave registers: sum_j g[j]*H(X)[j] = sum_q X[q]*Ht(g)[q].
+// The workgroup size NT and the columns per lane K are template parameters (row_config picks the
+// tightest shape for a width), which turns every slot distance into an instruction offset.
 //
 // Workgroup ids are remapped (xcd_contiguous_id) so all filters and bands of one input plane run
 // on one XCD and its integral plane stays in that XCD's L2.
@@ -48,12 +52,10 @@ namespace {
 extern __shared__ __align__(16) unsigned char smem_raw[];
 
 // Largest workgroup of the row-streaming kernels (8 waves). A wide row is spread over more lanes
-// rather than more columns per lane: per-lane state (sliding rows, prefetched rows, accumulators)
-// scales with the columns per lane, and these kernels hide HBM latency with occupancy.
+// rather than over more than 4 columns per lane: per-lane state (sliding rows, prefetched rows,
+// accumulators) scales with the columns per lane, and these kernels hide HBM latency with
+// occupancy.
 constexpr int kMaxRowThreads = 512;
-#ifndef BOXCONV_STREAM_UNROLL
-#define BOXCONV_STREAM_UNROLL 0
-#endif
 constexpr int kMaxRowWaves = kMaxRowThreads / 64;
 
 template <class T>
@@ -639,14 +641,12 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
     load_g(i0 + 1, g1);
 
     int flip = 0;
-    auto row_pair = [&](int i, auto prefetch_tag, auto flip_tag) {
+    auto row_pair = [&](int i, auto prefetch_tag) {
         constexpr bool PREFETCH = decltype(prefetch_tag)::value;   // see forward_rows_kernel
-#if BOXCONV_STREAM_UNROLL
-        constexpr int FLIP = decltype(flip_tag)::value;
-#else
+        // (the LDS buffer alternates at run time here: unrolling this loop over both buffers, as
+        // the forward kernel does, costs more registers than the kernel can afford)
         const int FLIP = flip;
         flip ^= 1;
-#endif
         T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {}, m0[K] = {}, m1[K] = {};
         if (PREFETCH) {
             if (PARAMS)
@@ -793,21 +793,8 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
         __builtin_amdgcn_sched_barrier(0);
     };
     int i = i0;
-#if BOXCONV_STREAM_UNROLL
-    for (; i + 4 < i1; i += 4) {
-        row_pair(i, std::true_type{}, Flip0{});
-        row_pair(i + 2, std::true_type{}, Flip1{});
-    }
-    if (i + 2 < i1) {
-        row_pair(i, std::true_type{}, Flip0{});
-        row_pair(i + 2, std::false_type{}, Flip1{});
-    } else {
-        row_pair(i, std::false_type{}, Flip0{});
-    }
-#else
-    for (; i + 2 < i1; i += 2) row_pair(i, std::true_type{}, 0);
-    row_pair(i, std::false_type{}, 0);
-#endif
+    for (; i + 2 < i1; i += 2) row_pair(i, std::true_type{});
+    row_pair(i, std::false_type{});
 
     if (PARAMS) {
         __syncthreads();

@@ -621,7 +621,11 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
         idx_ymin = (j_ymin >= 0 && j_ymin < w) ? j_ymin + kGPad : 0;
     }
 
-    T sum[5] = {T(0), T(0), T(0), T(0), T(0)};
+    // The five sums are added up in T only within one row pair of one lane (2*K products each);
+    // from there on in double. The products are large against the final sums (V grows along the
+    // row like a running integral while the sums are differences of such terms), so longer T
+    // chains would lose the low digits.
+    double total[5] = {0.0, 0.0, 0.0, 0.0, 0.0};
     T colacc[K];                                      // SCAN: columns K*tid .. K*tid+K-1
 #pragma unroll
     for (int k = 0; k < K; ++k) colacc[k] = T(0);
@@ -684,6 +688,7 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
         __syncthreads();                                                     // rows are in LDS
 
         if (PARAMS) {
+            T sum[5] = {T(0), T(0), T(0), T(0), T(0)};
 #pragma unroll
             for (int k = 0; k < K; ++k) {
                 const T dt0 = t0[k] - ta[k], db0 = b1[k] - bc[k];
@@ -727,6 +732,8 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
                 sum[3] += vw0 * gmax.r0 + vw1 * gmax.r1;
                 sum[2] -= vw0 * gmin.r0 + vw1 * gmin.r1;
             }
+#pragma unroll
+            for (int n = 0; n < 5; ++n) total[n] += static_cast<double>(sum[n]);
         }
 
         if (SCAN) {
@@ -798,16 +805,13 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
 
     if (PARAMS) {
         __syncthreads();
-        const double v[5] = {static_cast<double>(sum[0]), static_cast<double>(sum[1]),
-                             static_cast<double>(sum[2]), static_cast<double>(sum[3]),
-                             static_cast<double>(sum[4])};
         // slots > 0: one slot per workgroup, summed by the finalize kernel in a fixed order
         // (no clearing pass, no atomics, bit-reproducible); else atomics into the box's five sums
         if (a.acc_slots > 0)
-            block_accumulate5(v, a.acc + ((static_cast<int64_t>(a.plane0 + p) * a.F + f) * a.acc_slots + band) * 5,
+            block_accumulate5(total, a.acc + ((static_cast<int64_t>(a.plane0 + p) * a.F + f) * a.acc_slots + band) * 5,
                               lds.red, false);
         else
-            block_accumulate5(v, a.acc + static_cast<int64_t>(k_par) * 5, lds.red);
+            block_accumulate5(total, a.acc + static_cast<int64_t>(k_par) * 5, lds.red);
     }
 }
 

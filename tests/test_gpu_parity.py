@@ -85,34 +85,36 @@ def run_both(hip, oracle, x, boxes, reparam_h, reparam_w, normalize, exact, grad
 
 
 def assert_parity(cpu, gpu, dtype, what="", i_max=0.0, gi_max=0.0, pg_scale=0.0):
-    """max|gpu-cpu| <= tol * max|cpu| + 8 eps * (largest integral-image entry).
+    """max|gpu-cpu| <= tol * scale + rounding noise, per tensor.
 
-    The additive term is the rounding noise both implementations carry: every output is a
-    difference of integral-image entries, each known to half a unit in its last place. It only
-    matters for tensors that are (nearly) zero, e.g. a box that misses the image entirely.
+    forward / grad_input: scale = max|cpu|, noise = 8 eps * (largest integral-image entry): every
+    output is a difference of integral-image entries, each known to half a unit in its last place;
+    it only matters for tensors that are (nearly) zero, e.g. a box that misses the image.
     i_max / gi_max: largest |entry| of the integral image of the input / of grad_output.
-    Parameter gradients are sums of grad_output times differences of integral-image entries,
-    scaled by the reparametrization factor; when every box of a tensor misses the image the true
-    gradients are zero and the float32 CPU result is rounding noise of the order eps * pg_scale
-    (pg_scale = i_max * max|grad_output| * reparametrization * sqrt(h*w): a random walk over the
-    pixels; the float64 oracle gives exact zeros there), which then is the scale they are compared
-    on. For boxes that do touch the image the gradients are of the order pg_scale itself."""
+
+    Parameter gradients: scale = max(max|cpu|, 1e-2 * largest of the four tensors), noise =
+    eps * pg_scale with pg_scale = i_max * max|grad_output| * reparametrization * sqrt(h*w). They
+    are sums over all pixels of grad_output times differences of integral-image entries, scaled
+    by the reparametrization factor, so the float32 reference itself carries a random-walk error
+    of that order (checked against the float64 oracle: e.g. input mean 3, 65x1535, whole-pixel
+    boxes: the float32 CPU result is off by 0.55 %, the GPU result by 0.09 %); for boxes that miss
+    the image the true gradients are exactly zero and the reference returns pure noise."""
     tol_f, tol_p = TOL[dtype]
     eps = float(np.finfo(dtype).eps)
     (out_c, back_c), (out_g, back_g) = cpu, gpu
 
-    def close(got, want, tol, atol):
+    def close(got, want, tol, atol, scale_floor=0.0):
         want = np.asarray(want, dtype=np.float64)
         diff = np.abs(np.asarray(got, dtype=np.float64) - want).max() if want.size else 0.0
-        return diff <= tol * (np.abs(want).max() if want.size else 0.0) + atol
+        return diff <= tol * max(np.abs(want).max() if want.size else 0.0, scale_floor) + atol
 
     assert close(out_g, out_c, tol_f, 8 * eps * i_max), what + " forward"
     if back_c[0] is not None:
         assert close(back_g[0], back_c[0], tol_f, 8 * eps * gi_max), what + " grad_input"
-    floor = max(param_grad_floor(back_c[1:]), 8 * eps * pg_scale)
+    floor = param_grad_floor(back_c[1:])
     for k, name in enumerate(("x_min", "x_max", "y_min", "y_max")):
         if back_c[1 + k] is not None:
-            assert rel_err(back_g[1 + k], back_c[1 + k], floor) <= tol_p, what + " grad_" + name
+            assert close(back_g[1 + k], back_c[1 + k], tol_p, eps * pg_scale, floor), what + " grad_" + name
 
 
 SMALL_CASES = [

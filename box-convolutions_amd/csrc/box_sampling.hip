@@ -73,6 +73,7 @@ struct SampleArgs {
     int64_t total;        // workgroups with work
     int64_t per_xcd;      // ceil(total / 8)
     int normalize;
+    int reverse;          // grad input only: walk the work items last to first
 };
 
 // Two rows of the same column, adjacent in LDS: every LDS access of the row kernels moves the
@@ -300,8 +301,9 @@ __global__ void __launch_bounds__(NT) forward_rows_kernel(SampleArgs<T> a) {
 template <class T, int NT, int K, int RB, bool EXACT, bool FULL, bool OFFS>
 __global__ void __launch_bounds__(NT) grad_input_rows_kernel(SampleArgs<T> a) {
     static_assert(RB % 4 == 0, "rows are handled in pairs, and pairs alternate between two LDS buffers");
-    const unsigned vid = xcd_contiguous_id(a.per_xcd);
+    unsigned vid = xcd_contiguous_id(a.per_xcd);
     if (vid >= a.total) return;
+    if (a.reverse) vid = static_cast<unsigned>(a.total) - 1u - vid;
     const unsigned nbands = a.nb;
     const int band = static_cast<int>(vid % nbands);
     const int64_t p = vid / nbands;
@@ -767,7 +769,9 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
                 // and wave n takes n + 1 of them
                 add_waves_left<T, 0>(lds.wave_tot, wave, carry0, carry1);
                 // the lane's K consecutive columns K*tid+1 .. K*tid+K of integral rows i+1, i+2:
-                // a wave stores one contiguous run of 64*K elements per row
+                // a wave stores one contiguous run of 64*K elements per row. Ordinary cache
+                // policy: the grad-input kernel starts with the planes written last and finds
+                // part of them still in the memory-side cache.
                 T* o0 = lrows + static_cast<int64_t>(i + 1) * pitch;
                 const bool second = i + 1 < i1;
                 const RowRef ob0 = lout.row(i + 1);
@@ -776,8 +780,8 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
 #pragma unroll
                 for (int k = 0; k < K; ++k) { out0[k] = carry0 + loc0[k]; out1[k] = carry1 + loc1[k]; }
                 const int first = (1 + K * tid) * static_cast<int>(sizeof(T));
-                buffer_store_run<kCacheStream, FULL>(out0, ob0, first, static_cast<int>(row_bytes + sizeof(T)));
-                buffer_store_run<kCacheStream, FULL>(out1, ob1, first, static_cast<int>(row_bytes + sizeof(T)));
+                buffer_store_run<kCacheDefault, FULL>(out0, ob0, first, static_cast<int>(row_bytes + sizeof(T)));
+                buffer_store_run<kCacheDefault, FULL>(out1, ob1, first, static_cast<int>(row_bytes + sizeof(T)));
                 if (tid == 0) {
                     o0[0] = T(0);
                     if (second) o0[pitch] = T(0);
@@ -1014,6 +1018,16 @@ inline bool row_kernels_apply(int h, int w, size_t elem_size) {
     return w <= kMaxRowStreamWidth && plane_bytes < (1ull << 31) && !force_gather_kernels();
 }
 
+// The grad-input kernel runs right after the pass that wrote the integral of grad_output; the
+// planes written last are the ones most likely still held by the memory-side cache.
+inline bool reverse_grad_input() {
+    static const bool v = [] {
+        const char* e = std::getenv("BOXCONV_GI_REVERSE");
+        return e == nullptr || e[0] != '0';
+    }();
+    return v;
+}
+
 inline RowConfig stream_row_config(int w) {
     static const int prefer = preferred_row_threads("BOXCONV_STREAM_THREADS", 256);
     return row_config(w, prefer);
@@ -1099,6 +1113,7 @@ hipError_t grad_input_launch(const T* gint, int band_rows, BoxParams<T> prm, T* 
     SampleArgs<T> a = base_args(prm, d);
     a.src = gint; a.dst = grad_in; a.normalize = normalize ? 1 : 0;
     a.off_R = band_rows;
+    a.reverse = (band_rows > 0 && reverse_grad_input()) ? 1 : 0;
 
     if (!row_kernels_apply(d.h, d.w, sizeof(T))) {
         if (band_rows > 0) return hipErrorInvalidValue;         // the gather kernel needs a true integral

@@ -31,6 +31,7 @@ struct IntegralPlan {
     int nb;                // horizontal bands per plane
     int R;                 // rows per band
     int64_t aux_doubles;   // scratch for the column sums of all bands but the last
+    bool lookback;         // geometry fits the single-pass kernel (bands of <= 32 rows, one tile wide)
 };
 // `want`: number of workgroups to aim for.
 IntegralPlan plan_integral(int64_t planes, int h, int w, int64_t want = 1024);

@@ -11,7 +11,11 @@
 //   2. band_prefix_kernel  : running sum of aux over bands (in place) -> sum of all bands above
 //   3. band_scan_kernel    : per band, rows top to bottom: column accumulators (registers) +=
 //                            input row, then a row-direction prefix of the accumulators.
-// With a single band (tall enough grid without cutting) only launch 3 runs.
+// With a single band (tall enough grid without cutting) only launch 3 runs. Rows of at most 2048
+// columns use band_scan_rows_kernel for launch 3, which adds up the bands above itself (no launch
+// 2). For float rows that fill a workgroup exactly and planes of at most 16 bands of 32 rows, one
+// kernel does everything in a single pass over the input (band_scan_lookback_kernel): workgroups
+// hand their column sums to the ones below them, with a bounded wait.
 //
 // Arithmetic. All sums are carried in double and rounded once on store, so every stored value
 // is the correctly rounded exact sum (the CPU reference carries row sums in double as well but
@@ -20,6 +24,8 @@
 // Memory. Loads are 4 consecutive elements per lane (16 B for float, coalesced across the wave).
 // The output pitch w+1 is odd, so results are staged through LDS and written as consecutive
 // dwords per lane (256 B contiguous per wave instruction).
+
+#include <cstdlib>
 
 #include "boxconv_device.hpp"
 #include "boxconv_host.hpp"
@@ -336,6 +342,178 @@ band_scan_rows_kernel(const T* __restrict__ in, T* __restrict__ out, const doubl
     }
 }
 
+// ---- single pass, rows no wider than one tile and bands of at most 32 rows ----------------------
+// Same tiling as band_scan_rows_kernel, but the input is read exactly once: a workgroup first
+// loads its whole band into registers and publishes the band's column sums in `aux`, then collects
+// the column sums of the bands above it in the same plane and scans its rows out of the registers.
+//
+// Hand-over. `aux` is filled with a marker value before the launch (fill_marker_kernel); every
+// column sum is published with one 64-bit device-scope atomic store and collected with 64-bit
+// device-scope atomic loads that are repeated while they return the marker. Data and "ready" are
+// the same memory word, so no ordering between different locations (no fence, no cache
+// write-back or invalidation) is needed. The marker is a NaN whose low mantissa bits are set: a sum
+// of floats converted to double can be a NaN only with a payload that came from a float, whose
+// low 29 bits are zero, so no published value equals the marker.
+//
+// Progress. A workgroup publishes before it collects and publishing depends on nothing, so a
+// collecting workgroup only needs the workgroups of the bands above to have been started. Those
+// have lower workgroup ids on the same XCD (per_xcd is a multiple of nb, so a plane never
+// straddles two XCDs) and workgroups of one XCD are started in id order. The wait is nevertheless
+// bounded: after `spin_limit` rounds of loads a lane sums the band's input rows for its own
+// columns instead, which gives the same value bit for bit (same rows, same order, double
+// accumulation). A launch therefore terminates and is correct whatever the start order;
+// spin_limit = 0 takes that path for every band (used by the tests).
+constexpr int kLookbackRows = 32;     // band height limit: 32 rows x 4 columns per lane in registers
+constexpr int kLookbackBands = 64;
+constexpr unsigned long long kNotPublished = 0x7ff8deadbeef0001ull;
+
+__global__ void __launch_bounds__(256) fill_marker_kernel(unsigned long long* dst, int64_t n) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i < n) dst[i] = kNotPublished;
+}
+
+template <int WAVES, int RB, bool VEC, bool FULL>
+__global__ void __launch_bounds__(WAVES * 64)
+band_scan_lookback_kernel(const float* __restrict__ in, float* __restrict__ out, double* aux,
+                          int h, int w, int nb, int R, int64_t planes, int64_t per_xcd,
+                          int reverse, int spin_limit) {
+    using T = float;
+    constexpr int NT = WAVES * 64;
+    constexpr int RMAX = kLookbackRows;
+    __shared__ double wave_tot[2][RB][WAVES];
+
+    const unsigned blk = xcd_contiguous_id(per_xcd);    // p * nb + band, bands of a plane in order
+    const int band = static_cast<int>(blk % static_cast<unsigned>(nb));
+    int64_t p = blk / static_cast<unsigned>(nb);
+    if (p >= planes) return;
+    if (reverse) p = planes - 1 - p;
+    const int r0 = band * R;
+    const int r1 = min(h, r0 + R);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int64_t W1 = static_cast<int64_t>(w) + 1;
+    const int c0 = 4 * tid;
+
+    const T* src = in + p * static_cast<int64_t>(h) * w;
+    const Rows<const T, false> irows(src, w, w, h);
+    T* dst = out + p * static_cast<int64_t>(h + 1) * W1;
+    const Rows<T, FULL> orows(dst, W1, w + 1, h + 1);
+    unsigned long long* sums = reinterpret_cast<unsigned long long*>(aux) +
+                               p * static_cast<int64_t>(nb - 1) * w;      // [nb-1][w]
+    const int in_off = c0 * static_cast<int>(sizeof(T));
+    const int out_off = (c0 + 1) * static_cast<int>(sizeof(T));
+
+    // Loads are unconditional (a clamped address, the value dropped afterwards) so that all rows
+    // of the band are in flight together; the row address is wave-uniform, the lane part 32 bits.
+    const bool lane_in = c0 < w;
+    const unsigned lane_col = lane_in ? static_cast<unsigned>(c0) : 0u;
+    auto load_row = [&](int row, bool exists, T (&x)[4]) {
+        if (VEC) {
+            const T* rowp = src + static_cast<int64_t>(min(row, h - 1)) * w;
+            load_quad(rowp + lane_col, x);
+            if (!(exists && lane_in)) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) x[v] = T(0);
+            }
+        } else {
+            buffer_load_run<kCacheStream>(x, irows.row(min(row, h - 1), exists), in_off);
+        }
+    };
+
+    // -- the whole band into registers, its column sums published
+    T x[RMAX][4];
+#pragma unroll
+    for (int r = 0; r < RMAX; ++r) load_row(r0 + r, r < R && r0 + r < r1, x[r]);
+
+    if (band == 0)
+        for (int c = tid; c <= w; c += NT) dst[c] = T(0);
+
+    if (band < nb - 1) {
+        double own[4] = {0.0, 0.0, 0.0, 0.0};
+#pragma unroll
+        for (int r = 0; r < RMAX; ++r)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) own[v] += static_cast<double>(x[r][v]);
+        unsigned long long* mine = sums + static_cast<int64_t>(band) * w + c0;
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+            if (c0 + v < w)
+                __hip_atomic_store(mine + v, static_cast<unsigned long long>(__double_as_longlong(own[v])),
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+
+    // -- column sums of the bands above
+    double colacc[4] = {0.0, 0.0, 0.0, 0.0};
+    for (int b = 0; b < band; ++b) {
+        const unsigned long long* theirs = sums + static_cast<int64_t>(b) * w + c0;
+        unsigned long long bits[4] = {0ull, 0ull, 0ull, 0ull};
+        bool have = false;
+        for (int it = 0; it < spin_limit; ++it) {
+            have = true;
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                if (c0 + v < w) {
+                    bits[v] = __hip_atomic_load(theirs + v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    have = have && bits[v] != kNotPublished;
+                }
+            if (have) break;
+            __builtin_amdgcn_s_sleep(8);
+        }
+        if (have) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                colacc[v] += __longlong_as_double(static_cast<long long>(bits[v]));
+        } else {
+            double part[4] = {0.0, 0.0, 0.0, 0.0};
+            for (int r = b * R; r < (b + 1) * R; ++r) {      // bands above are complete bands
+                T t[4];
+                load_row(r, true, t);
+#pragma unroll
+                for (int v = 0; v < 4; ++v) part[v] += static_cast<double>(t[v]);
+            }
+#pragma unroll
+            for (int v = 0; v < 4; ++v) colacc[v] += part[v];
+        }
+    }
+
+    // -- scan the rows out of the registers, RB at a time (one barrier per batch)
+#pragma unroll
+    for (int bi = 0; bi < RMAX / RB; ++bi) {
+        if (bi * RB >= R) break;
+        const int buf = bi & 1;
+        double pre[RB][4], excl[RB];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            double run = 0.0;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                colacc[v] += static_cast<double>(x[bi * RB + rb][v]);
+                run += colacc[v];
+                pre[rb][v] = run;
+            }
+            const double incl = wave_inclusive_scan(run);
+            excl[rb] = incl - run;
+            if (lane == 63) wave_tot[buf][rb][wave] = incl;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            const int row = r0 + bi * RB + rb;
+            double left = excl[rb];
+#pragma unroll
+            for (int wv = 0; wv < WAVES - 1; ++wv)
+                if (wv < wave) left += wave_tot[buf][rb][wv];
+            T res[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) res[v] = static_cast<T>(left + pre[rb][v]);
+            const RowRef orow = orows.row(min(row + 1, h), row < r1);
+            buffer_store_run<kCacheDefault, FULL>(res, orow, out_off, (w + 1) * static_cast<int>(sizeof(T)));
+            if (tid == 0 && row < r1) dst[static_cast<int64_t>(row + 1) * W1] = T(0);
+        }
+    }
+}
+
 template <class T>
 bool aligned_for_vec4(const T* p, int w) {
     return (w % 4 == 0) && (reinterpret_cast<uintptr_t>(p) % (4 * sizeof(T)) == 0);
@@ -377,6 +555,59 @@ hipError_t launch_scan_rows(const T* in, T* out, const double* aux, int64_t plan
     return hipGetLastError();
 }
 
+// Polls of a band flag before the band is summed directly instead.
+// (both read at every call, so that a test can switch them within one process)
+int lookback_spin_limit() {
+    const char* e = getenv("BOXCONV_INTEGRAL_SPIN");
+    return e != nullptr ? std::max(0, atoi(e)) : (1 << 16);
+}
+// BOXCONV_INTEGRAL_LOOKBACK=2: single-pass kernel for every shape it covers, not only those where
+// it was measured to be faster (used by the tests to reach its partial-row and partial-band code).
+bool lookback_any_shape() {
+    const char* e = getenv("BOXCONV_INTEGRAL_LOOKBACK");
+    return e != nullptr && atoi(e) == 2;
+}
+bool lookback_enabled() {
+    const char* e = getenv("BOXCONV_INTEGRAL_LOOKBACK");
+    return e == nullptr || atoi(e) != 0;
+}
+
+template <int WAVES>
+hipError_t launch_lookback(const float* in, float* out, double* aux, int64_t planes, int h, int w,
+                           int nb, int R, bool reverse, hipStream_t stream) {
+    const int64_t nsums = planes * static_cast<int64_t>(nb - 1) * w;
+    BOXCONV_LAUNCH("fill_marker", fill_marker_kernel, dim3(static_cast<unsigned>((nsums + 255) / 256)),
+                   dim3(256), 0, stream, reinterpret_cast<unsigned long long*>(aux), nsums);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    const int64_t per_xcd = ((planes + kXcds - 1) / kXcds) * nb;     // whole planes per XCD
+    const int rev = reverse ? 1 : 0;
+    const int spin = lookback_spin_limit();
+    const dim3 grid(static_cast<unsigned>(per_xcd * kXcds));
+    const dim3 block(WAVES * 64);
+    const bool vec = aligned_for_vec4(in, w), full = (w == WAVES * 256);
+#define LAUNCH_LOOKBACK(VEC, FULL)                                                                 \
+    BOXCONV_LAUNCH("band_scan", (band_scan_lookback_kernel<WAVES, 4, VEC, FULL>), grid, block, 0,  \
+                   stream, in, out, aux, h, w, nb, R, planes, per_xcd, rev, spin)
+    if (vec && full) LAUNCH_LOOKBACK(true, true);
+    else if (vec)    LAUNCH_LOOKBACK(true, false);
+    else             LAUNCH_LOOKBACK(false, false);
+#undef LAUNCH_LOOKBACK
+    return hipGetLastError();
+}
+template <class T>
+hipError_t lookback_by_width(const T*, T*, double*, int64_t, int, int, int, int, bool, hipStream_t) {
+    return hipErrorInvalidValue;       // float only
+}
+template <>
+hipError_t lookback_by_width<float>(const float* in, float* out, double* aux, int64_t planes, int h,
+                                    int w, int nb, int R, bool reverse, hipStream_t stream) {
+    if (w <= 256)       return launch_lookback<1>(in, out, aux, planes, h, w, nb, R, reverse, stream);
+    else if (w <= 512)  return launch_lookback<2>(in, out, aux, planes, h, w, nb, R, reverse, stream);
+    else if (w <= 1024) return launch_lookback<4>(in, out, aux, planes, h, w, nb, R, reverse, stream);
+    else                return launch_lookback<8>(in, out, aux, planes, h, w, nb, R, reverse, stream);
+}
+
 // Rows this narrow are scanned by band_scan_rows_kernel, which sums the band column sums itself;
 // the bands above a workgroup are few (nb <= h/32), so re-reading them is cheaper than a pass.
 constexpr int kMaxScanRowsWidth = 2048;
@@ -392,8 +623,19 @@ IntegralPlan plan_integral(int64_t planes, int h, int w, int64_t want) {
     // Enough workgroups to cover 256 CUs several times over, but bands no shorter than 32 rows
     // (the per-band column-sum vector is 8 B per column, i.e. 2/R of the input bytes) and no
     // taller than 256 (size of the per-row carry array in LDS).
-    int nb = static_cast<int>(std::min<int64_t>((want + planes - 1) / std::max<int64_t>(planes, 1),
-                                                std::max(1, h / 32)));
+    const int64_t wanted = (want + planes - 1) / std::max<int64_t>(planes, 1);
+    int nb = static_cast<int>(std::min<int64_t>(wanted, std::max(1, h / 32)));
+    // Where planes get cut anyway and the single-pass kernel covers the width, cut them into
+    // bands of at most 32 rows, which that kernel holds in registers.
+    // Measured against the three launches (32..256 planes): 0.55-0.95 of their time for rows that
+    // fill the workgroup exactly and planes of up to 16 bands; slower (1.1-1.4) for other widths and
+    // for taller planes, where collecting the sums of many bands costs more than the pass it saves.
+    const bool single_pass = wanted >= 2 && h > kLookbackRows && scan_by_rows(h, w, sizeof(float)) &&
+                             (h + kLookbackRows - 1) / kLookbackRows <= kLookbackBands &&
+                             (lookback_any_shape() ||
+                              ((w == 256 || w == 512 || w == 1024 || w == 2048) &&
+                               h <= 16 * kLookbackRows));
+    if (single_pass) nb = (h + kLookbackRows - 1) / kLookbackRows;
     nb = std::max(nb, (h + 255) / 256);
     nb = std::max(nb, 1);
     int R = (h + nb - 1) / nb;
@@ -403,6 +645,8 @@ IntegralPlan plan_integral(int64_t planes, int h, int w, int64_t want) {
     pl.nb = nb;
     pl.R = R;
     pl.aux_doubles = (nb > 1) ? planes * static_cast<int64_t>(nb - 1) * w : 0;
+    pl.lookback = single_pass && nb > 1 && nb <= kLookbackBands && R <= kLookbackRows &&
+                  planes * nb < (1ll << 31);
     return pl;
 }
 
@@ -412,6 +656,8 @@ hipError_t integral_image_launch(const T* in, T* out, int64_t planes, int h, int
                                  bool reverse_order, hipStream_t stream) {
     if (planes == 0) return hipSuccess;
     const int nb = pl.nb, R = pl.R;
+    if (pl.lookback && sizeof(T) == sizeof(float) && !colsums_ready && lookback_enabled())
+        return lookback_by_width<T>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
     if (nb > 1 && !colsums_ready) {
         const int strips = (w + 1023) / 1024;
         const dim3 grid(static_cast<unsigned>(planes * (nb - 1) * strips));

@@ -28,12 +28,20 @@ INTEGRAL_SHAPES = [
     (1, 2, 2), (3, 5, 7), (2, 10, 10), (6, 28, 28), (1, 33, 257), (2, 64, 128), (1, 200, 36),
     (1, 300, 1023), (2, 130, 1024), (1, 70, 2048), (1, 40, 2500), (1, 36, 4100), (1, 9, 9000),
     (5, 1, 1), (2, 1, 300), (2, 300, 1),
+    # single-pass kernel: many bands, partial last band, 64 bands, one band too many for it
+    (3, 512, 1000), (1, 2048, 64), (1, 2100, 40), (40, 100, 520), (9, 97, 1536),
 ]
 
 
+@pytest.mark.parametrize("single_pass", ["where_faster", "wherever_possible"])
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("planes,h,w", INTEGRAL_SHAPES)
-def test_integral_image(hip, oracle, planes, h, w, dtype):
+def test_integral_image(hip, oracle, monkeypatch, planes, h, w, dtype, single_pass):
+    if single_pass == "wherever_possible":
+        if dtype == np.float64:
+            pytest.skip("the single-pass kernel is float32 only")
+        # by default that kernel serves only the shapes it is faster on; reach the others too
+        monkeypatch.setenv("BOXCONV_INTEGRAL_LOOKBACK", "2")
     rng = np.random.default_rng(planes * 1000003 + h * 1009 + w)
     x = (rng.random((planes, h, w)) * 2 - 0.5).astype(dtype)
     got = host(hip.integral_image(dev(x)))
@@ -52,6 +60,25 @@ def test_integral_image(hip, oracle, planes, h, w, dtype):
         ideal = exact.astype(np.float32)
         assert np.mean(got != ideal) < 1e-4
         assert np.all(np.abs(got - ideal) <= np.spacing(np.abs(ideal)))
+
+
+@pytest.mark.parametrize("planes,h,w", [(1, 33, 257), (3, 200, 36), (2, 130, 1024), (2, 512, 1000),
+                                        (1, 2048, 64), (17, 96, 2048)])
+def test_integral_image_single_pass_waits_are_bounded(hip, monkeypatch, planes, h, w):
+    """The single-pass kernel waits a bounded number of polls for the bands above; a band whose
+    flag is still down is summed from the input instead. With a limit of zero polls every band
+    goes that way, and the result is the same bit for bit. So is the three-launch path's."""
+    x = torch.from_numpy(np.random.default_rng(h * w).random((planes, h, w), dtype=np.float32) - 0.3).cuda()
+    monkeypatch.setenv("BOXCONV_INTEGRAL_LOOKBACK", "2")       # single pass for every shape it covers
+    usual = hip.integral_image(x)
+    monkeypatch.setenv("BOXCONV_INTEGRAL_SPIN", "0")
+    assert torch.equal(hip.integral_image(x), usual)
+    monkeypatch.delenv("BOXCONV_INTEGRAL_SPIN")
+    monkeypatch.setenv("BOXCONV_INTEGRAL_LOOKBACK", "0")       # same bands, three launches
+    three = hip.integral_image(x)
+    monkeypatch.delenv("BOXCONV_INTEGRAL_LOOKBACK")
+    # (the default may cut the planes into different bands: same sums, associated differently)
+    assert torch.allclose(three, usual, rtol=2e-7, atol=0) and torch.allclose(hip.integral_image(x), usual, rtol=2e-7, atol=0)
 
 
 def test_integral_image_leading_dims(hip, oracle):

@@ -19,8 +19,8 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "build")
 LIB_PATH = os.path.join(HERE, "box_convolution", "libboxconv_hip.so")
 
-SOURCES = ["integral_image.hip", "box_sampling.hip", "box_misc.hip", "boxconv_c_abi.hip"]
-HEADERS = ["boxconv_device.hpp", "boxconv_host.hpp", os.path.join("..", "..", "include", "boxconv.h")]
+SOURCES = ["box_sampling.hip", "box_forward.hip", "integral_image.hip", "box_misc.hip", "boxconv_c_abi.hip"]
+HEADERS = ["boxconv_device.hpp", "boxconv_host.hpp", "box_sampling_common.hpp", os.path.join("..", "..", "include", "boxconv.h")]
 
 ARCH = os.environ.get("BOXCONV_OFFLOAD_ARCH", "gfx950")
 # packed-fp32 instructions stay disabled: scalar float code only.
@@ -63,7 +63,7 @@ def build(force=False, verbose=True):
             print(" ".join(cmd), flush=True)
         subprocess.check_call(cmd)
 
-    with ThreadPoolExecutor(max_workers=min(4, max(1, len(jobs)))) as pool:
+    with ThreadPoolExecutor(max_workers=min(5, max(1, len(jobs)))) as pool:
         list(pool.map(run, jobs))
 
     if force or jobs or _stale(LIB_PATH, objs):

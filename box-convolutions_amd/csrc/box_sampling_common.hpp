@@ -1,0 +1,283 @@
+// Shared by the translation units that hold the box-sampling kernels: lane/slot addressing, row
+// loads, the LDS row-pair layout, the gather helpers, and the host-side choice of workgroup shape.
+// Everything here lives in an unnamed namespace: each translation unit gets its own copy.
+#pragma once
+
+#include <cstdlib>
+#include <type_traits>
+
+#include "boxconv_device.hpp"
+#include "boxconv_host.hpp"
+
+namespace boxconv {
+
+namespace {
+
+
+extern __shared__ __align__(16) unsigned char smem_raw[];
+
+// Largest workgroup of the row-streaming kernels (8 waves). A wide row is spread over more lanes
+// rather than over more than 4 columns per lane: per-lane state (sliding rows, prefetched rows,
+// accumulators) scales with the columns per lane, and these kernels hide HBM latency with
+// occupancy.
+constexpr int kMaxRowThreads = 512;
+constexpr int kMaxRowWaves = kMaxRowThreads / 64;
+
+template <class T>
+struct SampleArgs {
+    const T* src;         // integral planes, (h+1) x (w+1) each, contiguous
+    BoxParams<T> prm;
+    T* dst;               // forward: [planes,F,h,w]; grad input: [planes,h,w]
+    const T* grad_out;    // param grads only: [planes,F,h,w]
+    double* acc;          // param grads only: [C*F*5], or [planes*F*acc_slots*5] workgroup slots
+    int acc_slots;        // param grads only: slots per (plane, filter), 0 = atomics on [C*F*5]
+    int off_R;                // grad input only: rows per band of a band-local integral, 0 = true integral
+    int C, F, h, w;
+    int nb, R;            // bands per plane and rows per band
+    int64_t plane0;       // global index of the first plane (selects the boxes)
+    int64_t total;        // workgroups with work
+    int64_t per_xcd;      // ceil(total / 8)
+    int normalize;
+    int reverse;          // grad input only: walk the work items last to first
+};
+
+// Two rows of the same column, adjacent in LDS: every LDS access of the row kernels moves the
+// values of both rows of the current row pair at once.
+template <class T>
+struct alignas(2 * sizeof(T)) RowPair {
+    T r0, r1;
+};
+
+// Per-lane column slots. Lane `tid` owns integral columns q = 1 + tid + NT*k (pixel columns
+// j = q - 1), k < K, NT = workgroup size. q1 = (1 + tid) * sizeof(T) is the byte offset of the
+// lane's first column in a row of T; the other slots are compile-time distances away, so one
+// register addresses all of them (instruction offsets for LDS and for buffers).
+// FULL: w == K * NT, so every (lane, k) slot is a valid column and no bounds checks are compiled
+// in; otherwise a slot is valid iff its byte offset is <= w * sizeof(T).
+template <class T>
+__device__ __forceinline__ int lane_q1() {
+    return (1 + static_cast<int>(threadIdx.x)) * static_cast<int>(sizeof(T));
+}
+template <class T, int NT>
+__device__ __forceinline__ constexpr int slot_bytes(int k) {
+    return NT * k * static_cast<int>(sizeof(T));
+}
+template <class T, int NT, bool FULL>
+__device__ __forceinline__ bool slot_valid(int q1, int k, unsigned row_bytes) {
+    return FULL || static_cast<unsigned>(q1 + slot_bytes<T, NT>(k)) <= row_bytes;
+}
+template <class T, int NT, int POLICY>
+__device__ __forceinline__ T load_slot(const RowRef& r, int q1, int k) {
+    return buffer_load<POLICY>(r, q1 + slot_bytes<T, NT>(k), T());
+}
+template <class T, int NT, int POLICY>
+__device__ __forceinline__ void store_slot(T v, const RowRef& r, int q1, int k) {
+    buffer_store<POLICY>(v, r, q1 + slot_bytes<T, NT>(k));
+}
+
+// Columns 1.. of one row into the lane's slots; slots past the end of the row read 0.
+template <class T, int NT, int K>
+__device__ __forceinline__ void load_row(const RowRef& r, int q1, T (&dst)[K]) {
+#pragma unroll
+    for (int k = 0; k < K; ++k) dst[k] = load_slot<T, NT, kCacheDefault>(r, q1, k);
+}
+
+// The four rows that become new when the window moves from output rows (i-2, i-1) to (i, i+1):
+// I[t(i)], I[t(i+1)], I[b(i+1)], I[b(i+2)].
+template <class T, int NT, int K, bool FULL>
+__device__ __forceinline__ void load_pair(const LoadRows<T>& rows, int i, int xlo, int xhi,
+                                          int h, int q1, T (&t0)[K], T (&t1)[K], T (&b1)[K],
+                                          T (&b2)[K]) {
+    load_row<T, NT, K>(rows.row(clampi(i + xlo, 0, h)), q1, t0);
+    load_row<T, NT, K>(rows.row(clampi(i + 1 + xlo, 0, h)), q1, t1);
+    load_row<T, NT, K>(rows.row(clampi(i + 1 + xhi, 0, h)), q1, b1);
+    load_row<T, NT, K>(rows.row(clampi(i + 2 + xhi, 0, h)), q1, b2);
+}
+
+template <class T, bool EXACT>
+__device__ __forceinline__ T blend(T lo_adv, T lo, T hi, T hi_adv, T flo, T fhi) {
+    T v = hi - lo;
+    if (EXACT) v += fhi * (hi_adv - hi) + flo * (lo - lo_adv);
+    return v;
+}
+
+// Row vectors V(i), V(i+1) into LDS. Layout: V[q+1] for q = -1..w+1 with V(-1) = V(0) = 0 (written
+// once by clear_row_pads) and V(w+1) = V(w), so a clamped column pair is always two adjacent
+// entries.
+template <class T, int NT, int K, bool FULL>
+__device__ __forceinline__ void publish_rows(RowPair<T>* __restrict__ V, const T (&v0)[K],
+                                             const T (&v1)[K], int w, unsigned row_bytes, int q1) {
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const RowPair<T> pr{v0[k], v1[k]};
+        if (slot_valid<T, NT, FULL>(q1, k, row_bytes)) *at_bytes(V + 1 + NT * k, 2 * q1) = pr;
+        if (FULL ? (k == K - 1 && static_cast<int>(threadIdx.x) == NT - 1)
+                 : (static_cast<unsigned>(q1 + slot_bytes<T, NT>(k)) == row_bytes))
+            V[w + 2] = pr;
+    }
+}
+template <class T>
+__device__ __forceinline__ void clear_row_pads(RowPair<T>* vbuf, int vlen) {
+    if (threadIdx.x < 4) vbuf[(threadIdx.x >> 1) * vlen + (threadIdx.x & 1)] = RowPair<T>{T(0), T(0)};
+}
+
+// LDS byte offsets of the column pairs (lAdv, l) = (lo, lo+1) and (r, rAdv) = (hi, hi+1) of the
+// lane's pixels.
+template <class T, int NT, int K>
+__device__ __forceinline__ void column_taps(unsigned (&lo)[K], unsigned (&hi)[K], int ylo, int yhi,
+                                            int w) {
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const int j = static_cast<int>(threadIdx.x) + NT * k;
+        lo[k] = static_cast<unsigned>(clampi(j + ylo, 0, w + 1)) * static_cast<unsigned>(sizeof(RowPair<T>));
+        hi[k] = static_cast<unsigned>(clampi(j + yhi, -1, w) + 1) * static_cast<unsigned>(sizeof(RowPair<T>));
+    }
+}
+
+// Box sums of one pixel column slot for both rows of the pair.
+template <class T, bool EXACT>
+__device__ __forceinline__ RowPair<T> sample_columns(const RowPair<T>* __restrict__ V, unsigned lo,
+                                                     unsigned hi, T fylo, T fyhi) {
+    const RowPair<T>* L = at_bytes(V, lo);
+    const RowPair<T>* H = at_bytes(V, hi);
+    const RowPair<T> l = L[1], r = H[0];
+    RowPair<T> la = l, ra = r;
+    if (EXACT) { la = L[0]; ra = H[1]; }
+    return {blend<T, EXACT>(la.r0, l.r0, r.r0, ra.r0, fylo, fyhi),
+            blend<T, EXACT>(la.r1, l.r1, r.r1, ra.r1, fylo, fyhi)};
+}
+
+template <class T>
+struct BoxOfWorkgroup {
+    T xmin, xmax, ymin, ymax;
+};
+template <class T>
+__device__ __forceinline__ BoxOfWorkgroup<T> load_box(const BoxParams<T>& prm, int k_par) {
+    return {prm.xmin[k_par], prm.xmax[k_par], prm.ymin[k_par], prm.ymax[k_par]};
+}
+
+using Flip0 = std::integral_constant<int, 0>;
+using Flip1 = std::integral_constant<int, 1>;
+
+// ---------------------------------------------------------------------------------------------
+// Gather kernels: one thread per output pixel, the 16 integral samples are read straight from
+// global memory. Any width; also the cross-check implementation for the row-streaming kernels.
+template <class T, bool EXACT>
+__device__ __forceinline__ T gather_V(const T* __restrict__ plane, int64_t pitch, int ta, int t,
+                                      int b, int ba, int q, T fxlo, T fxhi) {
+    const T vt = plane[t * pitch + q], vb = plane[b * pitch + q];
+    T vta = T(0), vba = T(0);
+    if (EXACT) { vta = plane[ta * pitch + q]; vba = plane[ba * pitch + q]; }
+    return blend<T, EXACT>(vta, vt, vb, vba, fxlo, fxhi);
+}
+
+template <class T, bool EXACT>
+__device__ __forceinline__ T gather_box(const T* __restrict__ plane, const BoxSplit<T>& s, int i,
+                                        int j, int h, int w) {
+    const int64_t pitch = w + 1;
+    const int t = clampi(i + s.xlo, 0, h), ta = clampi(i + s.xlo - 1, 0, h);
+    const int b = clampi(i + s.xhi, 0, h), ba = clampi(i + s.xhi + 1, 0, h);
+    const int l = clampi(j + s.ylo, 0, w), la = clampi(j + s.ylo - 1, 0, w);
+    const int r = clampi(j + s.yhi, 0, w), ra = clampi(j + s.yhi + 1, 0, w);
+    const T vl = gather_V<T, EXACT>(plane, pitch, ta, t, b, ba, l, s.fxlo, s.fxhi);
+    const T vr = gather_V<T, EXACT>(plane, pitch, ta, t, b, ba, r, s.fxlo, s.fxhi);
+    T vla = T(0), vra = T(0);
+    if (EXACT) {
+        vla = gather_V<T, EXACT>(plane, pitch, ta, t, b, ba, la, s.fxlo, s.fxhi);
+        vra = gather_V<T, EXACT>(plane, pitch, ta, t, b, ba, ra, s.fxlo, s.fxhi);
+    }
+    return blend<T, EXACT>(vla, vl, vr, vra, s.fylo, s.fyhi);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Workgroup shapes the row kernels are compiled for: (threads, columns per lane).
+//   (64,1) widths up to 64; (256,1..4) up to 256..1024; (512,1..4) up to 512..2048.
+// Each kernel has a preferred size (measured at width 1024: 512 threads for forward and grad
+// input, 256 for the grad_output pass); rows too wide for 4 columns per lane at that size take
+// 512 threads, which bounds the register footprint and the length of the per-lane float
+// accumulation chains.
+struct RowConfig { int nt; int K; bool full; };
+inline int preferred_row_threads(const char* env_name, int fallback) {
+    const char* e = std::getenv(env_name);
+    const int n = e ? std::atoi(e) : fallback;
+    return (n == 256 || n == 512) ? n : fallback;
+}
+inline RowConfig row_config(int w, int prefer) {
+    RowConfig c;
+    if (w <= 64) {
+        c.nt = 64; c.K = 1;
+    } else {
+        // fewest column slots (K * threads) that cover the row; the preferred size wins ties
+        const int other = prefer == 256 ? 512 : 256;
+        const int kp = (w + prefer - 1) / prefer, ko = (w + other - 1) / other;
+        const bool use_other = kp > 4 || (ko <= 4 && ko * other < kp * prefer);
+        c.nt = use_other ? other : prefer;
+        c.K = std::min(std::max(use_other ? ko : kp, 1), 4);
+    }
+    c.full = (c.K * c.nt == w);
+    return c;
+}
+
+// The row kernels address a plane with 32-bit byte offsets and hold a full row per workgroup.
+inline bool row_kernels_apply(int h, int w, size_t elem_size) {
+    const uint64_t plane_bytes = (static_cast<uint64_t>(h) + 1) * (static_cast<uint64_t>(w) + 1) * elem_size;
+    return w <= kMaxRowStreamWidth && plane_bytes < (1ull << 31) && !force_gather_kernels();
+}
+
+// The grad-input kernel runs right after the pass that wrote the integral of grad_output; the
+// planes written last are the ones most likely still held by the memory-side cache.
+inline bool reverse_grad_input() {
+    static const bool v = [] {
+        const char* e = std::getenv("BOXCONV_GI_REVERSE");
+        return e == nullptr || e[0] != '0';
+    }();
+    return v;
+}
+
+inline RowConfig stream_row_config(int w) {
+    static const int prefer = preferred_row_threads("BOXCONV_STREAM_THREADS", 256);
+    return row_config(w, prefer);
+}
+
+inline int bands_for(int64_t independent, int h, int min_rows, int64_t want) {
+    int nb = static_cast<int>(std::min<int64_t>((want + independent - 1) / std::max<int64_t>(independent, 1),
+                                                std::max(1, h / min_rows)));
+    return std::max(nb, 1);
+}
+
+template <class T>
+SampleArgs<T> base_args(BoxParams<T> prm, const Dims& d) {
+    SampleArgs<T> a{};
+    a.prm = prm; a.C = d.C; a.F = d.F; a.h = d.h; a.w = d.w; a.plane0 = d.plane0;
+    return a;
+}
+
+template <class T>
+void finish_args(SampleArgs<T>& a, int64_t total) {
+    a.total = total;
+    a.per_xcd = (total + kXcds - 1) / kXcds;
+}
+
+#define BOXCONV_DISPATCH_K(KERNEL, NT, K, ...)                                       \
+    switch (K) {                                                                     \
+        case 1: KERNEL(NT, 1, __VA_ARGS__); break;                                   \
+        case 2: KERNEL(NT, 2, __VA_ARGS__); break;                                   \
+        case 3: KERNEL(NT, 3, __VA_ARGS__); break;                                   \
+        default: KERNEL(NT, 4, __VA_ARGS__); break;                                  \
+    }
+#define BOXCONV_DISPATCH_SHAPE(KERNEL, RC, ...)                                      \
+    if ((RC).nt == 64)       { KERNEL(64, 1, __VA_ARGS__); }                         \
+    else if ((RC).nt == 256) { BOXCONV_DISPATCH_K(KERNEL, 256, (RC).K, __VA_ARGS__) } \
+    else                     { BOXCONV_DISPATCH_K(KERNEL, 512, (RC).K, __VA_ARGS__) }
+#define BOXCONV_DISPATCH_SHAPE_EXACT_FULL(KERNEL, RC, EXACT)                         \
+    if (EXACT) {                                                                     \
+        if ((RC).full) { BOXCONV_DISPATCH_SHAPE(KERNEL, RC, true, true) }            \
+        else           { BOXCONV_DISPATCH_SHAPE(KERNEL, RC, true, false) }           \
+    } else {                                                                         \
+        if ((RC).full) { BOXCONV_DISPATCH_SHAPE(KERNEL, RC, false, true) }           \
+        else           { BOXCONV_DISPATCH_SHAPE(KERNEL, RC, false, false) }          \
+    }
+
+}  // namespace
+
+}  // namespace boxconv

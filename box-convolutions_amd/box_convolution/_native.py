@@ -40,7 +40,12 @@ for _s in ("f32", "f64"):
     _SIGNATURES["boxconv_clip_parameters_" + _s] = (_i, [_vp] * 4 + [_i] + [_d] * 4 + [_i, _vp])
     _SIGNATURES["boxconv_clip_reparametrize_" + _s] = (_i, [_vp] * 5 + [_i] + [_d] * 4 + [_i, _vp])
 
+_SIGNATURES["boxconv_forward_fused_f32"] = (_i, [_vp] * 6 + [_i] + [_vp] * 3 + [_i] * 8 + [_vp])
+
 EXPORTED_SYMBOLS = tuple(sorted(_SIGNATURES))
+
+# output_dtype codes of boxconv_forward_fused_f32 (include/boxconv.h)
+_FUSED_OUTPUT = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 
 _SUFFIX = {torch.float32: "f32", torch.float64: "f64"}
 
@@ -176,6 +181,62 @@ def box_convolution_forward(input_integrated, x_min, x_max, y_min, y_max, normal
             _ptr(output), B, C, F, h, w, int(bool(normalize)), int(bool(exact)),
             _stream(output.device))
     _check(rc, "box_convolution_forward")
+    return output
+
+
+def box_convolution_forward_fused(input_integrated, x_min, x_max, y_min, y_max, normalize, exact,
+                                  output_dtype=torch.float32, channel_scale=None,
+                                  channel_shift=None, residual=None, relu=False):
+    """Forward box sums from a float32 integral image, written as ``output_dtype`` (float32,
+    float16 or bfloat16), with an optional tail fused into the store:
+    ``y = S * channel_scale[ch] + channel_shift[ch] + residual``, then ``relu`` (the tail of the
+    reference's BottleneckBoxConv in eval mode, examples/Cityscapes/models/ENet.py:290-304).
+    Parameters are in real pixel units, float32. Inference only: nothing here is differentiable.
+
+    Returns ``[B, C*F, h, w]`` of ``output_dtype``."""
+    if input_integrated.device != x_min.device:
+        raise RuntimeError("BoxConv2d: input and parameters are on different devices")
+    _require_device(input_integrated, "input")
+    if input_integrated.dim() != 4:
+        raise RuntimeError("BoxConv2d: input must have 4 dimensions")
+    if input_integrated.dtype != torch.float32:
+        raise RuntimeError("box_convolution: the fused forward takes a float32 integral image, got %s"
+                           % input_integrated.dtype)
+    if output_dtype not in _FUSED_OUTPUT:
+        raise RuntimeError("box_convolution: the fused forward writes float32, float16 or bfloat16, "
+                           "not %s" % output_dtype)
+    _check_params(x_min, x_max, y_min, y_max, input_integrated.size(1), "BoxConv2d: ")
+    lib = load()
+    input_integrated = input_integrated.contiguous()
+    x_min, x_max, y_min, y_max = _same_kind((x_min, x_max, y_min, y_max), input_integrated, "input")
+    B, C, h1, w1 = input_integrated.shape
+    F = x_min.size(1)
+    h, w = h1 - 1, w1 - 1
+    if h < 1 or w < 1:
+        raise RuntimeError("BoxConv2d: integral image must be at least 2x2")
+    dev = input_integrated.device
+    per_channel = []
+    for name, t in (("channel_scale", channel_scale), ("channel_shift", channel_shift)):
+        if t is not None:
+            if t.device != dev or t.numel() != C * F:
+                raise RuntimeError("box_convolution: %s must hold %d values on %s" % (name, C * F, dev))
+            t = t.detach().to(torch.float32).contiguous()
+        per_channel.append(t)
+    if residual is not None:
+        if residual.device != dev or tuple(residual.shape) != (B, C * F, h, w):
+            raise RuntimeError("box_convolution: residual must have the shape of the output, "
+                               "%s, on %s" % ((B, C * F, h, w), dev))
+        residual = residual.detach().to(output_dtype).contiguous()
+    output = torch.empty((B, C * F, h, w), dtype=output_dtype, device=dev)
+    if output.numel() == 0:
+        return output
+    with torch.cuda.device(dev):
+        rc = lib.boxconv_forward_fused_f32(
+            _ptr(input_integrated), _ptr(x_min), _ptr(x_max), _ptr(y_min), _ptr(y_max),
+            _ptr(output), _FUSED_OUTPUT[output_dtype], _ptr(residual), _ptr(per_channel[0]),
+            _ptr(per_channel[1]), int(bool(relu)), B, C, F, h, w, int(bool(normalize)),
+            int(bool(exact)), _stream(dev))
+    _check(rc, "box_convolution_forward_fused")
     return output
 
 

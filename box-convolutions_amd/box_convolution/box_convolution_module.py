@@ -98,7 +98,11 @@ class BoxConv2d(torch.nn.Module):
             self._clip_parameters()
         return self
 
+    _HALF_TYPES = (torch.float16, torch.bfloat16)
+
     def forward(self, input):
+        if input.dtype in self._HALF_TYPES:
+            return self._forward_half(input)
         real_parameters = None
         if self.training:
             if self.x_min.is_cuda:
@@ -114,3 +118,54 @@ class BoxConv2d(torch.nn.Module):
             input, self.x_min, self.x_max, self.y_min, self.y_max,
             self.reparametrization_h, self.reparametrization_w, self.normalize, self.exact,
             real_parameters)
+
+    def _forward_half(self, input):
+        """float16 / bfloat16 input (not offered by the reference's CPU path, and its CUDA path
+        would integrate in half precision): sums are always formed in float32. Without autograd
+        the kernel writes the half-precision output directly; when a gradient is needed the
+        float32 path runs between two casts."""
+        params = (self.x_min, self.x_max, self.y_min, self.y_max)
+        if torch.is_grad_enabled() and (input.requires_grad or any(p.requires_grad for p in params)):
+            if self.training:
+                self._clip_parameters()
+            output = BoxConvolutionFunction.apply(
+                input.float(), *(p.float() for p in params),
+                self.reparametrization_h, self.reparametrization_w, self.normalize, self.exact)
+            return output.to(input.dtype)
+        if self.training:
+            self._clip_parameters()
+        return self.forward_fused(input)
+
+    def forward_fused(self, input, channel_scale=None, channel_shift=None, residual=None,
+                      relu=False, output_dtype=None):
+        """Inference-only forward with the next element-wise steps of a block folded into the
+        kernel's store: ``y = boxconv(input) * channel_scale[ch] + channel_shift[ch] + residual``,
+        then ``max(y, 0)`` if ``relu``. That is the tail of the reference's BottleneckBoxConv in
+        eval mode (BoxConv2d -> BatchNorm2d -> Dropout2d -> ``+ x`` -> ReLU,
+        examples/Cityscapes/models/ENet.py:290-304); ``fold_batch_norm`` turns an eval-mode
+        BatchNorm2d into the two per-channel vectors.
+
+        ``input`` may be float32, float16 or bfloat16; the integral image and the sums are
+        float32, the result is ``output_dtype`` (default: the input's). Not differentiable."""
+        if output_dtype is None:
+            output_dtype = input.dtype
+        with torch.no_grad():
+            real = reparametrize(
+                self.x_min.float(), self.x_max.float(), self.y_min.float(), self.y_max.float(),
+                self.reparametrization_h, self.reparametrization_w, inverse=True)
+            integrated = _native.integral_image(input.float())
+            return _native.box_convolution_forward_fused(
+                integrated, *real, self.normalize, self.exact, output_dtype,
+                channel_scale, channel_shift, residual, relu)
+
+    @staticmethod
+    def fold_batch_norm(batch_norm):
+        """``(scale, shift)`` with ``batch_norm(x) == x * scale[ch] + shift[ch]`` in eval mode."""
+        with torch.no_grad():
+            scale = torch.rsqrt(batch_norm.running_var.float() + batch_norm.eps)
+            if batch_norm.weight is not None:
+                scale = scale * batch_norm.weight.float()
+            shift = -batch_norm.running_mean.float() * scale
+            if batch_norm.bias is not None:
+                shift = shift + batch_norm.bias.float()
+        return scale, shift

@@ -12,8 +12,24 @@ namespace {
 // ---------------------------------------------------------------------------------------------
 // Forward. Work item = (plane p, filter f, band). blockDim = NT, K >= ceil(w / NT).
 // LDS: [2 buffers][w+3] RowPair<T>.
-template <class T, int NT, int K, bool EXACT, bool FULL>
-__global__ void __launch_bounds__(NT) forward_rows_kernel(SampleArgs<T> a) {
+//
+// TO: element type of the output (T, or a 16-bit type when T is float). TAIL: what happens to a
+// box sum S on its way out, fused into the store (inference only, there is no backward for it):
+//   y = S * channel_scale[c*F+f] + channel_shift[c*F+f]  (+ residual[same pixel])  (max(y, 0))
+// which is the tail of a block such as BoxConv -> BatchNorm (eval) -> residual add -> ReLU.
+// Absent pieces are neutral: a null scale/shift reads as 1/0, a null residual as zeros (its row
+// descriptors get size 0, so the loads return 0 without a branch).
+template <class TO>
+struct ForwardTail {
+    TO* dst;
+    const TO* residual;
+    const float* channel_scale;
+    const float* channel_shift;
+    int relu;
+};
+
+template <class T, class TO, int NT, int K, bool EXACT, bool FULL, bool TAIL>
+__global__ void __launch_bounds__(NT) forward_rows_kernel(SampleArgs<T> a, ForwardTail<TO> tl) {
     const unsigned vid = xcd_contiguous_id(a.per_xcd);
     if (vid >= a.total) return;
     const unsigned nbands = a.nb, nfilt = a.F;
@@ -34,7 +50,16 @@ __global__ void __launch_bounds__(NT) forward_rows_kernel(SampleArgs<T> a) {
     const T* plane = a.src + p * static_cast<int64_t>(h + 1) * pitch;
     // output rows start one element early so that column slot q = j + 1 lands on pixel j
     const LoadRows<T> irows(plane, pitch, w + 1, h + 1);
-    const Rows<T, FULL> orows(a.dst + pf * static_cast<int64_t>(h) * w - 1, w, w + 1, h);
+    const Rows<TO, FULL> orows(tl.dst + pf * static_cast<int64_t>(h) * w - 1, w, w + 1, h);
+    const Rows<const TO, false> rrows((tl.residual != nullptr ? tl.residual : tl.dst) +
+                                          pf * static_cast<int64_t>(h) * w - 1,
+                                      w, tl.residual != nullptr ? w + 1 : 0, h);
+    T ch_scale = T(1), ch_shift = T(0);
+    if (TAIL) {
+        if (tl.channel_scale != nullptr) ch_scale = static_cast<T>(tl.channel_scale[k_par]);
+        if (tl.channel_shift != nullptr) ch_shift = static_cast<T>(tl.channel_shift[k_par]);
+    }
+    const bool relu = TAIL && tl.relu != 0;
     RowPair<T>* vbuf = reinterpret_cast<RowPair<T>*>(smem_raw);
     const int vlen = w + 3;
     clear_row_pads(vbuf, vlen);
@@ -43,6 +68,7 @@ __global__ void __launch_bounds__(NT) forward_rows_kernel(SampleArgs<T> a) {
     const int i1 = min(h, i0 + a.R);
 
     const int q1 = lane_q1<T>();
+    const int qo = lane_q1<TO>();         // the same column slots in a row of TO
     unsigned lo[K], hi[K];
     column_taps<T, NT, K>(lo, hi, s.ylo, s.yhi, w);
 
@@ -64,6 +90,18 @@ __global__ void __launch_bounds__(NT) forward_rows_kernel(SampleArgs<T> a) {
         if (PREFETCH)
             load_pair<T, NT, K, FULL>(irows, i + 2, s.xlo, s.xhi, h, q1, n0, n1, n2, n3);
 
+        // residual of the two output rows: issued with the row loads, used after the barrier
+        TO res0[K] = {}, res1[K] = {};
+        if (TAIL) {
+            const RowRef rb0 = rrows.row(i);
+            const RowRef rb1 = rrows.row(min(i + 1, h - 1), i + 1 < i1);
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                res0[k] = load_slot<TO, NT, kCacheStream>(rb0, qo, k);
+                res1[k] = load_slot<TO, NT, kCacheStream>(rb1, qo, k);
+            }
+        }
+
         RowPair<T>* V = vbuf + (FLIP ? vlen : 0);
         T v0[K], v1[K];
 #pragma unroll
@@ -80,8 +118,17 @@ __global__ void __launch_bounds__(NT) forward_rows_kernel(SampleArgs<T> a) {
         for (int k = 0; k < K; ++k) {
             if (slot_valid<T, NT, FULL>(q1, k, row_bytes)) {
                 const RowPair<T> o = sample_columns<T, EXACT>(V, lo[k], hi[k], s.fylo, s.fyhi);
-                store_slot<T, NT, kCacheStream>(o.r0 * scale, ob0, q1, k);
-                store_slot<T, NT, kCacheStream>(o.r1 * scale, ob1, q1, k);
+                T y0 = o.r0 * scale, y1 = o.r1 * scale;
+                if (TAIL) {
+                    y0 = y0 * ch_scale + ch_shift + static_cast<T>(widen(res0[k]));
+                    y1 = y1 * ch_scale + ch_shift + static_cast<T>(widen(res1[k]));
+                    if (relu) { y0 = y0 < T(0) ? T(0) : y0; y1 = y1 < T(0) ? T(0) : y1; }
+                }
+                TO z0, z1;
+                narrow(y0, z0);
+                narrow(y1, z1);
+                store_slot<TO, NT, kCacheStream>(z0, ob0, qo, k);
+                store_slot<TO, NT, kCacheStream>(z1, ob1, qo, k);
             }
         }
         if (PREFETCH) {
@@ -105,8 +152,8 @@ __global__ void __launch_bounds__(NT) forward_rows_kernel(SampleArgs<T> a) {
     }
 }
 
-template <class T, bool EXACT>
-__global__ void __launch_bounds__(256) forward_gather_kernel(SampleArgs<T> a) {
+template <class T, class TO, bool EXACT, bool TAIL>
+__global__ void __launch_bounds__(256) forward_gather_kernel(SampleArgs<T> a, ForwardTail<TO> tl) {
     const int64_t hw = static_cast<int64_t>(a.h) * a.w;
     const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (idx >= a.total) return;
@@ -120,24 +167,33 @@ __global__ void __launch_bounds__(256) forward_gather_kernel(SampleArgs<T> a) {
     const T scale = a.normalize
         ? inverse_extent(bx.xmin, bx.xmax, bx.ymin, bx.ymax, EXACT, true, true) : T(1);
     const T* plane = a.src + p * static_cast<int64_t>(a.h + 1) * (a.w + 1);
-    a.dst[idx] = gather_box<T, EXACT>(plane, s, i, j, a.h, a.w) * scale;
+    T y = gather_box<T, EXACT>(plane, s, i, j, a.h, a.w) * scale;
+    if (TAIL) {
+        const T ch_scale = tl.channel_scale != nullptr ? static_cast<T>(tl.channel_scale[k_par]) : T(1);
+        const T ch_shift = tl.channel_shift != nullptr ? static_cast<T>(tl.channel_shift[k_par]) : T(0);
+        const T res = tl.residual != nullptr ? static_cast<T>(widen(tl.residual[idx])) : T(0);
+        y = y * ch_scale + ch_shift + res;
+        if (tl.relu != 0 && y < T(0)) y = T(0);
+    }
+    narrow(y, tl.dst[idx]);
 }
 
 }  // namespace
 
-template <class T>
-hipError_t forward_launch(const T* integ, BoxParams<T> prm, T* out, Dims d, bool normalize,
-                          bool exact, hipStream_t stream) {
+// TAIL selects the kernels with the fused tail; without it only tail.dst is used.
+template <class T, class TO, bool TAIL>
+hipError_t forward_launch_any(const T* integ, BoxParams<T> prm, ForwardTail<TO> tail, Dims d,
+                              bool normalize, bool exact, hipStream_t stream) {
     const int64_t planes_f = d.planes * d.F;
     if (planes_f == 0 || d.hw() == 0) return hipSuccess;
     SampleArgs<T> a = base_args(prm, d);
-    a.src = integ; a.dst = out; a.normalize = normalize ? 1 : 0;
+    a.src = integ; a.normalize = normalize ? 1 : 0;
 
     if (!row_kernels_apply(d.h, d.w, sizeof(T))) {
         finish_args(a, planes_f * d.hw());
         const dim3 grid(static_cast<unsigned>((a.total + 255) / 256));
-        if (exact) BOXCONV_LAUNCH("forward_gather", (forward_gather_kernel<T, true>), grid, dim3(256), 0, stream, a);
-        else       BOXCONV_LAUNCH("forward_gather", (forward_gather_kernel<T, false>), grid, dim3(256), 0, stream, a);
+        if (exact) BOXCONV_LAUNCH("forward_gather", (forward_gather_kernel<T, TO, true, TAIL>), grid, dim3(256), 0, stream, a, tail);
+        else       BOXCONV_LAUNCH("forward_gather", (forward_gather_kernel<T, TO, false, TAIL>), grid, dim3(256), 0, stream, a, tail);
         return hipGetLastError();
     }
 
@@ -151,13 +207,37 @@ hipError_t forward_launch(const T* integ, BoxParams<T> prm, T* out, Dims d, bool
     const dim3 grid(static_cast<unsigned>(a.per_xcd * kXcds));
     const size_t lds = 4 * static_cast<size_t>(d.w + 3) * sizeof(T);
 #define LAUNCH_FWD(NT, KK, EX, FU) \
-    BOXCONV_LAUNCH("forward_rows", (forward_rows_kernel<T, NT, KK, EX, FU>), grid, dim3(NT), lds, stream, a)
+    BOXCONV_LAUNCH("forward_rows", (forward_rows_kernel<T, TO, NT, KK, EX, FU, TAIL>), grid, dim3(NT), lds, stream, a, tail)
     BOXCONV_DISPATCH_SHAPE_EXACT_FULL(LAUNCH_FWD, rc, exact)
 #undef LAUNCH_FWD
     return hipGetLastError();
 }
 
+template <class T>
+hipError_t forward_launch(const T* integ, BoxParams<T> prm, T* out, Dims d, bool normalize,
+                          bool exact, hipStream_t stream) {
+    return forward_launch_any<T, T, false>(integ, prm, ForwardTail<T>{out, nullptr, nullptr, nullptr, 0},
+                                           d, normalize, exact, stream);
+}
+
+template <class TO>
+hipError_t forward_fused_launch(const float* integ, BoxParams<float> prm, TO* out, const TO* residual,
+                                const float* channel_scale, const float* channel_shift, bool relu,
+                                Dims d, bool normalize, bool exact, hipStream_t stream) {
+    const ForwardTail<TO> tail{out, residual, channel_scale, channel_shift, relu ? 1 : 0};
+    if (residual == nullptr && channel_scale == nullptr && channel_shift == nullptr && !relu)
+        return forward_launch_any<float, TO, false>(integ, prm, tail, d, normalize, exact, stream);
+    return forward_launch_any<float, TO, true>(integ, prm, tail, d, normalize, exact, stream);
+}
+
 template hipError_t forward_launch<float>(const float*, BoxParams<float>, float*, Dims, bool, bool, hipStream_t);
 template hipError_t forward_launch<double>(const double*, BoxParams<double>, double*, Dims, bool, bool, hipStream_t);
+#define BOXCONV_INSTANTIATE_FUSED(TO)                                                              \
+    template hipError_t forward_fused_launch<TO>(const float*, BoxParams<float>, TO*, const TO*,   \
+                                                 const float*, const float*, bool, Dims, bool,     \
+                                                 bool, hipStream_t);
+BOXCONV_INSTANTIATE_FUSED(float)
+BOXCONV_INSTANTIATE_FUSED(f16_t)
+BOXCONV_INSTANTIATE_FUSED(bf16_t)
 
 }  // namespace boxconv

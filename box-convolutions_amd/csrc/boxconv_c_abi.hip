@@ -364,6 +364,39 @@ int boxconv_forward_f64(const double* input_integrated, const double* x_min, con
                                 in_planes, num_filters, h, w, normalize, exact, stream);
 }
 
+int boxconv_forward_fused_f32(const float* input_integrated, const float* x_min,
+                              const float* x_max, const float* y_min, const float* y_max,
+                              void* output, int output_dtype, const void* residual,
+                              const float* channel_scale, const float* channel_shift, int relu,
+                              int batch, int in_planes, int num_filters, int h, int w,
+                              int normalize, int exact, void* stream) {
+    if (int rc = check_dims(batch, in_planes, num_filters, h, w)) return rc;
+    if (output_dtype != BOXCONV_F32 && output_dtype != BOXCONV_F16 && output_dtype != BOXCONV_BF16)
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "fused forward: unknown output_dtype %d", output_dtype);
+    if (static_cast<int64_t>(batch) * in_planes * num_filters == 0) return 0;
+    if (!input_integrated || !x_min || !x_max || !y_min || !y_max || !output)
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "fused forward: null tensor pointer");
+    const boxconv::Dims d{in_planes, num_filters, h, w, static_cast<int64_t>(batch) * in_planes, 0};
+    const boxconv::BoxParams<float> prm{x_min, x_max, y_min, y_max};
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipError_t e;
+    if (output_dtype == BOXCONV_F32)
+        e = boxconv::forward_fused_launch<float>(
+            input_integrated, prm, static_cast<float*>(output), static_cast<const float*>(residual),
+            channel_scale, channel_shift, relu != 0, d, normalize != 0, exact != 0, s);
+    else if (output_dtype == BOXCONV_F16)
+        e = boxconv::forward_fused_launch<boxconv::f16_t>(
+            input_integrated, prm, static_cast<boxconv::f16_t*>(output),
+            static_cast<const boxconv::f16_t*>(residual), channel_scale, channel_shift, relu != 0, d,
+            normalize != 0, exact != 0, s);
+    else
+        e = boxconv::forward_fused_launch<boxconv::bf16_t>(
+            input_integrated, prm, static_cast<boxconv::bf16_t*>(output),
+            static_cast<const boxconv::bf16_t*>(residual), channel_scale, channel_shift, relu != 0, d,
+            normalize != 0, exact != 0, s);
+    return hip_result(e, "fused forward launch");
+}
+
 size_t boxconv_backward_workspace_bytes(int batch, int in_planes, int num_filters, int h, int w,
                                         int elem_size, int input_needs_grad,
                                         int params_need_grad) {

@@ -207,6 +207,43 @@ __device__ __forceinline__ void buffer_store(double v, const RowRef& r, int off)
     __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u, v), r.rs, off, r.soff, POLICY);
 }
 
+// 16-bit storage types for kernels that compute in float but read or write half precision
+// (IEEE binary16 and bfloat16). Conversions round to nearest even.
+struct f16_t { unsigned short bits; };
+struct bf16_t { unsigned short bits; };
+__device__ __forceinline__ float widen(float v) { return v; }
+__device__ __forceinline__ double widen(double v) { return v; }
+__device__ __forceinline__ float widen(f16_t v) {
+    return static_cast<float>(__builtin_bit_cast(_Float16, v.bits));
+}
+__device__ __forceinline__ float widen(bf16_t v) {
+    return __builtin_bit_cast(float, static_cast<unsigned>(v.bits) << 16);
+}
+__device__ __forceinline__ void narrow(float v, float& o) { o = v; }
+__device__ __forceinline__ void narrow(double v, double& o) { o = v; }
+__device__ __forceinline__ void narrow(float v, f16_t& o) {
+    o.bits = __builtin_bit_cast(unsigned short, static_cast<_Float16>(v));
+}
+__device__ __forceinline__ void narrow(float v, bf16_t& o) {
+    o.bits = __builtin_bit_cast(unsigned short, static_cast<__bf16>(v));
+}
+template <int POLICY>
+__device__ __forceinline__ f16_t buffer_load(const RowRef& r, int off, f16_t) {
+    return {static_cast<unsigned short>(__builtin_amdgcn_raw_buffer_load_b16(r.rs, off, r.soff, POLICY))};
+}
+template <int POLICY>
+__device__ __forceinline__ bf16_t buffer_load(const RowRef& r, int off, bf16_t) {
+    return {static_cast<unsigned short>(__builtin_amdgcn_raw_buffer_load_b16(r.rs, off, r.soff, POLICY))};
+}
+template <int POLICY>
+__device__ __forceinline__ void buffer_store(f16_t v, const RowRef& r, int off) {
+    __builtin_amdgcn_raw_buffer_store_b16(v.bits, r.rs, off, r.soff, POLICY);
+}
+template <int POLICY>
+__device__ __forceinline__ void buffer_store(bf16_t v, const RowRef& r, int off) {
+    __builtin_amdgcn_raw_buffer_store_b16(v.bits, r.rs, off, r.soff, POLICY);
+}
+
 // K consecutive elements per lane starting at byte offset `off` of a row of `limit` bytes. A
 // lane whose run lies inside the row stores it with one wide instruction (16, 12 or 8 bytes;
 // dword alignment suffices); the at most one lane per row whose run straddles the end goes

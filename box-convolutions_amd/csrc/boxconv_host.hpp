@@ -50,6 +50,16 @@ template <class T>
 hipError_t forward_launch(const T* integ, BoxParams<T> prm, T* out, Dims d, bool normalize,
                           bool exact, hipStream_t stream);
 
+// Forward with the output written as TO (float, f16_t or bf16_t; boxconv_device.hpp) and an
+// optional fused tail: y = S * channel_scale[c*F+f] + channel_shift[c*F+f] + residual, then
+// max(y, 0) if relu. Null pointers leave their piece out. Inference only.
+struct f16_t;
+struct bf16_t;
+template <class TO>
+hipError_t forward_fused_launch(const float* integ, BoxParams<float> prm, TO* out, const TO* residual,
+                                const float* channel_scale, const float* channel_shift, bool relu,
+                                Dims d, bool normalize, bool exact, hipStream_t stream);
+
 // band_rows: 0 when `gint` holds true integral images; otherwise `gint` holds band-local
 // integrals (each band of band_rows rows restarts at zero).
 template <class T>

@@ -82,6 +82,30 @@ int boxconv_forward_f64(const double* input_integrated, const double* x_min, con
                         int in_planes, int num_filters, int h, int w, int normalize, int exact,
                         void* stream);
 
+/* ---- forward, half-precision output and fused tail (inference) ------------------------------
+ * The same box sums as boxconv_forward_f32 (reference src/box_convolution_interface.cpp:13-139),
+ * computed in float from a float integral image, with what a network does to them next folded
+ * into the store: the tail of the reference's BottleneckBoxConv block in eval mode, BoxConv2d ->
+ * BatchNorm2d -> Dropout2d (identity) -> residual add -> ReLU
+ * (examples/Cityscapes/models/ENet.py:290-304):
+ *     y = S * channel_scale[c*F+f] + channel_shift[c*F+f] + residual[b][c*F+f][i][j]
+ *     output = relu ? max(y, 0) : y,  rounded to nearest even into the output type.
+ * output_dtype: BOXCONV_F32, BOXCONV_F16 (IEEE binary16) or BOXCONV_BF16; `output` and `residual`
+ * point at elements of that type, [batch, in_planes*num_filters, h, w]. channel_scale and
+ * channel_shift are float [in_planes*num_filters] (an eval-mode BatchNorm folds to
+ * scale = gamma / sqrt(var + eps), shift = beta - mean * scale). residual, channel_scale and
+ * channel_shift may each be NULL (no residual, scale 1, shift 0). There is no backward for
+ * this entry point. */
+#define BOXCONV_F32 0
+#define BOXCONV_F16 1
+#define BOXCONV_BF16 2
+int boxconv_forward_fused_f32(const float* input_integrated, const float* x_min,
+                              const float* x_max, const float* y_min, const float* y_max,
+                              void* output, int output_dtype, const void* residual,
+                              const float* channel_scale, const float* channel_shift, int relu,
+                              int batch, int in_planes, int num_filters, int h, int w,
+                              int normalize, int exact, void* stream);
+
 /* ---- backward ---------------------------------------------------------------------------------
  * Replaces `box_convolution_backward(input_integrated, x_min, x_max, y_min, y_max, grad_output,
  * output, reparametrization_h, reparametrization_w, normalize, exact, input_needs_grad,

@@ -50,6 +50,12 @@ def test_argument_errors_are_reported_without_launching(lib):
     assert rc == -1
     rc = lib.boxconv_forward_f64(null, null, null, null, null, null, 1, 1, 1, 0, 4, 1, 1, null)
     assert rc == -1
+    rc = lib.boxconv_forward_fused_f32(null, null, null, null, null, null, 7, null, null, null, 0,
+                                       1, 1, 1, 4, 4, 1, 1, null)
+    assert rc == -1 and b"output_dtype" in lib.boxconv_last_error()
+    rc = lib.boxconv_forward_fused_f32(null, null, null, null, null, null, 1, null, null, null, 0,
+                                       1, 1, 1, 4, 4, 1, 1, null)
+    assert rc == -1 and b"null" in lib.boxconv_last_error()
     # more than 2^31-1 elements
     rc = lib.boxconv_forward_f32(null, null, null, null, null, null, 64, 64, 64, 4096, 4096, 1, 1, null)
     assert rc == -3

@@ -1,0 +1,167 @@
+"""Forward with half-precision output and the fused tail (scale, shift, residual, ReLU).
+
+The reference has no such function: the expected values are the plain forward (itself checked
+against the CPU oracle in test_gpu_parity.py) followed by the same element-wise steps in torch,
+which is what the reference's BottleneckBoxConv does in eval mode
+(examples/Cityscapes/models/ENet.py:290-304). Tolerances: float32 results within a few float32
+roundings of the composition (the kernel contracts scale and shift into one fused multiply-add);
+half-precision results without a tail are the float32 forward rounded to the half type (bar ties
+of that rounding), with a tail they are within one unit in the last place of the half type.
+"""
+import numpy as np
+import pytest
+import torch
+
+from box_convolution import BoxConv2d
+from helpers import make_boxes
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+# B, C, F, h, w: partial rows, full rows at 256 and 512 threads, three columns per lane, gather
+SHAPES = [(2, 3, 4, 37, 53), (1, 2, 2, 64, 256), (1, 1, 2, 40, 1024), (1, 2, 1, 18, 1536),
+          (1, 1, 1, 8, 2100), (3, 1, 5, 9, 64)]
+HALF_ULP = {torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}
+
+
+def setup_case(hip, shape, seed, kind="inside"):
+    B, C, F, h, w = shape
+    rng = np.random.default_rng(seed)
+    boxes = [torch.from_numpy(b).to(DEV) for b in make_boxes(rng, C, F, h, w, kind)]
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    x = torch.randn(B, C, h, w, generator=g).to(DEV)
+    integ = hip.integral_image(x)
+    scale = (torch.rand(C * F, generator=g) * 2 - 0.7).to(DEV)
+    shift = torch.randn(C * F, generator=g).to(DEV)
+    residual = torch.randn(B, C * F, h, w, generator=g).to(DEV)
+    return integ, boxes, scale, shift, residual
+
+
+def compose(plain, scale, shift, residual, relu):
+    y = plain
+    if scale is not None:
+        y = y * scale[None, :, None, None]
+    if shift is not None:
+        y = y + shift[None, :, None, None]
+    if residual is not None:
+        y = y + residual
+    return torch.relu(y) if relu else y
+
+
+@pytest.mark.parametrize("exact", [True, False])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_fused_tail_float32(hip, shape, exact):
+    integ, boxes, scale, shift, residual = setup_case(hip, shape, 11)
+    plain = hip.box_convolution_forward(integ, *boxes, True, exact)
+    # nothing to fuse: the very same numbers as the plain entry point
+    assert torch.equal(hip.box_convolution_forward_fused(integ, *boxes, True, exact), plain)
+    for use_scale, use_shift, use_res, relu in [(1, 1, 1, 1), (1, 0, 0, 0), (0, 1, 0, 0), (0, 0, 1, 0),
+                                                (0, 0, 0, 1), (1, 1, 0, 1), (0, 0, 1, 1)]:
+        args = (scale if use_scale else None, shift if use_shift else None,
+                residual if use_res else None, bool(relu))
+        got = hip.box_convolution_forward_fused(integ, *boxes, True, exact, torch.float32, *args)
+        want = compose(plain, *args)
+        # sizes of the terms that get rounded
+        mag = (plain.abs() * (scale.abs().max() if use_scale else 1)).max().item() + 4.0
+        assert (got - want).abs().max().item() <= 4e-7 * mag, (use_scale, use_shift, use_res, relu)
+        if relu:
+            assert got.min().item() >= 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_half_precision_output(hip, shape, dtype):
+    integ, boxes, scale, shift, residual = setup_case(hip, shape, 23, kind="hanging")
+    for normalize in (True, False):
+        plain = hip.box_convolution_forward(integ, *boxes, normalize, True)
+        got = hip.box_convolution_forward_fused(integ, *boxes, normalize, True, dtype)
+        assert got.dtype == dtype and got.shape == plain.shape
+        # (float16 overflows to inf where the unnormalized sums exceed 65504, as .to() does)
+        want = plain.to(dtype)
+        # The kernel may round the product sum * (1/area) to the half type in one step
+        # (mixed-precision multiply); where the float32 product is a tie between two half
+        # values that differs from rounding twice, and is then the closer one.
+        assert (got != want).float().mean().item() < 1e-3
+        finite = want.float().isfinite()
+        assert torch.equal(got.float().isfinite(), finite)
+        assert torch.all(((got.float() - plain).abs() <= (want.float() - plain).abs() * (1 + 1e-6))[finite])
+    plain = hip.box_convolution_forward(integ, *boxes, True, True)
+    res16 = residual.to(dtype)
+    got = hip.box_convolution_forward_fused(integ, *boxes, True, True, dtype, scale, shift, res16, True)
+    want = compose(plain, scale, shift, res16.float(), True)
+    err = (got.float() - want).abs()
+    bound = HALF_ULP[dtype] * want.abs().clamp_min(2.0 ** -14) + 1e-6
+    assert torch.all(err <= bound)
+    # and nearly all entries are the correctly rounded value of the float32 composition
+    assert (got != want.to(dtype)).float().mean().item() < 0.02
+
+
+def test_argument_checks(hip):
+    integ, boxes, scale, shift, residual = setup_case(hip, (1, 2, 2, 8, 8), 3)
+    with pytest.raises(RuntimeError, match="float32 integral image"):
+        hip.box_convolution_forward_fused(integ.double(), *boxes, True, True)
+    with pytest.raises(RuntimeError, match="float32, float16 or bfloat16"):
+        hip.box_convolution_forward_fused(integ, *boxes, True, True, torch.float64)
+    with pytest.raises(RuntimeError, match="must hold 4 values"):
+        hip.box_convolution_forward_fused(integ, *boxes, True, True, torch.float32, scale[:3])
+    with pytest.raises(RuntimeError, match="shape of the output"):
+        hip.box_convolution_forward_fused(integ, *boxes, True, True, torch.float32, None, None,
+                                          residual[:, :3])
+
+
+def make_module(C, F, h, w, seed):
+    import random
+    random.seed(seed)
+    return BoxConv2d(C, F, h, w).to(DEV)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_module_takes_half_precision_input(dtype):
+    m = make_module(3, 4, 40, 72, 5).eval()
+    x = torch.randn(2, 3, 40, 72, device=DEV).to(dtype)
+    with torch.no_grad():
+        got = m(x)
+        want = m(x.float())
+    assert got.dtype == dtype and (got != want.to(dtype)).float().mean().item() < 1e-3
+    assert torch.allclose(got.float(), want, rtol=HALF_ULP[dtype], atol=1e-7)
+    # with autograd: float32 in between, gradients come back in the input's type
+    m.train()
+    xg = x.clone().requires_grad_(True)
+    out = m(xg)
+    assert out.dtype == dtype and out.requires_grad
+    go = torch.randn_like(out)
+    out.backward(go)
+    x32 = x.float().requires_grad_(True)
+    ref_grads = torch.autograd.grad(m(x32), [x32, m.x_min, m.y_max], go.float())
+    assert xg.grad.dtype == dtype
+    assert torch.allclose(xg.grad.float(), ref_grads[0], rtol=2 * HALF_ULP[dtype], atol=1e-3)
+    assert torch.allclose(m.x_min.grad, ref_grads[1], rtol=1e-4, atol=1e-4 * ref_grads[1].abs().max().item())
+    assert torch.allclose(m.y_max.grad, ref_grads[2], rtol=1e-4, atol=1e-4 * ref_grads[2].abs().max().item())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_bottleneck_tail_in_one_launch(dtype):
+    """BoxConv2d -> BatchNorm2d -> Dropout2d -> + x -> ReLU in eval mode, as the reference's
+    BottleneckBoxConv ends (ENet.py:290-304), against the same chain of torch modules."""
+    C, F, h, w = 4, 4, 32, 64
+    m = make_module(C, F, h, w, 9).eval()
+    bn = torch.nn.BatchNorm2d(C * F).to(DEV)
+    with torch.no_grad():
+        bn.running_mean.normal_()
+        bn.running_var.uniform_(0.5, 2.0)
+        bn.weight.normal_()
+        bn.bias.normal_()
+    bn.eval()
+    drop = torch.nn.Dropout2d(0.25).eval()
+    x = torch.randn(2, C, h, w, device=DEV)
+    skip = torch.randn(2, C * F, h, w, device=DEV).to(dtype)
+    with torch.no_grad():
+        want = torch.relu(skip.float() + drop(bn(m(x))))
+        scale, shift = BoxConv2d.fold_batch_norm(bn)
+        got = m.forward_fused(x.to(dtype), scale, shift, skip, relu=True)
+        want_in = torch.relu(skip.float() + drop(bn(m(x.to(dtype).float()))))
+    assert got.dtype == dtype
+    if dtype == torch.float32:
+        assert torch.allclose(got, want, rtol=1e-5, atol=1e-5)
+    else:
+        assert torch.all((got.float() - want_in).abs() <= HALF_ULP[dtype] * want_in.abs() + 1e-5)

@@ -106,6 +106,10 @@ def main():
     ap.add_argument("--workload", type=int, default=3, choices=[1, 2, 3, 4, 5])
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--phases", action="store_true", help="also print per-kernel times to stderr")
+    ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
+                    help="after the timed steps, run torch.neg on a float tensor of this many MiB "
+                         "(reads MIB, writes MIB): the plain streaming kernel of known size that "
+                         "the FETCH_SIZE / WRITE_SIZE counters are calibrated against")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus %d is not supported (box convolution "
@@ -168,6 +172,13 @@ def main():
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     dom_ms, dom_launches = _native.profile_collect()
+
+    if args.copy_probe > 0:
+        src = torch.ones(args.copy_probe * (1 << 20) // 4, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.neg(src, out=dst)
+        torch.cuda.synchronize()
 
     ms_per_step = 1e3 * elapsed / args.steps
     value = ab["alg"] / (elapsed / args.steps) / 1e9

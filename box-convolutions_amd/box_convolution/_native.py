@@ -94,7 +94,31 @@ def _require_device(t, what):
 
 
 def _stream(device):
-    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    """The current stream of `device` as a raw hipStream_t."""
+    index = device.index
+    if index is None:
+        index = torch.cuda.current_device()
+    return ctypes.c_void_p(torch._C._cuda_getCurrentRawStream(index))
+
+
+class _on_device:
+    """``with _on_device(dev):`` makes `dev` the current device for the native call; it does
+    nothing when it already is (the usual case, and ``torch.cuda.device`` costs microseconds)."""
+    __slots__ = ("guard",)
+
+    def __init__(self, device):
+        index = device.index
+        self.guard = (torch.cuda.device(index)
+                      if index is not None and index != torch.cuda.current_device() else None)
+
+    def __enter__(self):
+        if self.guard is not None:
+            self.guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self.guard is not None:
+            return self.guard.__exit__(*exc)
+        return False
 
 
 def _ptr(t):
@@ -121,7 +145,7 @@ def integral_image(input):
     if h == 0 or w == 0:
         return output.zero_()
     planes = input.numel() // (h * w)
-    with torch.cuda.device(input.device):
+    with _on_device(input.device):
         nbytes = lib.boxconv_integral_image_workspace_bytes(planes, h, w)
         ws = _workspace(nbytes, input.device)
         rc = getattr(lib, "boxconv_integral_image_" + sfx)(
@@ -175,7 +199,7 @@ def box_convolution_forward(input_integrated, x_min, x_max, y_min, y_max, normal
                          device=input_integrated.device)
     if output.numel() == 0:
         return output
-    with torch.cuda.device(input_integrated.device):
+    with _on_device(input_integrated.device):
         rc = getattr(lib, "boxconv_forward_" + sfx)(
             _ptr(input_integrated), _ptr(x_min), _ptr(x_max), _ptr(y_min), _ptr(y_max),
             _ptr(output), B, C, F, h, w, int(bool(normalize)), int(bool(exact)),
@@ -230,7 +254,7 @@ def box_convolution_forward_fused(input_integrated, x_min, x_max, y_min, y_max, 
     output = torch.empty((B, C * F, h, w), dtype=output_dtype, device=dev)
     if output.numel() == 0:
         return output
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = lib.boxconv_forward_fused_f32(
             _ptr(input_integrated), _ptr(x_min), _ptr(x_max), _ptr(y_min), _ptr(y_max),
             _ptr(output), _FUSED_OUTPUT[output_dtype], _ptr(residual), _ptr(per_channel[0]),
@@ -276,7 +300,7 @@ def box_convolution_backward(input_integrated, x_min, x_max, y_min, y_max, grad_
     want_input = input_needs_grad and grad_input.numel() > 0 and F > 0
     want_params = any(needs_p) and C * F > 0
     if want_input or want_params:
-        with torch.cuda.device(dev):
+        with _on_device(dev):
             nbytes = lib.boxconv_backward_workspace_bytes(
                 B, C, F, h, w, grad_output.element_size(), int(want_input), int(want_params))
             ws = _workspace(nbytes, dev)
@@ -321,7 +345,7 @@ def clip_parameters(x_min, x_max, y_min, y_max, reparametrization_h, reparametri
             for p, s in zip(params, staged):
                 p.detach().copy_(s)
         return
-    with torch.cuda.device(x_min.device):
+    with _on_device(x_min.device):
         rc = getattr(lib, "boxconv_clip_parameters_" + sfx)(
             _ptr(x_min), _ptr(x_max), _ptr(y_min), _ptr(y_max), n,
             float(reparametrization_h), float(reparametrization_w), float(max_input_h),
@@ -345,7 +369,7 @@ def clip_reparametrize(x_min, x_max, y_min, y_max, reparametrization_h, reparame
     real = torch.empty((4,) + tuple(x_min.shape), dtype=x_min.dtype, device=x_min.device)
     if n > 0:
         lib = load()
-        with torch.cuda.device(x_min.device):
+        with _on_device(x_min.device):
             rc = getattr(lib, "boxconv_clip_reparametrize_" + sfx)(
                 _ptr(x_min), _ptr(x_max), _ptr(y_min), _ptr(y_max), _ptr(real), n,
                 float(reparametrization_h), float(reparametrization_w), float(max_input_h),

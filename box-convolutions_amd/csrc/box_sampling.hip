@@ -337,6 +337,11 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
     const LoadRows<T> irows(a.src + p * static_cast<int64_t>(h + 1) * pitch, pitch, w + 1, h + 1);
     const LoadRows<T> grows(a.grad_out + pf * static_cast<int64_t>(h) * w - 1, w, w + 1, h);
     T* lrows = SCAN ? a.dst + pf * static_cast<int64_t>(h + 1) * pitch : nullptr;
+    // The bands an XCD writes last (the final keep_tail bytes of its range) are stored with the
+    // ordinary cache policy, everything before them non-temporally: see the store below.
+    const unsigned from_end = static_cast<unsigned>(a.per_xcd) - 1u - vid % static_cast<unsigned>(a.per_xcd);
+    const bool keep_in_cache =
+        static_cast<uint64_t>(from_end) * a.R * pitch * sizeof(T) < static_cast<uint64_t>(a.keep_tail);
     const Rows<T, FULL> lout(lrows, pitch, w + 1, h + 1);
     const StreamLds<T> lds = carve_stream_lds<T>(K, nt);
     const int glen = lds.glen;
@@ -524,9 +529,11 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
                 // and wave n takes n + 1 of them
                 add_waves_left<T, 0>(lds.wave_tot, wave, carry0, carry1);
                 // the lane's K consecutive columns K*tid+1 .. K*tid+K of integral rows i+1, i+2:
-                // a wave stores one contiguous run of 64*K elements per row. Ordinary cache
-                // policy: the grad-input kernel starts with the planes written last and finds
-                // part of them still in the memory-side cache.
+                // a wave stores one contiguous run of 64*K elements per row. The grad-input
+                // kernel starts with the planes written last and finds them still in the
+                // memory-side cache if they were stored with the ordinary policy; the rest is
+                // stored non-temporally so that it does not push the integral plane of the
+                // input, which all filters of a plane re-read, out of the L2.
                 T* o0 = lrows + static_cast<int64_t>(i + 1) * pitch;
                 const bool second = i + 1 < i1;
                 const RowRef ob0 = lout.row(i + 1);
@@ -535,8 +542,13 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
 #pragma unroll
                 for (int k = 0; k < K; ++k) { out0[k] = carry0 + loc0[k]; out1[k] = carry1 + loc1[k]; }
                 const int first = (1 + K * tid) * static_cast<int>(sizeof(T));
-                buffer_store_run<kCacheDefault, FULL>(out0, ob0, first, static_cast<int>(row_bytes + sizeof(T)));
-                buffer_store_run<kCacheDefault, FULL>(out1, ob1, first, static_cast<int>(row_bytes + sizeof(T)));
+                if (keep_in_cache) {
+                    buffer_store_run<kCacheDefault, FULL>(out0, ob0, first, static_cast<int>(row_bytes + sizeof(T)));
+                    buffer_store_run<kCacheDefault, FULL>(out1, ob1, first, static_cast<int>(row_bytes + sizeof(T)));
+                } else {
+                    buffer_store_run<kCacheStream, FULL>(out0, ob0, first, static_cast<int>(row_bytes + sizeof(T)));
+                    buffer_store_run<kCacheStream, FULL>(out1, ob1, first, static_cast<int>(row_bytes + sizeof(T)));
+                }
                 if (tid == 0) {
                     o0[0] = T(0);
                     if (second) o0[pitch] = T(0);
@@ -750,6 +762,16 @@ StreamPlan plan_grad_output_stream(int64_t planes_f, int h, int w, size_t elem_s
     return sp;
 }
 
+// How much of the band-local integral, counted from its end, is written with the ordinary cache
+// policy (the memory-side cache holds 256 MB; the grad-input kernel reads that part first).
+inline int64_t cached_tail_bytes() {
+    static const int64_t v = [] {
+        const char* e = std::getenv("BOXCONV_L_KEEP_MB");
+        return static_cast<int64_t>(e != nullptr ? std::max(0, std::atoi(e)) : 192) << 20;
+    }();
+    return v;
+}
+
 template <class T>
 hipError_t grad_output_stream_launch(const T* integ, const T* grad_out, BoxParams<T> prm,
                                      double* acc, int acc_slots, T* local_integral,
@@ -762,6 +784,7 @@ hipError_t grad_output_stream_launch(const T* integ, const T* grad_out, BoxParam
     a.src = integ; a.grad_out = grad_out; a.acc = acc; a.acc_slots = acc_slots; a.dst = local_integral;
     if (acc_slots != 0 && acc_slots != sp.nb) return hipErrorInvalidValue;
     a.nb = sp.nb; a.R = sp.R;
+    a.keep_tail = scan ? cached_tail_bytes() / kXcds : 0;
     finish_args(a, planes_f * a.nb);
     const RowConfig rc = stream_row_config(d.w);
     const dim3 grid(static_cast<unsigned>(a.per_xcd * kXcds));

@@ -39,6 +39,8 @@ struct SampleArgs {
     int64_t per_xcd;      // ceil(total / 8)
     int normalize;
     int reverse;          // grad input only: walk the work items last to first
+    int64_t keep_tail;    // grad_output pass only: bytes at the end of each XCD's share of the
+                          // band-local integral that are stored with the ordinary cache policy
 };
 
 // Two rows of the same column, adjacent in LDS: every LDS access of the row kernels moves the

@@ -45,6 +45,67 @@ bool force_gather_kernels() {
 
 namespace {
 
+// Turns the five sums per box into the four gradients (reference:
+// src/box_convolution_interface.cpp:345-391): optional 1/area, the d(1/area) term
+// sum(g*out) * (+-1)/(extent along the parameter's axis), and the reparametrization scale.
+// One wave per box. slots == 0: acc holds the five sums per box. Otherwise acc holds one slot of
+// five partial sums per (batch item b, box, band): [(b*n + box)*slots + band][5]; the wave adds
+// them in a fixed order.
+template <class T>
+struct FinalizeArgs {
+    const double* acc;     // null: nothing to do
+    int batch, slots;
+    T* g[4];               // gradients w.r.t. x_min, x_max, y_min, y_max; null = not wanted
+    int n;                 // boxes
+    float reparam_h, reparam_w;
+    int normalize, exact;
+};
+
+template <class T>
+__device__ __forceinline__ void finalize_box(const FinalizeArgs<T>& fa, const BoxParams<T>& prm,
+                                             int k, int lane) {
+    double sum[5] = {0.0, 0.0, 0.0, 0.0, 0.0};
+    if (fa.slots > 0) {
+        const int per_box = fa.batch * fa.slots;
+        for (int e = lane; e < per_box; e += 64) {
+            const int b = e / fa.slots, band = e % fa.slots;
+            const double* part = fa.acc + ((static_cast<int64_t>(b) * fa.n + k) * fa.slots + band) * 5;
+#pragma unroll
+            for (int m = 0; m < 5; ++m) sum[m] += part[m];
+        }
+#pragma unroll
+        for (int m = 0; m < 5; ++m) sum[m] = wave_sum_to_last(sum[m]);
+    } else {
+#pragma unroll
+        for (int m = 0; m < 5; ++m) sum[m] = fa.acc[k * 5 + m];
+    }
+    if (lane != 63) return;
+    const T xmin = prm.xmin[k], xmax = prm.xmax[k], ymin = prm.ymin[k], ymax = prm.ymax[k];
+    const bool ex = fa.exact != 0;
+    const T inv_area = fa.normalize ? inverse_extent(xmin, xmax, ymin, ymax, ex, true, true) : T(1);
+    const T s = fa.normalize ? static_cast<T>(sum[4]) * inv_area : T(0);   // sum(g * output)
+#pragma unroll
+    for (int which = 0; which < 4; ++which) {
+        if (fa.g[which] == nullptr) continue;
+        T g = static_cast<T>(sum[which]);
+        if (fa.normalize) {
+            g *= inv_area;
+            const bool is_x = which < 2;
+            const T inv_ext = inverse_extent(xmin, xmax, ymin, ymax, ex, is_x, !is_x);
+            const T sign = (which == 1 || which == 3) ? T(-1) : T(1);
+            g = g + sign * s * inv_ext;
+        }
+        g *= static_cast<T>(static_cast<double>(which < 2 ? fa.reparam_h : fa.reparam_w));
+        fa.g[which][k] = g;
+    }
+}
+
+template <class T>
+__global__ void __launch_bounds__(64)
+param_grad_finalize_kernel(FinalizeArgs<T> fa, BoxParams<T> prm) {
+    finalize_box(fa, prm, static_cast<int>(blockIdx.x), static_cast<int>(threadIdx.x));
+}
+
 // ---------------------------------------------------------------------------------------------
 // Gradient w.r.t. the input. Work item = (plane p = (b,c), band of RB rows); the F mirrored boxes
 // are visited in order and summed in registers, so no [B,C,F,h,w] temporary exists.
@@ -54,8 +115,12 @@ namespace {
 // the first row this workgroup touches for the filter): the bulk of the integral cancels before
 // it is ever added.
 template <class T, int NT, int K, int RB, bool EXACT, bool FULL, bool OFFS>
-__global__ void __launch_bounds__(NT) grad_input_rows_kernel(SampleArgs<T> a) {
+__global__ void __launch_bounds__(NT) grad_input_rows_kernel(SampleArgs<T> a, FinalizeArgs<T> fin) {
     static_assert(RB % 4 == 0, "rows are handled in pairs, and pairs alternate between two LDS buffers");
+    // Rides along: the first fin.n workgroups each finish the parameter gradients of one box from
+    // the sums the preceding launch left (one wave's work; saves a launch of its own).
+    if (fin.acc != nullptr && blockIdx.x < static_cast<unsigned>(fin.n) && threadIdx.x < 64)
+        finalize_box(fin, a.prm, static_cast<int>(blockIdx.x), static_cast<int>(threadIdx.x));
     unsigned vid = xcd_contiguous_id(a.per_xcd);
     if (vid >= a.total) return;
     if (a.reverse) vid = static_cast<unsigned>(a.total) - 1u - vid;
@@ -655,62 +720,25 @@ __global__ void fill_zero_kernel(double* __restrict__ p, int n) {
     if (i < n) p[i] = 0.0;
 }
 
-// Turns the five sums per box into the four gradients (reference:
-// src/box_convolution_interface.cpp:345-391): optional 1/area, the d(1/area) term
-// sum(g*out) * (+-1)/(extent along the parameter's axis), and the reparametrization scale.
-// One wave per box. slots == 0: acc holds the five sums per box. Otherwise acc holds one slot of
-// five partial sums per (batch item b, box, band): [(b*n + box)*slots + band][5]; the wave adds
-// them in a fixed order.
-template <class T>
-__global__ void __launch_bounds__(64)
-param_grad_finalize_kernel(const double* __restrict__ acc, int batch, int slots, BoxParams<T> prm,
-                           T* g0, T* g1, T* g2, T* g3, int n, float reparam_h, float reparam_w,
-                           int normalize, int exact) {
-    const int k = blockIdx.x;
-    const int lane = threadIdx.x;
-    double sum[5] = {0.0, 0.0, 0.0, 0.0, 0.0};
-    if (slots > 0) {
-        const int per_box = batch * slots;
-        for (int e = lane; e < per_box; e += 64) {
-            const int b = e / slots, band = e % slots;
-            const double* part = acc + ((static_cast<int64_t>(b) * n + k) * slots + band) * 5;
-#pragma unroll
-            for (int m = 0; m < 5; ++m) sum[m] += part[m];
-        }
-#pragma unroll
-        for (int m = 0; m < 5; ++m) sum[m] = wave_sum_to_last(sum[m]);
-    } else {
-#pragma unroll
-        for (int m = 0; m < 5; ++m) sum[m] = acc[k * 5 + m];
-    }
-    if (lane != 63) return;
-    const T xmin = prm.xmin[k], xmax = prm.xmax[k], ymin = prm.ymin[k], ymax = prm.ymax[k];
-    const bool ex = exact != 0;
-    const T inv_area = normalize ? inverse_extent(xmin, xmax, ymin, ymax, ex, true, true) : T(1);
-    const T s = normalize ? static_cast<T>(sum[4]) * inv_area : T(0);   // sum(g * output)
-    T* outp[4] = {g0, g1, g2, g3};
-#pragma unroll
-    for (int which = 0; which < 4; ++which) {
-        if (outp[which] == nullptr) continue;
-        T g = static_cast<T>(sum[which]);
-        if (normalize) {
-            g *= inv_area;
-            const bool is_x = which < 2;
-            const T inv_ext = inverse_extent(xmin, xmax, ymin, ymax, ex, is_x, !is_x);
-            const T sign = (which == 1 || which == 3) ? T(-1) : T(1);
-            g = g + sign * s * inv_ext;
-        }
-        g *= static_cast<T>(static_cast<double>(which < 2 ? reparam_h : reparam_w));
-        outp[which][k] = g;
-    }
-}
 
 }  // namespace
 
 
 template <class T>
+FinalizeArgs<T> finalize_args(const ParamFinish<T>& f) {
+    FinalizeArgs<T> fa{};
+    fa.acc = f.acc; fa.batch = f.batch; fa.slots = f.acc_slots;
+    for (int i = 0; i < 4; ++i) fa.g[i] = f.grad[i];
+    fa.n = f.n_boxes; fa.reparam_h = f.reparam_h; fa.reparam_w = f.reparam_w;
+    fa.normalize = f.normalize ? 1 : 0; fa.exact = f.exact ? 1 : 0;
+    return fa;
+}
+
+template <class T>
 hipError_t grad_input_launch(const T* gint, int band_rows, BoxParams<T> prm, T* grad_in, Dims d,
-                             bool normalize, bool exact, hipStream_t stream) {
+                             bool normalize, bool exact, hipStream_t stream,
+                             const ParamFinish<T>* finish, bool* finish_done) {
+    if (finish_done != nullptr) *finish_done = false;
     if (d.planes == 0 || d.hw() == 0) return hipSuccess;
     SampleArgs<T> a = base_args(prm, d);
     a.src = gint; a.dst = grad_in; a.normalize = normalize ? 1 : 0;
@@ -734,9 +762,14 @@ hipError_t grad_input_launch(const T* gint, int band_rows, BoxParams<T> prm, T* 
     finish_args(a, d.planes * a.nb);
     const dim3 grid(static_cast<unsigned>(a.per_xcd * kXcds));
     const size_t lds = 4 * static_cast<size_t>(d.w + 3) * sizeof(T);
+    FinalizeArgs<T> fin{};
+    if (finish != nullptr && finish->acc != nullptr && grid.x >= static_cast<unsigned>(finish->n_boxes)) {
+        fin = finalize_args(*finish);
+        if (finish_done != nullptr) *finish_done = true;
+    }
 #define LAUNCH_GI(NT, KK, EX, FU) \
-    if (band_rows > 0) BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, NT, KK, RB, EX, FU, true>), grid, dim3(NT), lds, stream, a); \
-    else BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, NT, KK, RB, EX, FU, false>), grid, dim3(NT), lds, stream, a)
+    if (band_rows > 0) BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, NT, KK, RB, EX, FU, true>), grid, dim3(NT), lds, stream, a, fin); \
+    else BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, NT, KK, RB, EX, FU, false>), grid, dim3(NT), lds, stream, a, fin)
     BOXCONV_DISPATCH_SHAPE_EXACT_FULL(LAUNCH_GI, rc, exact)
 #undef LAUNCH_GI
     return hipGetLastError();
@@ -815,26 +848,22 @@ hipError_t grad_params_gather_launch(const T* integ, const T* grad_out, BoxParam
 }
 
 template <class T>
-hipError_t grad_params_finish(const double* acc, int batch, int acc_slots, BoxParams<T> prm,
-                              T* gxmin, T* gxmax, T* gymin, T* gymax, int n_boxes, float reparam_h,
-                              float reparam_w, bool normalize, bool exact, hipStream_t stream) {
-    if (n_boxes == 0) return hipSuccess;
-    BOXCONV_LAUNCH("param_grad_finalize", (param_grad_finalize_kernel<T>), dim3(n_boxes), dim3(64), 0,
-                   stream, acc, batch, acc_slots, prm, gxmin, gxmax, gymin, gymax, n_boxes, reparam_h,
-                   reparam_w, normalize ? 1 : 0, exact ? 1 : 0);
+hipError_t grad_params_finish(const ParamFinish<T>& f, BoxParams<T> prm, hipStream_t stream) {
+    if (f.n_boxes == 0) return hipSuccess;
+    BOXCONV_LAUNCH("param_grad_finalize", (param_grad_finalize_kernel<T>), dim3(f.n_boxes), dim3(64), 0,
+                   stream, finalize_args(f), prm);
     return hipGetLastError();
 }
 
 #define BOXCONV_INSTANTIATE(T)                                                                     \
     template hipError_t grad_input_launch<T>(const T*, int, BoxParams<T>, T*, Dims, bool, bool,    \
-                                             hipStream_t);                                         \
+                                             hipStream_t, const ParamFinish<T>*, bool*);           \
     template hipError_t grad_output_stream_launch<T>(const T*, const T*, BoxParams<T>, double*, int, \
                                                      T*, const StreamPlan&, Dims, bool,            \
                                                      hipStream_t);                                 \
     template hipError_t grad_params_gather_launch<T>(const T*, const T*, BoxParams<T>, double*,    \
                                                      Dims, bool, hipStream_t);                     \
-    template hipError_t grad_params_finish<T>(const double*, int, int, BoxParams<T>, T*, T*, T*,   \
-                                              T*, int, float, float, bool, bool, hipStream_t);
+    template hipError_t grad_params_finish<T>(const ParamFinish<T>&, BoxParams<T>, hipStream_t);
 
 BOXCONV_INSTANTIATE(float)
 BOXCONV_INSTANTIATE(double)

@@ -229,6 +229,9 @@ int backward_impl(const T* integ, const T* x_min, const T* x_max, const T* y_min
         if (int rc = hip_result(boxconv::grad_params_begin(acc, n_boxes, s), "accumulator clear"))
             return rc;
 
+    const boxconv::ParamFinish<T> finish{acc, batch, L.acc_slots, {gx_min, gx_max, gy_min, gy_max},
+                                         n_boxes, reparam_h, reparam_w, normalize != 0, exact != 0};
+    bool finished = false;
     const int64_t planes = static_cast<int64_t>(batch) * in_planes;
     const int64_t hw = static_cast<int64_t>(h) * w;
     const int64_t ipl = static_cast<int64_t>(h + 1) * (w + 1);
@@ -246,9 +249,13 @@ int backward_impl(const T* integ, const T* x_min, const T* x_max, const T* y_min
                     integ_chunk, go_chunk, prm, acc, L.acc_slots, gint, sp, d, exact != 0, s),
                     "grad_output streaming launch"))
                 return rc;
+            // (the sums of all chunks are complete once the last chunk's pass over grad_output
+            // is: its grad-input launch finishes the parameter gradients on the side)
+            const bool last = p0 + np == planes;
             if (need_input)
                 if (int rc = hip_result(boxconv::grad_input_launch<T>(
-                        gint, sp.R, prm, gin_chunk, d, normalize != 0, exact != 0, s),
+                        gint, sp.R, prm, gin_chunk, d, normalize != 0, exact != 0, s,
+                        need_params && last ? &finish : nullptr, &finished),
                         "input-gradient launch"))
                     return rc;
         } else {
@@ -272,10 +279,9 @@ int backward_impl(const T* integ, const T* x_min, const T* x_max, const T* y_min
             }
         }
     }
-    if (need_params)
-        if (int rc = hip_result(boxconv::grad_params_finish<T>(
-                acc, batch, L.acc_slots, prm, gx_min, gx_max, gy_min, gy_max, n_boxes, reparam_h, reparam_w,
-                normalize != 0, exact != 0, s), "parameter-gradient finish"))
+    if (need_params && !finished)
+        if (int rc = hip_result(boxconv::grad_params_finish<T>(finish, prm, s),
+                                "parameter-gradient finish"))
             return rc;
     return 0;
 }

@@ -60,11 +60,26 @@ hipError_t forward_fused_launch(const float* integ, BoxParams<float> prm, TO* ou
                                 const float* channel_scale, const float* channel_shift, bool relu,
                                 Dims d, bool normalize, bool exact, hipStream_t stream);
 
+// The last step of the parameter gradients: from the five sums per box (or per box, batch item
+// and band, see grad_output_stream_launch) to the four gradients.
+template <class T>
+struct ParamFinish {
+    const double* acc;
+    int batch, acc_slots;
+    T* grad[4];            // w.r.t. x_min, x_max, y_min, y_max; null = not wanted
+    int n_boxes;
+    float reparam_h, reparam_w;
+    bool normalize, exact;
+};
+
 // band_rows: 0 when `gint` holds true integral images; otherwise `gint` holds band-local
 // integrals (each band of band_rows rows restarts at zero).
+// finish (may be null): parameter-gradient sums that are complete when this launch starts; the
+// row kernel then finishes them on the side (no launch of its own) and *finish_done is set.
 template <class T>
 hipError_t grad_input_launch(const T* gint, int band_rows, BoxParams<T> prm, T* grad_in, Dims d,
-                             bool normalize, bool exact, hipStream_t stream);
+                             bool normalize, bool exact, hipStream_t stream,
+                             const ParamFinish<T>* finish = nullptr, bool* finish_done = nullptr);
 
 // The streaming pass over grad_output (parameter-gradient sums and/or band-local integral).
 struct StreamPlan {
@@ -89,9 +104,7 @@ template <class T>
 hipError_t grad_params_gather_launch(const T* integ, const T* grad_out, BoxParams<T> prm,
                                      double* acc, Dims d, bool exact, hipStream_t stream);
 template <class T>
-hipError_t grad_params_finish(const double* acc, int batch, int acc_slots, BoxParams<T> prm,
-                              T* gxmin, T* gxmax, T* gymin, T* gymax, int n_boxes, float reparam_h,
-                              float reparam_w, bool normalize, bool exact, hipStream_t stream);
+hipError_t grad_params_finish(const ParamFinish<T>& finish, BoxParams<T> prm, hipStream_t stream);
 
 // real: null, or [4][n] receiving the clipped bounds times their reparametrization factor.
 template <class T>

@@ -39,6 +39,8 @@ for _s in ("f32", "f64"):
         _i, [_vp] * 7 + [_f, _f, _i, _i] + [_vp] * 5 + [_i] * 5 + [_vp, _sz, _vp])
     _SIGNATURES["boxconv_clip_parameters_" + _s] = (_i, [_vp] * 4 + [_i] + [_d] * 4 + [_i, _vp])
     _SIGNATURES["boxconv_clip_reparametrize_" + _s] = (_i, [_vp] * 5 + [_i] + [_d] * 4 + [_i, _vp])
+    _SIGNATURES["boxconv_training_forward_" + _s] = (
+        _i, [_vp] * 8 + [_i] * 5 + [_d] * 4 + [_i, _i] + [_vp, _sz, _vp])
 
 _SIGNATURES["boxconv_forward_fused_f32"] = (_i, [_vp] * 6 + [_i] + [_vp] * 3 + [_i] * 8 + [_vp])
 
@@ -376,6 +378,49 @@ def clip_reparametrize(x_min, x_max, y_min, y_max, reparametrization_h, reparame
                 float(max_input_w), int(bool(exact)), _stream(x_min.device))
         _check(rc, "clip_reparametrize")
     return real[0], real[1], real[2], real[3]
+
+
+def training_forward(input, x_min, x_max, y_min, y_max, reparametrization_h, reparametrization_w,
+                     max_input_h, max_input_w, normalize, exact):
+    """``BoxConv2d.forward`` in training mode as one native call (reference
+    box_convolution_module.py:203-214, box_convolution_function.py:41-46): clips the stored
+    parameters in place, converts them to real pixel units, integrates the input and samples the
+    boxes. Returns ``(input_integrated, output, (x_min, x_max, y_min, y_max) in real units)``."""
+    _require_device(input, "input")
+    if input.dim() != 4:
+        raise RuntimeError("BoxConv2d: input must have 4 dimensions")
+    params = (x_min, x_max, y_min, y_max)
+    for p in params:
+        if p.device != input.device:
+            raise RuntimeError("BoxConv2d: input and parameters are on different devices")
+        if p.dtype != input.dtype:
+            raise RuntimeError("box_convolution: input and parameters have different dtypes (%s, %s)"
+                               % (input.dtype, p.dtype))
+        if not p.is_contiguous():
+            raise RuntimeError("box_convolution: parameters must be contiguous to be clipped in place")
+    sfx = _suffix(input, "input")
+    _check_params(x_min, x_max, y_min, y_max, input.size(1), "BoxConv2d: ")
+    lib = load()
+    input = input.contiguous()
+    B, C, h, w = input.shape
+    F = x_min.size(1)
+    if h < 1 or w < 1:
+        raise RuntimeError("BoxConv2d: input must be at least 1x1")
+    dev = input.device
+    integrated = torch.empty((B, C, h + 1, w + 1), dtype=input.dtype, device=dev)
+    output = torch.empty((B, C * F, h, w), dtype=input.dtype, device=dev)
+    real = torch.empty((4, C, F), dtype=input.dtype, device=dev)
+    with _on_device(dev):
+        nbytes = lib.boxconv_integral_image_workspace_bytes(B * C, h, w)
+        ws = _workspace(nbytes, dev)
+        rc = getattr(lib, "boxconv_training_forward_" + sfx)(
+            _ptr(input), _ptr(x_min), _ptr(x_max), _ptr(y_min), _ptr(y_max), _ptr(real),
+            _ptr(integrated), _ptr(output), B, C, F, h, w,
+            float(reparametrization_h), float(reparametrization_w), float(max_input_h),
+            float(max_input_w), int(bool(normalize)), int(bool(exact)), _ptr(ws), nbytes,
+            _stream(dev))
+    _check(rc, "training_forward")
+    return integrated, output, (real[0], real[1], real[2], real[3])
 
 
 KERNEL_NAMES = ("band_colsum", "band_prefix", "band_scan", "forward_rows", "grad_output_stream",

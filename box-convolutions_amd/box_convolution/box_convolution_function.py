@@ -38,29 +38,30 @@ class BoxConvolutionFunction(torch.autograd.Function):
     normalize, exact) -> output [B, C*F, h, w]``; parameters in stored units.
     (reference box_convolution_function.py:30-65)
 
-    One optional trailing argument that the reference does not have: ``real_parameters``, the four
-    parameters already in real pixel units (what ``reparametrize(..., inverse=True)`` would
-    return for the stored ones). ``BoxConv2d`` passes it in training mode, where the clip kernel
-    produces them on the side.
+    One optional trailing argument that the reference does not have: ``clip_to``, the pair
+    ``(max_input_h, max_input_w)``. When given, the stored parameters are first clipped in place
+    to those limits (what ``BoxConv2d.forward`` does in training mode before calling ``apply``),
+    and clip, unit conversion, integral image and sampling run as one native call.
     """
 
     @staticmethod
     def forward(ctx, input, x_min, x_max, y_min, y_max,
-                reparametrization_h, reparametrization_w, normalize, exact, real_parameters=None):
+                reparametrization_h, reparametrization_w, normalize, exact, clip_to=None):
         ctx.normalize = normalize
         ctx.reparametrization_h = reparametrization_h
         ctx.reparametrization_w = reparametrization_w
         ctx.exact = exact
 
-        if real_parameters is not None:
-            x_min, x_max, y_min, y_max = real_parameters
+        if clip_to is not None:
+            input_integrated, output, (x_min, x_max, y_min, y_max) = _native.training_forward(
+                input, x_min.detach(), x_max.detach(), y_min.detach(), y_max.detach(),
+                reparametrization_h, reparametrization_w, clip_to[0], clip_to[1], normalize, exact)
         else:
             x_min, x_max, y_min, y_max = reparametrize(
                 x_min, x_max, y_min, y_max, reparametrization_h, reparametrization_w, inverse=True)
-
-        input_integrated = _native.integral_image(input)
-        output = _native.box_convolution_forward(
-            input_integrated, x_min, x_max, y_min, y_max, normalize, exact)
+            input_integrated = _native.integral_image(input)
+            output = _native.box_convolution_forward(
+                input_integrated, x_min, x_max, y_min, y_max, normalize, exact)
 
         # The saved forward output of the reference is not kept: the backward kernels rebuild the
         # one sum that needs it from the integral image.
@@ -75,6 +76,5 @@ class BoxConvolutionFunction(torch.autograd.Function):
             input_integrated, x_min, x_max, y_min, y_max, grad_output, None,
             ctx.reparametrization_h, ctx.reparametrization_w,
             ctx.normalize, ctx.exact, *ctx.needs_input_grad[:5])
-        # no gradients for reparametrization_h, reparametrization_w, normalize, exact,
-        # real_parameters
+        # no gradients for reparametrization_h, reparametrization_w, normalize, exact, clip_to
         return tuple(grads) + (None,) * 5

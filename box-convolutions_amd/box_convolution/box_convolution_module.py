@@ -103,21 +103,18 @@ class BoxConv2d(torch.nn.Module):
     def forward(self, input):
         if input.dtype in self._HALF_TYPES:
             return self._forward_half(input)
-        real_parameters = None
+        clip_to = None
         if self.training:
-            if self.x_min.is_cuda:
-                # the projection and the stored -> real conversion in one launch
-                real_parameters = _native.clip_reparametrize(
-                    self.x_min.detach(), self.x_max.detach(), self.y_min.detach(), self.y_max.detach(),
-                    self.reparametrization_h, self.reparametrization_w,
-                    self.max_input_h, self.max_input_w, self.exact)
+            if self.x_min.is_cuda and input.is_cuda and input.dim() == 4 and input.dtype == self.x_min.dtype:
+                # the projection rides along in the native forward call
+                clip_to = (self.max_input_h, self.max_input_w)
             else:
                 self._clip_parameters()
 
         return BoxConvolutionFunction.apply(
             input, self.x_min, self.x_max, self.y_min, self.y_max,
             self.reparametrization_h, self.reparametrization_w, self.normalize, self.exact,
-            real_parameters)
+            clip_to)
 
     def _forward_half(self, input):
         """float16 / bfloat16 input (not offered by the reference's CPU path, and its CUDA path

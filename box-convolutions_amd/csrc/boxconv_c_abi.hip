@@ -178,6 +178,49 @@ int integral_image_impl(const T* in, T* out, int64_t planes, int h, int w, void*
                       "integral image launch");
 }
 
+// BoxConv2d.forward in training mode, natively: clip (+ stored -> real units), integral image,
+// forward sampling; the clip rides on the launch that prepares the integral image's workspace.
+template <class T>
+int training_forward_impl(const T* input, T* x_min, T* x_max, T* y_min, T* y_max, T* real,
+                          T* integ, T* output, int batch, int in_planes, int num_filters, int h,
+                          int w, double reparam_h, double reparam_w, double max_h, double max_w,
+                          int normalize, int exact, void* workspace, size_t workspace_bytes,
+                          void* stream) {
+    if (int rc = check_dims(batch, in_planes, num_filters, h, w)) return rc;
+    const int n = in_planes * num_filters;
+    if (n > 0 && (!x_min || !x_max || !y_min || !y_max || !real))
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "training forward: null parameter pointer");
+    if (!(reparam_h > 0) || !(reparam_w > 0))
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "training forward: reparametrization factors must be positive");
+    const int64_t planes = static_cast<int64_t>(batch) * in_planes;
+    if (planes > 0 && (!input || !integ || (n > 0 && !output)))
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "training forward: null tensor pointer");
+    const size_t need = boxconv_integral_image_workspace_bytes(planes, h, w);
+    if (need > 0 && (workspace == nullptr || workspace_bytes < need ||
+                     reinterpret_cast<uintptr_t>(workspace) % 8 != 0))
+        return fail(BOXCONV_E_WORKSPACE, "training forward: workspace of %zu bytes (8-byte aligned) required, got %zu",
+                    need, workspace_bytes);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    double* aux = static_cast<double*>(workspace);
+    const boxconv::IntegralPlan plan = boxconv::plan_integral(planes, h, w);
+    bool prepared = false;
+    if (int rc = hip_result(boxconv::clip_and_prepare_integral_launch<T>(
+            boxconv::clip_args<T>(x_min, x_max, y_min, y_max, real, n, reparam_h, reparam_w, max_h,
+                                  max_w, exact != 0),
+            planes, w, aux, plan, &prepared, s), "clip launch"))
+        return rc;
+    if (planes == 0) return 0;
+    if (int rc = hip_result(boxconv::integral_image_launch<T>(input, integ, planes, h, w, aux, plan,
+                                                              prepared, false, s),
+                            "integral image launch"))
+        return rc;
+    if (n == 0) return 0;
+    const boxconv::Dims d{in_planes, num_filters, h, w, planes, 0};
+    const boxconv::BoxParams<T> prm{real, real + n, real + 2 * n, real + 3 * n};
+    return hip_result(boxconv::forward_launch<T>(integ, prm, output, d, normalize != 0, exact != 0, s),
+                      "forward launch");
+}
+
 template <class T>
 int forward_impl(const T* integ, const T* x_min, const T* x_max, const T* y_min, const T* y_max,
                  T* output, int batch, int in_planes, int num_filters, int h, int w,
@@ -368,6 +411,31 @@ int boxconv_forward_f64(const double* input_integrated, const double* x_min, con
                         void* stream) {
     return forward_impl<double>(input_integrated, x_min, x_max, y_min, y_max, output, batch,
                                 in_planes, num_filters, h, w, normalize, exact, stream);
+}
+
+int boxconv_training_forward_f32(const float* input, float* x_min, float* x_max, float* y_min,
+                                 float* y_max, float* real_parameters, float* input_integrated,
+                                 float* output, int batch, int in_planes, int num_filters, int h,
+                                 int w, double reparametrization_h, double reparametrization_w,
+                                 double max_input_h, double max_input_w, int normalize, int exact,
+                                 void* workspace, size_t workspace_bytes, void* stream) {
+    return training_forward_impl<float>(input, x_min, x_max, y_min, y_max, real_parameters,
+                                        input_integrated, output, batch, in_planes, num_filters, h, w,
+                                        reparametrization_h, reparametrization_w, max_input_h,
+                                        max_input_w, normalize, exact, workspace, workspace_bytes,
+                                        stream);
+}
+int boxconv_training_forward_f64(const double* input, double* x_min, double* x_max, double* y_min,
+                                 double* y_max, double* real_parameters, double* input_integrated,
+                                 double* output, int batch, int in_planes, int num_filters, int h,
+                                 int w, double reparametrization_h, double reparametrization_w,
+                                 double max_input_h, double max_input_w, int normalize, int exact,
+                                 void* workspace, size_t workspace_bytes, void* stream) {
+    return training_forward_impl<double>(input, x_min, x_max, y_min, y_max, real_parameters,
+                                         input_integrated, output, batch, in_planes, num_filters, h,
+                                         w, reparametrization_h, reparametrization_w, max_input_h,
+                                         max_input_w, normalize, exact, workspace, workspace_bytes,
+                                         stream);
 }
 
 int boxconv_forward_fused_f32(const float* input_integrated, const float* x_min,

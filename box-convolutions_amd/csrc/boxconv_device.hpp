@@ -2,6 +2,8 @@
 // and reductions. Wave size is 64 everywhere (CDNA); nothing here is written for 32-wide waves.
 #pragma once
 
+#include "boxconv_host.hpp"
+
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -310,6 +312,46 @@ __device__ __forceinline__ void load_quad(const double* p, double (&v)[4]) {
     const d2 q0 = __builtin_nontemporal_load(reinterpret_cast<const d2*>(p));
     const d2 q1 = __builtin_nontemporal_load(reinterpret_cast<const d2*>(p) + 1);
     v[0] = q0.x; v[1] = q0.y; v[2] = q1.x; v[3] = q1.y;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Parameter clipping (reference cpu::clipParameters, src/box_convolution.cpp:729-763).
+// Confine both bounds to [-(max_size+1), max_size-1] pixels, and if the box got thinner than
+// min_size - 0.9999 pixels, re-centre it at that thickness. Bounds are stored divided by
+// `reparam`. The midpoint is rounded to T before use, as the reference does.
+template <class T>
+__device__ __forceinline__ void clip_pair(T& pmin, T& pmax, double reparam, double min_size,
+                                          double max_size) {
+    const double inv = 1.0 / reparam;
+    const double floor_v = -(max_size + 1) * inv;
+    const double ceil_v = (max_size - 1) * inv;
+    double lo = fmax(floor_v, fmin(ceil_v, static_cast<double>(pmin)));
+    double hi = fmax(floor_v, fmin(ceil_v, static_cast<double>(pmax)));
+    const double gap = (min_size - 0.9999) * inv;
+    if (lo + gap > hi) {
+        const T mean = static_cast<T>(0.5 * (lo + hi));
+        lo = mean - 0.5 * gap;
+        hi = mean + 0.5 * gap;
+    }
+    pmin = static_cast<T>(lo);
+    pmax = static_cast<T>(hi);
+}
+
+// Box i of a clip job: both pairs clipped in place, and optionally written in real pixel units.
+template <class T>
+__device__ __forceinline__ void clip_box(const ClipArgs<T>& c, int i) {
+    T a = c.xmin[i], b = c.xmax[i];
+    clip_pair(a, b, c.reparam_h, c.min_size, c.max_h);
+    c.xmin[i] = a; c.xmax[i] = b;
+    T lo = c.ymin[i], hi = c.ymax[i];
+    clip_pair(lo, hi, c.reparam_w, c.min_size, c.max_w);
+    c.ymin[i] = lo; c.ymax[i] = hi;
+    if (c.real != nullptr) {
+        // a T tensor times a Python float: the scalar is rounded to T, then one T multiplication
+        const T sh = static_cast<T>(c.reparam_h), sw = static_cast<T>(c.reparam_w);
+        const int n = c.n;
+        c.real[i] = a * sh; c.real[n + i] = b * sh; c.real[2 * n + i] = lo * sw; c.real[3 * n + i] = hi * sw;
+    }
 }
 
 // Workgroup index remapped so that a contiguous range of work items lands on one XCD.

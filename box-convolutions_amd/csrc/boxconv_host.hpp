@@ -36,14 +36,14 @@ struct IntegralPlan {
 // `want`: number of workgroups to aim for.
 IntegralPlan plan_integral(int64_t planes, int h, int w, int64_t want = 1024);
 
-// colsums_ready: aux already holds the per-band column sums (written by another kernel that read
-// the same input), so the first pass is skipped.
+// workspace_prepared: clip_and_prepare_integral_launch ran on this workspace with this plan and
+// reported it prepared (the single-pass kernel then needs no launch to mark its hand-over words).
 // reverse_order: walk the planes last to first. A kernel that re-reads what the previous kernel
 // on the stream just streamed through finds the most recently touched planes still in the
 // 256 MB memory-side cache if it starts with those.
 template <class T>
 hipError_t integral_image_launch(const T* in, T* out, int64_t planes, int h, int w, double* aux,
-                                 const IntegralPlan& plan, bool colsums_ready, bool reverse_order,
+                                 const IntegralPlan& plan, bool workspace_prepared, bool reverse_order,
                                  hipStream_t stream);
 
 template <class T>
@@ -105,6 +105,26 @@ hipError_t grad_params_gather_launch(const T* integ, const T* grad_out, BoxParam
                                      double* acc, Dims d, bool exact, hipStream_t stream);
 template <class T>
 hipError_t grad_params_finish(const ParamFinish<T>& finish, BoxParams<T> prm, hipStream_t stream);
+
+// One clip job: n boxes, bounds stored divided by reparam_*; real: null, or [4][n] receiving the
+// clipped bounds times their reparametrization factor.
+template <class T>
+struct ClipArgs {
+    T* xmin; T* xmax; T* ymin; T* ymax;
+    T* real;
+    int n;
+    double reparam_h, reparam_w, max_h, max_w, min_size;
+};
+template <class T>
+ClipArgs<T> clip_args(T* xmin, T* xmax, T* ymin, T* ymax, T* real, int n, double reparam_h,
+                      double reparam_w, double max_h, double max_w, bool exact);
+
+// The clip job and whatever the integral-image launch that follows needs done to `aux`
+// beforehand, in one launch. *prepared: pass it on to integral_image_launch.
+template <class T>
+hipError_t clip_and_prepare_integral_launch(const ClipArgs<T>& clip, int64_t planes, int w,
+                                            double* aux, const IntegralPlan& plan, bool* prepared,
+                                            hipStream_t stream);
 
 // real: null, or [4][n] receiving the clipped bounds times their reparametrization factor.
 template <class T>

@@ -26,6 +26,7 @@
 // dwords per lane (256 B contiguous per wave instruction).
 
 #include <cstdlib>
+#include <type_traits>
 
 #include "boxconv_device.hpp"
 #include "boxconv_host.hpp"
@@ -372,6 +373,20 @@ __global__ void __launch_bounds__(256) fill_marker_kernel(unsigned long long* ds
     if (i < n) dst[i] = kNotPublished;
 }
 
+// The same fill with a clip job on the side (its first clip_blocks workgroups): what a
+// training-mode forward does before the integral image, in one launch.
+template <class T>
+__global__ void __launch_bounds__(256)
+clip_and_fill_marker_kernel(ClipArgs<T> clip, int clip_blocks, unsigned long long* dst, int64_t n) {
+    if (static_cast<int>(blockIdx.x) < clip_blocks) {
+        const int i = blockIdx.x * 256 + threadIdx.x;
+        if (i < clip.n) clip_box(clip, i);
+        return;
+    }
+    const int64_t i = static_cast<int64_t>(blockIdx.x - clip_blocks) * 256 + threadIdx.x;
+    if (i < n) dst[i] = kNotPublished;
+}
+
 template <int WAVES, int RB, bool VEC, bool FULL>
 __global__ void __launch_bounds__(WAVES * 64)
 band_scan_lookback_kernel(const float* __restrict__ in, float* __restrict__ out, double* aux,
@@ -574,12 +589,14 @@ bool lookback_enabled() {
 
 template <int WAVES>
 hipError_t launch_lookback(const float* in, float* out, double* aux, int64_t planes, int h, int w,
-                           int nb, int R, bool reverse, hipStream_t stream) {
-    const int64_t nsums = planes * static_cast<int64_t>(nb - 1) * w;
-    BOXCONV_LAUNCH("fill_marker", fill_marker_kernel, dim3(static_cast<unsigned>((nsums + 255) / 256)),
-                   dim3(256), 0, stream, reinterpret_cast<unsigned long long*>(aux), nsums);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
+                           int nb, int R, bool reverse, bool prepared, hipStream_t stream) {
+    if (!prepared) {
+        const int64_t nsums = planes * static_cast<int64_t>(nb - 1) * w;
+        BOXCONV_LAUNCH("fill_marker", fill_marker_kernel, dim3(static_cast<unsigned>((nsums + 255) / 256)),
+                       dim3(256), 0, stream, reinterpret_cast<unsigned long long*>(aux), nsums);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
     const int64_t per_xcd = ((planes + kXcds - 1) / kXcds) * nb;     // whole planes per XCD
     const int rev = reverse ? 1 : 0;
     const int spin = lookback_spin_limit();
@@ -596,16 +613,22 @@ hipError_t launch_lookback(const float* in, float* out, double* aux, int64_t pla
     return hipGetLastError();
 }
 template <class T>
-hipError_t lookback_by_width(const T*, T*, double*, int64_t, int, int, int, int, bool, hipStream_t) {
+hipError_t lookback_by_width(const T*, T*, double*, int64_t, int, int, int, int, bool, bool, hipStream_t) {
     return hipErrorInvalidValue;       // float only
 }
 template <>
 hipError_t lookback_by_width<float>(const float* in, float* out, double* aux, int64_t planes, int h,
-                                    int w, int nb, int R, bool reverse, hipStream_t stream) {
-    if (w <= 256)       return launch_lookback<1>(in, out, aux, planes, h, w, nb, R, reverse, stream);
-    else if (w <= 512)  return launch_lookback<2>(in, out, aux, planes, h, w, nb, R, reverse, stream);
-    else if (w <= 1024) return launch_lookback<4>(in, out, aux, planes, h, w, nb, R, reverse, stream);
-    else                return launch_lookback<8>(in, out, aux, planes, h, w, nb, R, reverse, stream);
+                                    int w, int nb, int R, bool reverse, bool prepared,
+                                    hipStream_t stream) {
+    if (w <= 256)       return launch_lookback<1>(in, out, aux, planes, h, w, nb, R, reverse, prepared, stream);
+    else if (w <= 512)  return launch_lookback<2>(in, out, aux, planes, h, w, nb, R, reverse, prepared, stream);
+    else if (w <= 1024) return launch_lookback<4>(in, out, aux, planes, h, w, nb, R, reverse, prepared, stream);
+    else                return launch_lookback<8>(in, out, aux, planes, h, w, nb, R, reverse, prepared, stream);
+}
+
+template <class T>
+bool single_pass_applies(const IntegralPlan& pl) {
+    return pl.lookback && std::is_same<T, float>::value && lookback_enabled();
 }
 
 // Rows this narrow are scanned by band_scan_rows_kernel, which sums the band column sums itself;
@@ -651,14 +674,30 @@ IntegralPlan plan_integral(int64_t planes, int h, int w, int64_t want) {
 }
 
 template <class T>
+hipError_t clip_and_prepare_integral_launch(const ClipArgs<T>& clip, int64_t planes, int w,
+                                            double* aux, const IntegralPlan& pl, bool* prepared,
+                                            hipStream_t stream) {
+    const bool fill = single_pass_applies<T>(pl);
+    *prepared = fill;
+    const int clip_blocks = (clip.n + 255) / 256;
+    const int64_t nsums = fill ? planes * static_cast<int64_t>(pl.nb - 1) * w : 0;
+    const int64_t blocks = clip_blocks + (nsums + 255) / 256;
+    if (blocks == 0) return hipSuccess;
+    BOXCONV_LAUNCH("clip", (clip_and_fill_marker_kernel<T>), dim3(static_cast<unsigned>(blocks)), dim3(256),
+                   0, stream, clip, clip_blocks, reinterpret_cast<unsigned long long*>(aux), nsums);
+    return hipGetLastError();
+}
+
+template <class T>
 hipError_t integral_image_launch(const T* in, T* out, int64_t planes, int h, int w,
-                                 double* aux, const IntegralPlan& pl, bool colsums_ready,
+                                 double* aux, const IntegralPlan& pl, bool workspace_prepared,
                                  bool reverse_order, hipStream_t stream) {
     if (planes == 0) return hipSuccess;
     const int nb = pl.nb, R = pl.R;
-    if (pl.lookback && sizeof(T) == sizeof(float) && !colsums_ready && lookback_enabled())
-        return lookback_by_width<T>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
-    if (nb > 1 && !colsums_ready) {
+    if (single_pass_applies<T>(pl))
+        return lookback_by_width<T>(in, out, aux, planes, h, w, nb, R, reverse_order,
+                                    workspace_prepared, stream);
+    if (nb > 1) {
         const int strips = (w + 1023) / 1024;
         const dim3 grid(static_cast<unsigned>(planes * (nb - 1) * strips));
         if (aligned_for_vec4(in, w))
@@ -697,5 +736,9 @@ template hipError_t integral_image_launch<float>(const float*, float*, int64_t, 
                                                  double*, const IntegralPlan&, bool, bool, hipStream_t);
 template hipError_t integral_image_launch<double>(const double*, double*, int64_t, int, int,
                                                   double*, const IntegralPlan&, bool, bool, hipStream_t);
+template hipError_t clip_and_prepare_integral_launch<float>(const ClipArgs<float>&, int64_t, int, double*,
+                                                            const IntegralPlan&, bool*, hipStream_t);
+template hipError_t clip_and_prepare_integral_launch<double>(const ClipArgs<double>&, int64_t, int, double*,
+                                                             const IntegralPlan&, bool*, hipStream_t);
 
 }  // namespace boxconv

@@ -82,6 +82,30 @@ int boxconv_forward_f64(const double* input_integrated, const double* x_min, con
                         int in_planes, int num_filters, int h, int w, int normalize, int exact,
                         void* stream);
 
+/* ---- training-mode forward in one call -------------------------------------------------------
+ * What `BoxConv2d.forward` does when `self.training` (reference
+ * box_convolution/box_convolution_module.py:203-214 and box_convolution_function.py:41-46):
+ * clip_parameters on the stored bounds (in place), stored -> real units, integral_image,
+ * box_convolution_forward. Same results as boxconv_clip_reparametrize_*, boxconv_integral_image_*
+ * and boxconv_forward_* called in turn, with one launch fewer (the clip shares the launch that
+ * prepares the integral image's workspace).
+ * x_min..y_max: [in_planes*num_filters], stored units, clipped in place. real_parameters:
+ * [4][in_planes*num_filters] out (x_min, x_max, y_min, y_max in pixel units). input_integrated:
+ * [batch, in_planes, h+1, w+1] out. output: [batch, in_planes*num_filters, h, w] out.
+ * workspace: boxconv_integral_image_workspace_bytes(batch*in_planes, h, w) bytes, 8-byte aligned. */
+int boxconv_training_forward_f32(const float* input, float* x_min, float* x_max, float* y_min,
+                                 float* y_max, float* real_parameters, float* input_integrated,
+                                 float* output, int batch, int in_planes, int num_filters, int h,
+                                 int w, double reparametrization_h, double reparametrization_w,
+                                 double max_input_h, double max_input_w, int normalize, int exact,
+                                 void* workspace, size_t workspace_bytes, void* stream);
+int boxconv_training_forward_f64(const double* input, double* x_min, double* x_max, double* y_min,
+                                 double* y_max, double* real_parameters, double* input_integrated,
+                                 double* output, int batch, int in_planes, int num_filters, int h,
+                                 int w, double reparametrization_h, double reparametrization_w,
+                                 double max_input_h, double max_input_w, int normalize, int exact,
+                                 void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---- forward, half-precision output and fused tail (inference) ------------------------------
  * The same box sums as boxconv_forward_f32 (reference src/box_convolution_interface.cpp:13-139),
  * computed in float from a float integral image, with what a network does to them next folded

@@ -279,3 +279,33 @@ def test_training_forward_fuses_clip_and_reparametrize():
         now = [p.detach() for p in (m.x_min, m.x_max, m.y_min, m.y_max)]
         ref = BoxConvolutionFunction.apply(x, *now, m.reparametrization_h, m.reparametrization_w, True, True)
         assert torch.equal(out, ref)
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 4, 20, 30), (1, 2, 2, 96, 256), (2, 1, 3, 70, 1024)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_training_forward_in_one_native_call(shape, dtype):
+    """clip + unit conversion + integral image + sampling as one native call (the clip shares a
+    launch with the preparation of the integral image's workspace where the single-pass
+    integral-image kernel runs) against the same steps called one by one: identical bits."""
+    from box_convolution import BoxConv2d, _native
+    from box_convolution.box_convolution_function import reparametrize
+    B, C, F, h, w = shape
+    random.seed(17)
+    m = BoxConv2d(C, F, h, w).to("cuda", dtype)
+    with torch.no_grad():
+        m.x_min.mul_(2.5); m.y_max.add_(0.3); m.y_min.copy_(m.y_max - 1e-5)
+    x = torch.randn(B, C, h, w, device="cuda", dtype=dtype)
+    stored = [p.detach().clone() for p in (m.x_min, m.x_max, m.y_min, m.y_max)]
+    _native.clip_parameters(*stored, m.reparametrization_h, m.reparametrization_w, h, w, True)
+    real = reparametrize(*stored, m.reparametrization_h, m.reparametrization_w, inverse=True)
+    integ = _native.integral_image(x)
+    out = _native.box_convolution_forward(integ, *real, True, True)
+
+    live = [p.detach() for p in (m.x_min, m.x_max, m.y_min, m.y_max)]
+    got_integ, got_out, got_real = _native.training_forward(
+        x, *live, m.reparametrization_h, m.reparametrization_w, h, w, True, True)
+    for a, b in zip(live, stored):
+        assert torch.equal(a, b)
+    for a, b in zip(got_real, real):
+        assert torch.equal(a, b)
+    assert torch.equal(got_integ, integ) and torch.equal(got_out, out)

@@ -48,7 +48,7 @@ const char* boxconv_last_error(void);
  * a pair of HIP events recorded on the stream it is launched on (so the time is that kernel's
  * alone, whatever else the entry point launches). Names: "band_colsum", "band_prefix",
  * "band_scan", "forward_rows", "grad_output_stream", "grad_input_rows",
- * "param_grad_finalize", "fill_zero", "clip", "forward_gather", "grad_input_gather",
+ * "param_grad_finalize", "fill_zero", "fill_marker", "clip", "forward_gather", "grad_input_gather",
  * "grad_params_gather".
  * NULL or "" disarms. Arming discards earlier measurements.
  * boxconv_profile_collect(&total_ms, &launches): waits for the recorded events, returns the summed

@@ -77,6 +77,76 @@ class BoxConv2d(torch.nn.Module):
             self.x_min, self.x_max, self.y_min, self.y_max,
             self.reparametrization_h, self.reparametrization_w, inplace=True)
 
+    # colours of draw_boxes, one per filter (single-channel plots) or per input channel
+    _BOX_COLORS = (
+        (255, 0, 0), (0, 255, 0), (0, 0, 255), (255, 255, 255), (255, 255, 0), (255, 0, 255),
+        (0, 255, 255), (47, 20, 255), (255, 60, 160), (60, 170, 255), (30, 105, 210),
+        (222, 196, 176), (212, 255, 127), (250, 206, 135), (50, 205, 50), (0, 165, 255),
+        (60, 20, 220), (170, 178, 32))
+
+    def draw_boxes(self, channels=None, resolution=(600, 600), weights=None):
+        """Plot the rectangles of the box filters; returns an ``(H, W, 3)`` uint8 numpy array.
+
+        Same arguments, canvas, centre lines, colours, weighting and box -> pixel mapping as the
+        reference (box_convolution/box_convolution_module.py:99-181). The reference rasterises
+        with ``cv2.rectangle``; here the outlines are drawn with numpy (OpenCV is not a
+        dependency), so line pixels may differ from OpenCV's by a pixel at thick lines.
+
+        channels:   input channels to draw boxes for (default: all).
+        resolution: ``(h, w)`` of the returned image.
+        weights:    ``len(channels) x num_filters`` values in [0, 1]: importance of each box;
+                    unimportant boxes are drawn darker. Default: all ones.
+        """
+        import numpy as np
+
+        if channels is None:
+            channels = range(self.in_planes)
+        channels = list(channels)
+        shape = (len(channels), self.num_filters)
+        if weights is None:
+            weights = np.ones(shape, dtype=np.float32)
+        elif torch.is_tensor(weights):
+            weights = weights.detach().cpu().float().numpy()
+        weights = np.asarray(weights, dtype=np.float32).reshape(shape).clip(0.01, 1.0)
+
+        height, width = resolution
+        image = np.zeros((height, width, 3), dtype=np.uint8)
+        center = (height // 2, width // 2)
+        image[center[0], :] = 70
+        image[:, center[1]] = 70
+
+        x_min, x_max, y_min, y_max = (p.detach().float().cpu() for p in self.get_actual_parameters())
+        x_min = x_min / self.max_input_h * (height / 2) + center[0]
+        y_min = y_min / self.max_input_w * (width / 2) + center[1]
+        x_max = (x_max + 1) / self.max_input_h * (height / 2) + center[0]
+        y_max = (y_max + 1) / self.max_input_w * (width / 2) + center[1]
+
+        thickness = int(round(height / 500 + 0.5))
+
+        def fill(r0, r1, c0, c1, color):          # inclusive pixel ranges, clipped to the canvas
+            r0, r1 = max(min(r0, r1), 0), min(max(r0, r1), height - 1)
+            c0, c1 = max(min(c0, c1), 0), min(max(c0, c1), width - 1)
+            if r0 <= r1 and c0 <= c1:
+                image[r0:r1 + 1, c0:c1 + 1] = color
+
+        for row, channel in enumerate(channels):
+            for f in range(self.num_filters):
+                base = self._BOX_COLORS[(f if len(channels) == 1 else channel) % len(self._BOX_COLORS)]
+                # (the reference indexes the weights by channel number, test it with all channels)
+                color = (np.array(base, dtype=np.float32) * weights[row, f]).astype(np.uint8)
+                top, bottom = float(x_min[channel, f]), float(x_max[channel, f])
+                left, right = float(y_min[channel, f]), float(y_max[channel, f])
+                r0, r1, c0, c1 = (int(round(v)) for v in (top, bottom, left, right))
+                if top > bottom or left > right:   # a box of negative size is drawn filled
+                    fill(r0, r1, c0, c1, color)
+                    continue
+                before, after = thickness // 2, (thickness - 1) // 2
+                fill(r0 - before, r0 + after, c0 - before, c1 + after, color)
+                fill(r1 - before, r1 + after, c0 - before, c1 + after, color)
+                fill(r0 - before, r1 + after, c0 - before, c0 + after, color)
+                fill(r0 - before, r1 + after, c1 - before, c1 + after, color)
+        return image
+
     def get_actual_parameters(self):
         """The four bounds in real pixel units (new tensors)."""
         return reparametrize(

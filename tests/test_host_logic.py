@@ -150,3 +150,30 @@ def test_baseline_workloads_are_reproducible():
     assert torch.equal(sub.grad_output, full.grad_output.view(4, 32, 4, 128, 256)[:, :3].reshape(4, 12, 128, 256))
     assert algorithmic_bytes(2, 16, 8, 512, 1024)["alg"] == 2486765952
     assert algorithmic_bytes(2, 16, 8, 512, 1024)["io"] == 1207959552
+
+
+def test_draw_boxes_canvas_and_rectangles():
+    """draw_boxes: canvas, centre lines, colour and geometry rules of the reference
+    (box_convolution_module.py:99-181); the rasteriser is numpy instead of OpenCV."""
+    m = BoxConv2d(2, 3, 20, 40)
+    with torch.no_grad():
+        for p, v in zip((m.x_min, m.x_max, m.y_min, m.y_max), (-5.0, 4.0, -10.0, 9.0)):
+            p.fill_(v)
+        m.x_min /= m.reparametrization_h; m.x_max /= m.reparametrization_h
+        m.y_min /= m.reparametrization_w; m.y_max /= m.reparametrization_w
+    img = m.draw_boxes(resolution=(200, 400))
+    assert img.shape == (200, 400, 3) and img.dtype == np.uint8
+    assert tuple(img[100, 0]) == (70, 70, 70) and tuple(img[0, 200]) == (70, 70, 70)
+    # box rows -5 .. 4+1 of 20 -> 100 + (-5, 5) / 20 * 100 = 75, 125; columns 200 + (-10, 10) / 40 * 200
+    color = (0, 255, 0)                              # several channels: colour of the last channel drawn
+    for r, c in ((75, 150), (75, 250), (125, 150), (125, 250), (75, 200), (100, 150)):
+        assert tuple(img[r, c]) == color, (r, c)
+    assert tuple(img[90, 180]) == (0, 0, 0)          # inside the outline: untouched
+    # one channel: colour per filter, weights darken, a box with min > max is filled
+    with torch.no_grad():
+        m.x_max[0, 2] = m.x_min[0, 2] - 4.0 / m.reparametrization_h
+    w = torch.tensor([[1.0, 0.5, 1.0]])
+    one = m.draw_boxes(channels=[0], resolution=(200, 400), weights=w)
+    assert tuple(one[68, 220]) == (0, 0, 255)        # filter 2 (blue), filled between rows 60 and 75
+    assert tuple(one[125, 200]) == (0, 127, 0)       # filter 1 (green) at half weight, bottom edge
+    assert m.draw_boxes().shape == (600, 600, 3)

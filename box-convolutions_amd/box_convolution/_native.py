@@ -42,11 +42,12 @@ for _s in ("f32", "f64"):
     _SIGNATURES["boxconv_training_forward_" + _s] = (
         _i, [_vp] * 8 + [_i] * 5 + [_d] * 4 + [_i, _i] + [_vp, _sz, _vp])
 
+_SIGNATURES["boxconv_integral_image_half_f32"] = (_i, [_vp, _i, _vp, _i64, _i, _i, _vp, _sz, _vp])
 _SIGNATURES["boxconv_forward_fused_f32"] = (_i, [_vp] * 6 + [_i] + [_vp] * 3 + [_i] * 8 + [_vp])
 
 EXPORTED_SYMBOLS = tuple(sorted(_SIGNATURES))
 
-# output_dtype codes of boxconv_forward_fused_f32 (include/boxconv.h)
+# element type codes BOXCONV_F32 / BOXCONV_F16 / BOXCONV_BF16 (include/boxconv.h)
 _FUSED_OUTPUT = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 
 _SUFFIX = {torch.float32: "f32", torch.float64: "f64"}
@@ -133,25 +134,39 @@ def _workspace(nbytes, device):
     return torch.empty(nbytes, dtype=torch.uint8, device=device)
 
 
+_MAX_WIDENING_WIDTH = 2048     # widest row boxconv_integral_image_half_f32 reads directly
+
+
 def integral_image(input):
-    """``integral_image(Tensor) -> Tensor`` (reference src/integral_image_interface.cpp:8-27)."""
+    """``integral_image(Tensor) -> Tensor`` (reference src/integral_image_interface.cpp:8-27).
+
+    A float16 / bfloat16 input gives a float32 integral image (sums carried in double, as for
+    float32 input); the reference would integrate it in half precision."""
     if input.dim() < 2:
         raise RuntimeError("integral image input must have >=2 dimensions")
     _require_device(input, "integral image input")
-    sfx = _suffix(input, "integral image input")
+    half = input.dtype in (torch.float16, torch.bfloat16)
+    h, w = input.shape[-2:]
+    if half and (w > _MAX_WIDENING_WIDTH or (h + 1) * (w + 1) * 4 >= 2 ** 31):
+        input, half = input.float(), False
+    sfx = "half_f32" if half else _suffix(input, "integral image input")
     lib = load()
     input = input.contiguous()
-    h, w = input.shape[-2:]
     out_shape = tuple(input.shape[:-2]) + (h + 1, w + 1)
-    output = torch.empty(out_shape, dtype=input.dtype, device=input.device)
+    output = torch.empty(out_shape, dtype=torch.float32 if half else input.dtype, device=input.device)
     if h == 0 or w == 0:
         return output.zero_()
     planes = input.numel() // (h * w)
     with _on_device(input.device):
         nbytes = lib.boxconv_integral_image_workspace_bytes(planes, h, w)
         ws = _workspace(nbytes, input.device)
-        rc = getattr(lib, "boxconv_integral_image_" + sfx)(
-            _ptr(input), _ptr(output), planes, h, w, _ptr(ws), nbytes, _stream(input.device))
+        if half:
+            rc = lib.boxconv_integral_image_half_f32(
+                _ptr(input), _FUSED_OUTPUT[input.dtype], _ptr(output), planes, h, w, _ptr(ws), nbytes,
+                _stream(input.device))
+        else:
+            rc = getattr(lib, "boxconv_integral_image_" + sfx)(
+                _ptr(input), _ptr(output), planes, h, w, _ptr(ws), nbytes, _stream(input.device))
     _check(rc, "integral_image")
     return output
 

@@ -220,7 +220,9 @@ class BoxConv2d(torch.nn.Module):
             real = reparametrize(
                 self.x_min.float(), self.x_max.float(), self.y_min.float(), self.y_max.float(),
                 self.reparametrization_h, self.reparametrization_w, inverse=True)
-            integrated = _native.integral_image(input.float())
+            if input.dtype == torch.float64:
+                input = input.float()
+            integrated = _native.integral_image(input)       # float32 also for half-precision input
             return _native.box_convolution_forward_fused(
                 integrated, *real, self.normalize, self.exact, output_dtype,
                 channel_scale, channel_shift, residual, relu)

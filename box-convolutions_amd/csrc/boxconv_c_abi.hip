@@ -221,6 +221,20 @@ int training_forward_impl(const T* input, T* x_min, T* x_max, T* y_min, T* y_max
                       "forward launch");
 }
 
+template <class TI>
+int integral_image_widening_impl(const TI* in, float* out, int64_t planes, int h, int w,
+                                 void* workspace, size_t workspace_bytes, void* stream) {
+    const size_t need = boxconv_integral_image_workspace_bytes(planes, h, w);
+    if (need > 0 && (workspace == nullptr || workspace_bytes < need ||
+                     reinterpret_cast<uintptr_t>(workspace) % 8 != 0))
+        return fail(BOXCONV_E_WORKSPACE, "integral image: workspace of %zu bytes (8-byte aligned) required, got %zu",
+                    need, workspace_bytes);
+    return hip_result(boxconv::integral_image_widening_launch<TI>(
+                          in, out, planes, h, w, static_cast<double*>(workspace),
+                          boxconv::plan_integral(planes, h, w), static_cast<hipStream_t>(stream)),
+                      "integral image launch");
+}
+
 template <class T>
 int forward_impl(const T* integ, const T* x_min, const T* x_max, const T* y_min, const T* y_max,
                  T* output, int batch, int in_planes, int num_filters, int h, int w,
@@ -411,6 +425,31 @@ int boxconv_forward_f64(const double* input_integrated, const double* x_min, con
                         void* stream) {
     return forward_impl<double>(input_integrated, x_min, x_max, y_min, y_max, output, batch,
                                 in_planes, num_filters, h, w, normalize, exact, stream);
+}
+
+int boxconv_integral_image_half_f32(const void* in, int input_dtype, float* out, int64_t planes,
+                                    int h, int w, void* workspace, size_t workspace_bytes,
+                                    void* stream) {
+    if (planes < 0 || h < 1 || w < 1)
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "integral image: invalid sizes planes=%lld h=%d w=%d",
+                    static_cast<long long>(planes), h, w);
+    if (input_dtype != BOXCONV_F16 && input_dtype != BOXCONV_BF16)
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "integral image: input_dtype %d is neither BOXCONV_F16 nor BOXCONV_BF16",
+                    input_dtype);
+    if (planes == 0) return 0;
+    if (in == nullptr || out == nullptr)
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "integral image: null tensor pointer");
+    if (planes * static_cast<int64_t>(h + 1) * (w + 1) > kMaxElems)
+        return fail(BOXCONV_E_TOO_LARGE, "integral image: output exceeds 2^31-1 elements");
+    if (!boxconv::integral_image_widening_applies(h, w))
+        return fail(BOXCONV_E_TOO_LARGE, "integral image: half-precision input is read directly for rows "
+                    "of at most %d columns and planes below 2 GiB; convert wider inputs to float first",
+                    boxconv::kMaxRowStreamWidth);
+    if (input_dtype == BOXCONV_F16)
+        return integral_image_widening_impl(static_cast<const boxconv::f16_t*>(in), out, planes, h, w,
+                                            workspace, workspace_bytes, stream);
+    return integral_image_widening_impl(static_cast<const boxconv::bf16_t*>(in), out, planes, h, w,
+                                        workspace, workspace_bytes, stream);
 }
 
 int boxconv_training_forward_f32(const float* input, float* x_min, float* x_max, float* y_min,

@@ -224,7 +224,12 @@ __device__ __forceinline__ float widen(bf16_t v) {
 __device__ __forceinline__ void narrow(float v, float& o) { o = v; }
 __device__ __forceinline__ void narrow(double v, double& o) { o = v; }
 __device__ __forceinline__ void narrow(float v, f16_t& o) {
-    o.bits = __builtin_bit_cast(unsigned short, static_cast<_Float16>(v));
+    // The conversion is kept a separate instruction: left to the compiler it is merged with the
+    // multiplication in front of it into one mixed-precision operation that rounds once
+    // (differing from "float32 result, then converted" on ties) and measured slower.
+    unsigned r;
+    asm("v_cvt_f16_f32 %0, %1" : "=v"(r) : "v"(v));
+    o.bits = static_cast<unsigned short>(r);
 }
 __device__ __forceinline__ void narrow(float v, bf16_t& o) {
     o.bits = __builtin_bit_cast(unsigned short, static_cast<__bf16>(v));
@@ -352,6 +357,31 @@ __device__ __forceinline__ void clip_box(const ClipArgs<T>& c, int i) {
         const int n = c.n;
         c.real[i] = a * sh; c.real[n + i] = b * sh; c.real[2 * n + i] = lo * sw; c.real[3 * n + i] = hi * sw;
     }
+}
+
+// The same for half-precision sources (one 8-byte load), widened to float.
+__device__ __forceinline__ void unpack_quad(unsigned lo, unsigned hi, f16_t (&h)[4]) {
+    h[0].bits = static_cast<unsigned short>(lo & 0xffffu); h[1].bits = static_cast<unsigned short>(lo >> 16);
+    h[2].bits = static_cast<unsigned short>(hi & 0xffffu); h[3].bits = static_cast<unsigned short>(hi >> 16);
+}
+template <class H>
+__device__ __forceinline__ void load_quad_half(const H* p, float (&v)[4]) {
+    typedef unsigned u2 __attribute__((ext_vector_type(2)));
+    const u2 q = __builtin_nontemporal_load(reinterpret_cast<const u2*>(p));
+    f16_t raw[4];
+    unpack_quad(q.x, q.y, raw);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) v[k] = widen(H{raw[k].bits});
+}
+__device__ __forceinline__ void load_quad(const f16_t* p, float (&v)[4]) { load_quad_half(p, v); }
+__device__ __forceinline__ void load_quad(const bf16_t* p, float (&v)[4]) { load_quad_half(p, v); }
+
+// K consecutive elements of type TI per lane, element by element, converted to T.
+template <int POLICY, class TI, class T, int K>
+__device__ __forceinline__ void buffer_load_run_as(T (&v)[K], const RowRef& r, int off) {
+#pragma unroll
+    for (int k = 0; k < K; ++k)
+        v[k] = static_cast<T>(widen(buffer_load<POLICY>(r, off + static_cast<int>(sizeof(TI)) * k, TI())));
 }
 
 // Workgroup index remapped so that a contiguous range of work items lands on one XCD.

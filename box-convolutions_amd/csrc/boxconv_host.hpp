@@ -46,6 +46,15 @@ hipError_t integral_image_launch(const T* in, T* out, int64_t planes, int h, int
                                  const IntegralPlan& plan, bool workspace_prepared, bool reverse_order,
                                  hipStream_t stream);
 
+// float32 integral image of a float16 / bfloat16 input (TI = f16_t or bf16_t), for the shapes
+// integral_image_widening_applies() accepts (rows of at most 2048 columns, planes below 2 GiB).
+struct f16_t;
+struct bf16_t;
+template <class TI>
+hipError_t integral_image_widening_launch(const TI* in, float* out, int64_t planes, int h, int w,
+                                          double* aux, const IntegralPlan& plan, hipStream_t stream);
+bool integral_image_widening_applies(int h, int w);
+
 template <class T>
 hipError_t forward_launch(const T* integ, BoxParams<T> prm, T* out, Dims d, bool normalize,
                           bool exact, hipStream_t stream);
@@ -53,8 +62,6 @@ hipError_t forward_launch(const T* integ, BoxParams<T> prm, T* out, Dims d, bool
 // Forward with the output written as TO (float, f16_t or bf16_t; boxconv_device.hpp) and an
 // optional fused tail: y = S * channel_scale[c*F+f] + channel_shift[c*F+f] + residual, then
 // max(y, 0) if relu. Null pointers leave their piece out. Inference only.
-struct f16_t;
-struct bf16_t;
 template <class TO>
 hipError_t forward_fused_launch(const float* integ, BoxParams<float> prm, TO* out, const TO* residual,
                                 const float* channel_scale, const float* channel_shift, bool relu,

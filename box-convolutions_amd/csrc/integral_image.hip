@@ -41,9 +41,10 @@ struct alignas(4 * sizeof(T)) Vec4 { T v[4]; };
 // ---- pass 1 -----------------------------------------------------------------------------------
 // One workgroup per (plane, band, strip of 1024 columns); lane `tid` owns 4 consecutive columns
 // and keeps 8 row loads in flight. VEC: rows are 16-byte aligned and w is a multiple of 4.
-template <class T, bool VEC>
+// TI: element type of the input (T, or a 16-bit type widened to T = float on load).
+template <class T, class TI, bool VEC>
 __global__ void __launch_bounds__(256)
-band_colsum_kernel(const T* __restrict__ in, double* __restrict__ aux, int h, int w, int nb,
+band_colsum_kernel(const TI* __restrict__ in, double* __restrict__ aux, int h, int w, int nb,
                    int R, int strips) {
     constexpr int U = 8;
     unsigned blk = blockIdx.x;                      // (p * (nb-1) + band) * strips + strip
@@ -54,9 +55,9 @@ band_colsum_kernel(const T* __restrict__ in, double* __restrict__ aux, int h, in
     const int r0 = band * R;
     const int r1 = min(h, r0 + R);
     const int c0 = strip * 1024 + 4 * static_cast<int>(threadIdx.x);
-    const T* src = in + p * static_cast<int64_t>(h) * w;
-    const Rows<const T, false> irows(src, w, w, h);
-    const int off = c0 * static_cast<int>(sizeof(T));
+    const TI* src = in + p * static_cast<int64_t>(h) * w;
+    const Rows<const TI, false> irows(src, w, w, h);
+    const int off = c0 * static_cast<int>(sizeof(TI));
 
     double acc[4] = {0.0, 0.0, 0.0, 0.0};
     for (int r = r0; r < r1; r += U) {
@@ -68,7 +69,7 @@ band_colsum_kernel(const T* __restrict__ in, double* __restrict__ aux, int h, in
                 for (int v = 0; v < 4; ++v) x[u][v] = T(0);
                 if (r + u < r1 && c0 < w) load_quad(src + static_cast<int64_t>(r + u) * w + c0, x[u]);
             } else {
-                buffer_load_run<kCacheDefault>(x[u], irows.row(min(r + u, h - 1), r + u < r1), off);
+                buffer_load_run_as<kCacheDefault, TI>(x[u], irows.row(min(r + u, h - 1), r + u < r1), off);
             }
         }
 #pragma unroll
@@ -243,9 +244,9 @@ band_scan_kernel(const T* __restrict__ in, T* __restrict__ out, const double* __
 // next RB rows are in flight while the current ones are scanned; there is one barrier per RB rows
 // (wave totals, double-buffered) and results are stored straight from registers, 4 consecutive
 // elements per lane. VEC: rows are 16-byte aligned and w is a multiple of 4. FULL: w == 4 * threads.
-template <class T, int WAVES, int RB, bool VEC, bool FULL>
+template <class T, class TI, int WAVES, int RB, bool VEC, bool FULL>
 __global__ void __launch_bounds__(WAVES * 64)
-band_scan_rows_kernel(const T* __restrict__ in, T* __restrict__ out, const double* __restrict__ aux,
+band_scan_rows_kernel(const TI* __restrict__ in, T* __restrict__ out, const double* __restrict__ aux,
                       int h, int w, int nb, int R, int64_t total, int64_t per_xcd, int reverse) {
     constexpr int NT = WAVES * 64;
     __shared__ double wave_tot[2][RB][WAVES];
@@ -263,11 +264,11 @@ band_scan_rows_kernel(const T* __restrict__ in, T* __restrict__ out, const doubl
     const int64_t W1 = static_cast<int64_t>(w) + 1;
     const int c0 = 4 * tid;                       // first of the lane's columns
 
-    const T* src = in + p * static_cast<int64_t>(h) * w;
-    const Rows<const T, false> irows(src, w, w, h);
+    const TI* src = in + p * static_cast<int64_t>(h) * w;
+    const Rows<const TI, false> irows(src, w, w, h);
     T* dst = out + p * static_cast<int64_t>(h + 1) * W1;
     const Rows<T, FULL> orows(dst, W1, w + 1, h + 1);
-    const int in_off = c0 * static_cast<int>(sizeof(T));
+    const int in_off = c0 * static_cast<int>(sizeof(TI));
     const int out_off = (c0 + 1) * static_cast<int>(sizeof(T));
 
     if (band == 0)
@@ -294,7 +295,7 @@ band_scan_rows_kernel(const T* __restrict__ in, T* __restrict__ out, const doubl
                 for (int v = 0; v < 4; ++v) x[rb][v] = T(0);
                 if (row < r1 && c0 < w) load_quad(src + static_cast<int64_t>(row) * w + c0, x[rb]);
             } else {
-                buffer_load_run<kCacheStream>(x[rb], irows.row(min(row, h - 1), row < r1), in_off);
+                buffer_load_run_as<kCacheStream, TI>(x[rb], irows.row(min(row, h - 1), row < r1), in_off);
             }
         }
     };
@@ -387,9 +388,9 @@ clip_and_fill_marker_kernel(ClipArgs<T> clip, int clip_blocks, unsigned long lon
     if (i < n) dst[i] = kNotPublished;
 }
 
-template <int WAVES, int RB, bool VEC, bool FULL>
+template <class TI, int WAVES, int RB, bool VEC, bool FULL>
 __global__ void __launch_bounds__(WAVES * 64)
-band_scan_lookback_kernel(const float* __restrict__ in, float* __restrict__ out, double* aux,
+band_scan_lookback_kernel(const TI* __restrict__ in, float* __restrict__ out, double* aux,
                           int h, int w, int nb, int R, int64_t planes, int64_t per_xcd,
                           int reverse, int spin_limit) {
     using T = float;
@@ -410,13 +411,13 @@ band_scan_lookback_kernel(const float* __restrict__ in, float* __restrict__ out,
     const int64_t W1 = static_cast<int64_t>(w) + 1;
     const int c0 = 4 * tid;
 
-    const T* src = in + p * static_cast<int64_t>(h) * w;
-    const Rows<const T, false> irows(src, w, w, h);
+    const TI* src = in + p * static_cast<int64_t>(h) * w;
+    const Rows<const TI, false> irows(src, w, w, h);
     T* dst = out + p * static_cast<int64_t>(h + 1) * W1;
     const Rows<T, FULL> orows(dst, W1, w + 1, h + 1);
     unsigned long long* sums = reinterpret_cast<unsigned long long*>(aux) +
                                p * static_cast<int64_t>(nb - 1) * w;      // [nb-1][w]
-    const int in_off = c0 * static_cast<int>(sizeof(T));
+    const int in_off = c0 * static_cast<int>(sizeof(TI));
     const int out_off = (c0 + 1) * static_cast<int>(sizeof(T));
 
     // Loads are unconditional (a clamped address, the value dropped afterwards) so that all rows
@@ -425,14 +426,14 @@ band_scan_lookback_kernel(const float* __restrict__ in, float* __restrict__ out,
     const unsigned lane_col = lane_in ? static_cast<unsigned>(c0) : 0u;
     auto load_row = [&](int row, bool exists, T (&x)[4]) {
         if (VEC) {
-            const T* rowp = src + static_cast<int64_t>(min(row, h - 1)) * w;
+            const TI* rowp = src + static_cast<int64_t>(min(row, h - 1)) * w;
             load_quad(rowp + lane_col, x);
             if (!(exists && lane_in)) {
 #pragma unroll
                 for (int v = 0; v < 4; ++v) x[v] = T(0);
             }
         } else {
-            buffer_load_run<kCacheStream>(x, irows.row(min(row, h - 1), exists), in_off);
+            buffer_load_run_as<kCacheStream, TI>(x, irows.row(min(row, h - 1), exists), in_off);
         }
     };
 
@@ -551,8 +552,8 @@ hipError_t launch_scan(const T* in, T* out, const double* aux, int64_t planes, i
     return hipGetLastError();
 }
 
-template <class T, int WAVES, int RB>
-hipError_t launch_scan_rows(const T* in, T* out, const double* aux, int64_t planes, int h, int w,
+template <class T, class TI, int WAVES, int RB>
+hipError_t launch_scan_rows(const TI* in, T* out, const double* aux, int64_t planes, int h, int w,
                             int nb, int R, bool reverse, hipStream_t stream) {
     const int64_t total = planes * nb;
     const int64_t per_xcd = (total + kXcds - 1) / kXcds;
@@ -561,7 +562,7 @@ hipError_t launch_scan_rows(const T* in, T* out, const double* aux, int64_t plan
     const dim3 block(WAVES * 64);
     const bool vec = aligned_for_vec4(in, w), full = (w == WAVES * 256);
 #define LAUNCH_ROWS(VEC, FULL)                                                                     \
-    BOXCONV_LAUNCH("band_scan", (band_scan_rows_kernel<T, WAVES, RB, VEC, FULL>), grid, block, 0,  \
+    BOXCONV_LAUNCH("band_scan", (band_scan_rows_kernel<T, TI, WAVES, RB, VEC, FULL>), grid, block, 0,  \
                    stream, in, out, aux, h, w, nb, R, total, per_xcd, rev)
     if (vec && full) LAUNCH_ROWS(true, true);
     else if (vec)    LAUNCH_ROWS(true, false);
@@ -587,8 +588,8 @@ bool lookback_enabled() {
     return e == nullptr || atoi(e) != 0;
 }
 
-template <int WAVES>
-hipError_t launch_lookback(const float* in, float* out, double* aux, int64_t planes, int h, int w,
+template <class TI, int WAVES>
+hipError_t launch_lookback(const TI* in, float* out, double* aux, int64_t planes, int h, int w,
                            int nb, int R, bool reverse, bool prepared, hipStream_t stream) {
     if (!prepared) {
         const int64_t nsums = planes * static_cast<int64_t>(nb - 1) * w;
@@ -604,7 +605,7 @@ hipError_t launch_lookback(const float* in, float* out, double* aux, int64_t pla
     const dim3 block(WAVES * 64);
     const bool vec = aligned_for_vec4(in, w), full = (w == WAVES * 256);
 #define LAUNCH_LOOKBACK(VEC, FULL)                                                                 \
-    BOXCONV_LAUNCH("band_scan", (band_scan_lookback_kernel<WAVES, 4, VEC, FULL>), grid, block, 0,  \
+    BOXCONV_LAUNCH("band_scan", (band_scan_lookback_kernel<TI, WAVES, 4, VEC, FULL>), grid, block, 0,  \
                    stream, in, out, aux, h, w, nb, R, planes, per_xcd, rev, spin)
     if (vec && full) LAUNCH_LOOKBACK(true, true);
     else if (vec)    LAUNCH_LOOKBACK(true, false);
@@ -612,19 +613,22 @@ hipError_t launch_lookback(const float* in, float* out, double* aux, int64_t pla
 #undef LAUNCH_LOOKBACK
     return hipGetLastError();
 }
-template <class T>
-hipError_t lookback_by_width(const T*, T*, double*, int64_t, int, int, int, int, bool, bool, hipStream_t) {
-    return hipErrorInvalidValue;       // float only
-}
-template <>
-hipError_t lookback_by_width<float>(const float* in, float* out, double* aux, int64_t planes, int h,
-                                    int w, int nb, int R, bool reverse, bool prepared,
-                                    hipStream_t stream) {
-    if (w <= 256)       return launch_lookback<1>(in, out, aux, planes, h, w, nb, R, reverse, prepared, stream);
-    else if (w <= 512)  return launch_lookback<2>(in, out, aux, planes, h, w, nb, R, reverse, prepared, stream);
-    else if (w <= 1024) return launch_lookback<4>(in, out, aux, planes, h, w, nb, R, reverse, prepared, stream);
-    else                return launch_lookback<8>(in, out, aux, planes, h, w, nb, R, reverse, prepared, stream);
-}
+template <class T, class TI>
+struct LookbackByWidth {
+    static hipError_t run(const TI*, T*, double*, int64_t, int, int, int, int, bool, bool, hipStream_t) {
+        return hipErrorInvalidValue;       // float output only
+    }
+};
+template <class TI>
+struct LookbackByWidth<float, TI> {
+    static hipError_t run(const TI* in, float* out, double* aux, int64_t planes, int h, int w, int nb,
+                          int R, bool reverse, bool prepared, hipStream_t stream) {
+        if (w <= 256)       return launch_lookback<TI, 1>(in, out, aux, planes, h, w, nb, R, reverse, prepared, stream);
+        else if (w <= 512)  return launch_lookback<TI, 2>(in, out, aux, planes, h, w, nb, R, reverse, prepared, stream);
+        else if (w <= 1024) return launch_lookback<TI, 4>(in, out, aux, planes, h, w, nb, R, reverse, prepared, stream);
+        else                return launch_lookback<TI, 8>(in, out, aux, planes, h, w, nb, R, reverse, prepared, stream);
+    }
+};
 
 template <class T>
 bool single_pass_applies(const IntegralPlan& pl) {
@@ -688,28 +692,49 @@ hipError_t clip_and_prepare_integral_launch(const ClipArgs<T>& clip, int64_t pla
     return hipGetLastError();
 }
 
+// The tiled kernels for widths above 2048 read T only.
+template <class T, class TI>
+struct TiledScan {
+    static hipError_t run(const TI*, T*, double*, int64_t, int, int, int, int, bool, hipStream_t) {
+        return hipErrorInvalidValue;
+    }
+};
 template <class T>
-hipError_t integral_image_launch(const T* in, T* out, int64_t planes, int h, int w,
-                                 double* aux, const IntegralPlan& pl, bool workspace_prepared,
-                                 bool reverse_order, hipStream_t stream) {
+struct TiledScan<T, T> {
+    static hipError_t run(const T* in, T* out, double* aux, int64_t planes, int h, int w, int nb, int R,
+                          bool reverse_order, hipStream_t stream) {
+        // Tile width: one wave covers 256 columns per chunk, four waves 1024.
+        if (w <= 256)        return launch_scan<T, 1, 1, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
+        else if (w <= 512)   return launch_scan<T, 2, 1, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
+        else if (w <= 1024)  return launch_scan<T, 4, 1, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
+        else if (w <= 2048)  return launch_scan<T, 4, 2, 2>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
+        else                 return launch_scan<T, 4, 4, 1>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
+    }
+};
+
+template <class T, class TI>
+hipError_t integral_image_any(const TI* in, T* out, int64_t planes, int h, int w, double* aux,
+                              const IntegralPlan& pl, bool workspace_prepared, bool reverse_order,
+                              hipStream_t stream) {
     if (planes == 0) return hipSuccess;
     const int nb = pl.nb, R = pl.R;
+    const bool by_rows = scan_by_rows(h, w, sizeof(T));
+    if (!by_rows && !std::is_same<T, TI>::value) return hipErrorInvalidValue;
     if (single_pass_applies<T>(pl))
-        return lookback_by_width<T>(in, out, aux, planes, h, w, nb, R, reverse_order,
-                                    workspace_prepared, stream);
+        return LookbackByWidth<T, TI>::run(in, out, aux, planes, h, w, nb, R, reverse_order,
+                                           workspace_prepared, stream);
     if (nb > 1) {
         const int strips = (w + 1023) / 1024;
         const dim3 grid(static_cast<unsigned>(planes * (nb - 1) * strips));
         if (aligned_for_vec4(in, w))
-            BOXCONV_LAUNCH("band_colsum", (band_colsum_kernel<T, true>), grid, dim3(256), 0, stream,
+            BOXCONV_LAUNCH("band_colsum", (band_colsum_kernel<T, TI, true>), grid, dim3(256), 0, stream,
                            in, aux, h, w, nb, R, strips);
         else
-            BOXCONV_LAUNCH("band_colsum", (band_colsum_kernel<T, false>), grid, dim3(256), 0, stream,
+            BOXCONV_LAUNCH("band_colsum", (band_colsum_kernel<T, TI, false>), grid, dim3(256), 0, stream,
                            in, aux, h, w, nb, R, strips);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
-    const bool by_rows = scan_by_rows(h, w, sizeof(T));
     if (nb > 2 && !by_rows) {
         const int64_t n = planes * w;
         BOXCONV_LAUNCH("band_prefix", band_prefix_kernel,
@@ -719,19 +744,34 @@ hipError_t integral_image_launch(const T* in, T* out, int64_t planes, int h, int
         if (e != hipSuccess) return e;
     }
     if (by_rows) {
-        if (w <= 256)       return launch_scan_rows<T, 1, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
-        else if (w <= 512)  return launch_scan_rows<T, 2, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
-        else if (w <= 1024) return launch_scan_rows<T, 4, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
-        else                return launch_scan_rows<T, 8, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
+        if (w <= 256)       return launch_scan_rows<T, TI, 1, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
+        else if (w <= 512)  return launch_scan_rows<T, TI, 2, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
+        else if (w <= 1024) return launch_scan_rows<T, TI, 4, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
+        else                return launch_scan_rows<T, TI, 8, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
     }
-    // Tile width: one wave covers 256 columns per chunk, four waves 1024.
-    if (w <= 256)        return launch_scan<T, 1, 1, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
-    else if (w <= 512)   return launch_scan<T, 2, 1, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
-    else if (w <= 1024)  return launch_scan<T, 4, 1, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
-    else if (w <= 2048)  return launch_scan<T, 4, 2, 2>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
-    else                 return launch_scan<T, 4, 4, 1>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
+    return TiledScan<T, TI>::run(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
 }
 
+template <class T>
+hipError_t integral_image_launch(const T* in, T* out, int64_t planes, int h, int w,
+                                 double* aux, const IntegralPlan& pl, bool workspace_prepared,
+                                 bool reverse_order, hipStream_t stream) {
+    return integral_image_any<T, T>(in, out, planes, h, w, aux, pl, workspace_prepared, reverse_order,
+                                    stream);
+}
+
+template <class TI>
+hipError_t integral_image_widening_launch(const TI* in, float* out, int64_t planes, int h, int w,
+                                          double* aux, const IntegralPlan& pl, hipStream_t stream) {
+    return integral_image_any<float, TI>(in, out, planes, h, w, aux, pl, false, false, stream);
+}
+
+bool integral_image_widening_applies(int h, int w) { return scan_by_rows(h, w, sizeof(float)); }
+
+template hipError_t integral_image_widening_launch<f16_t>(const f16_t*, float*, int64_t, int, int,
+                                                          double*, const IntegralPlan&, hipStream_t);
+template hipError_t integral_image_widening_launch<bf16_t>(const bf16_t*, float*, int64_t, int, int,
+                                                           double*, const IntegralPlan&, hipStream_t);
 template hipError_t integral_image_launch<float>(const float*, float*, int64_t, int, int,
                                                  double*, const IntegralPlan&, bool, bool, hipStream_t);
 template hipError_t integral_image_launch<double>(const double*, double*, int64_t, int, int,

@@ -68,6 +68,21 @@ int boxconv_integral_image_f32(const float* in, float* out, int64_t planes, int 
 int boxconv_integral_image_f64(const double* in, double* out, int64_t planes, int h, int w,
                                void* workspace, size_t workspace_bytes, void* stream);
 
+/* Element type codes of the entry points that read or write half precision. */
+#define BOXCONV_F32 0
+#define BOXCONV_F16 1  /* IEEE binary16 */
+#define BOXCONV_BF16 2 /* bfloat16 */
+
+/* float32 integral image of a float16 / bfloat16 input (input_dtype: BOXCONV_F16 or BOXCONV_BF16),
+ * sums carried in double as for float input. The reference integrates a half-precision tensor in
+ * half precision (src/integral_image_cuda.cu:67-173, AT_DISPATCH_FLOATING_TYPES_AND_HALF), which
+ * overflows at 65504; this is what the inference entry point below is fed instead. Rows of at
+ * most 2048 columns (BOXCONV_E_TOO_LARGE otherwise: convert to float first). Same workspace as
+ * boxconv_integral_image_f32. */
+int boxconv_integral_image_half_f32(const void* in, int input_dtype, float* out, int64_t planes,
+                                    int h, int w, void* workspace, size_t workspace_bytes,
+                                    void* stream);
+
 /* ---- forward ----------------------------------------------------------------------------------
  * Replaces `box_convolution_forward(input_integrated, x_min, x_max, y_min, y_max, normalize,
  * exact) -> Tensor[B, C*F, h, w]`, reference src/box_convolution_interface.cpp:13-139 (kernels:
@@ -120,9 +135,6 @@ int boxconv_training_forward_f64(const double* input, double* x_min, double* x_m
  * scale = gamma / sqrt(var + eps), shift = beta - mean * scale). residual, channel_scale and
  * channel_shift may each be NULL (no residual, scale 1, shift 0). There is no backward for
  * this entry point. */
-#define BOXCONV_F32 0
-#define BOXCONV_F16 1
-#define BOXCONV_BF16 2
 int boxconv_forward_fused_f32(const float* input_integrated, const float* x_min,
                               const float* x_max, const float* y_min, const float* y_max,
                               void* output, int output_dtype, const void* residual,

@@ -56,6 +56,11 @@ def test_argument_errors_are_reported_without_launching(lib):
     rc = lib.boxconv_forward_fused_f32(null, null, null, null, null, null, 1, null, null, null, 0,
                                        1, 1, 1, 4, 4, 1, 1, null)
     assert rc == -1 and b"null" in lib.boxconv_last_error()
+    rc = lib.boxconv_integral_image_half_f32(null, 0, null, 1, 4, 4, null, 0, null)
+    assert rc == -1 and b"input_dtype" in lib.boxconv_last_error()
+    dummy16 = ctypes.c_void_p(256)
+    rc = lib.boxconv_integral_image_half_f32(dummy16, 1, dummy16, 1, 4, 4096, null, 0, null)
+    assert rc == -3 and b"2048" in lib.boxconv_last_error()
     # more than 2^31-1 elements
     rc = lib.boxconv_forward_f32(null, null, null, null, null, null, 64, 64, 64, 4096, 4096, 1, 1, null)
     assert rc == -3

@@ -96,6 +96,29 @@ def test_half_precision_output(hip, shape, dtype):
     assert (got != want.to(dtype)).float().mean().item() < 0.02
 
 
+# planes, h, w: single pass (full rows), two passes (partial rows, vector and element loads),
+# one band, 64 bands, wider than the direct path reads
+HALF_INTEGRAL_SHAPES = [(3, 96, 256), (2, 130, 1024), (2, 70, 2048), (3, 200, 36), (1, 300, 1023),
+                        (2, 100, 1000), (5, 9, 17), (40, 33, 257), (1, 2048, 64), (1, 12, 2500)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("planes,h,w", HALF_INTEGRAL_SHAPES)
+def test_integral_image_of_half_precision_input(hip, monkeypatch, planes, h, w, dtype):
+    """float32 integral image straight from float16 / bfloat16: the same bits as converting the
+    input to float32 first (which is pinned against the oracle in test_gpu_parity.py)."""
+    x = (torch.randn(planes, h, w, device=DEV) * 3 + 0.5).to(dtype)
+    want = hip.integral_image(x.float())
+    got = hip.integral_image(x)
+    assert got.dtype == torch.float32 and torch.equal(got, want)
+    # an odd start address (no 8-byte alignment): element-wise loads
+    flat = torch.empty(x.numel() + 1, device=DEV, dtype=dtype)
+    shifted = flat[1:].view_as(x).copy_(x)
+    assert shifted.data_ptr() % 8 != 0 and torch.equal(hip.integral_image(shifted), want)
+    monkeypatch.setenv("BOXCONV_INTEGRAL_LOOKBACK", "2")     # single pass wherever it applies
+    assert torch.equal(hip.integral_image(x), hip.integral_image(x.float()))
+
+
 def test_argument_checks(hip):
     integ, boxes, scale, shift, residual = setup_case(hip, (1, 2, 2, 8, 8), 3)
     with pytest.raises(RuntimeError, match="float32 integral image"):

@@ -243,7 +243,8 @@ def test_noncontiguous_input_and_dtype_errors(hip):
     assert not x.is_contiguous()
     assert torch.equal(hip.integral_image(x), hip.integral_image(x.contiguous()))
     with pytest.raises(RuntimeError, match="float32 or float64"):
-        hip.integral_image(torch.zeros(1, 4, 4, device=DEV, dtype=torch.float16))
+        hip.integral_image(torch.zeros(1, 4, 4, device=DEV, dtype=torch.int32))
+    # (float16 / bfloat16 inputs are integrated into float32: test_gpu_fused_forward.py)
     z = torch.zeros(2, 1, device=DEV)
     with pytest.raises(RuntimeError, match="as many rows"):
         hip.box_convolution_forward(torch.zeros(1, 3, 5, 5, device=DEV), z, z, z, z, True, True)

@@ -26,7 +26,7 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "box-convolutions_amd"))
 
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E
-SURVEYED_KERNELS = ("grad_output_stream", "band_scan", "band_colsum", "forward_rows", "grad_input_rows")
+TIMED_KERNELS = ("grad_output_stream", "band_scan", "band_colsum", "forward_rows", "grad_input_rows")
 METRIC = "BoxConv2d fwd+bwd ms/iter + effective HBM GB/s (% peak) at 2x16ch 512x1024 fp32"
 
 
@@ -153,7 +153,7 @@ def main():
 
     # which kernel takes the most time per step (one untimed step per candidate)
     per_kernel = {}
-    for name in SURVEYED_KERNELS:
+    for name in TIMED_KERNELS:
         _native.profile_arm(name)
         step()
         ms, launches = _native.profile_collect()

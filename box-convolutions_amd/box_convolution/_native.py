@@ -28,6 +28,7 @@ _SIGNATURES = {
     "boxconv_abi_version": (_i, []),
     "boxconv_last_error": (ctypes.c_char_p, []),
     "boxconv_profile_arm": (_i, [ctypes.c_char_p]),
+    "boxconv_profile_arm_every": (_i, [ctypes.c_char_p, _i]),
     "boxconv_profile_collect": (_i, [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int)]),
     "boxconv_integral_image_workspace_bytes": (_sz, [_i64, _i, _i]),
     "boxconv_backward_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i, _i, _i]),
@@ -443,9 +444,10 @@ KERNEL_NAMES = ("band_colsum", "band_prefix", "band_scan", "forward_rows", "grad
                 "forward_gather", "grad_input_gather", "grad_params_gather")
 
 
-def profile_arm(kernel_name):
-    """Bracket every later launch of `kernel_name` with HIP events (None disarms)."""
-    _check(load().boxconv_profile_arm(kernel_name.encode() if kernel_name else None),
+def profile_arm(kernel_name, every=1):
+    """Bracket later launches of `kernel_name` with HIP events, one launch in `every` (None
+    disarms)."""
+    _check(load().boxconv_profile_arm_every(kernel_name.encode() if kernel_name else None, every),
            "profile_arm")
 
 

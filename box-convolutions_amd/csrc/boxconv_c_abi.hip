@@ -21,6 +21,8 @@ std::mutex g_prof_mutex;
 std::string g_prof_name;                                   // empty: disarmed
 std::vector<std::pair<hipEvent_t, hipEvent_t>> g_prof_events;
 hipEvent_t g_prof_open = nullptr;
+int g_prof_every = 1;                                      // bracket one launch in this many
+long g_prof_seen = 0;                                      // launches of the armed kernel so far
 constexpr size_t kMaxProfiledLaunches = 1 << 16;
 }  // namespace
 
@@ -28,6 +30,7 @@ void profile_before(const char* name, hipStream_t stream) {
     if (g_prof_name.empty()) return;                       // unlocked fast path: not armed
     std::lock_guard<std::mutex> lock(g_prof_mutex);
     if (g_prof_name != name || g_prof_events.size() >= kMaxProfiledLaunches) return;
+    if (g_prof_seen++ % g_prof_every != 0) return;
     hipEvent_t start = nullptr;
     if (hipEventCreate(&start) != hipSuccess) return;
     (void)hipEventRecord(start, stream);
@@ -364,8 +367,13 @@ extern "C" {
 
 int boxconv_abi_version(void) { return BOXCONV_ABI_VERSION; }
 
-int boxconv_profile_arm(const char* kernel_name) {
+int boxconv_profile_arm(const char* kernel_name) { return boxconv_profile_arm_every(kernel_name, 1); }
+
+int boxconv_profile_arm_every(const char* kernel_name, int every) {
+    if (every < 1) return fail(BOXCONV_E_INVALID_ARGUMENT, "profile_arm_every: every must be >= 1");
     std::lock_guard<std::mutex> lock(boxconv::g_prof_mutex);
+    boxconv::g_prof_every = every;
+    boxconv::g_prof_seen = 0;
     for (auto& ev : boxconv::g_prof_events) {
         (void)hipEventDestroy(ev.first);
         (void)hipEventDestroy(ev.second);

@@ -51,9 +51,13 @@ const char* boxconv_last_error(void);
  * "param_grad_finalize", "fill_zero", "fill_marker", "clip", "forward_gather", "grad_input_gather",
  * "grad_params_gather".
  * NULL or "" disarms. Arming discards earlier measurements.
+ * boxconv_profile_arm_every(name, n): the same, but only every n-th launch of that kernel (the
+ * first, the (n+1)-th, ...) is bracketed; an event pair costs a few microseconds of GPU time, which
+ * a caller that also times the whole run may not want to pay at every launch.
  * boxconv_profile_collect(&total_ms, &launches): waits for the recorded events, returns the summed
  * kernel time and the number of launches, then disarms. Process-wide state; meant for benchmarks. */
 int boxconv_profile_arm(const char* kernel_name);
+int boxconv_profile_arm_every(const char* kernel_name, int every);
 int boxconv_profile_collect(double* total_ms, int* launches);
 
 /* ---- integral image ------------------------------------------------------------------------

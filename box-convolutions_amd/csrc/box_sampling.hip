@@ -114,8 +114,13 @@ param_grad_finalize_kernel(FinalizeArgs<T> fa, BoxParams<T> prm) {
 // involves differences between rows, so a row is corrected relative to a reference band (that of
 // the first row this workgroup touches for the filter): the bulk of the integral cancels before
 // it is ever added.
+//
+// Registers: the float shapes that need about 128 registers per lane are held to 128 (four waves per
+// SIMD, i.e. two 512-thread workgroups per CU; one register more would halve that); the wider
+// shapes need far more and are left to the compiler.
 template <class T, int NT, int K, int RB, bool EXACT, bool FULL, bool OFFS>
-__global__ void __launch_bounds__(NT) grad_input_rows_kernel(SampleArgs<T> a, FinalizeArgs<T> fin) {
+__global__ void __launch_bounds__(NT, (sizeof(T) == 4 && (K <= 2 || (K == 3 && !FULL)) ? 4 : 1))
+grad_input_rows_kernel(SampleArgs<T> a, FinalizeArgs<T> fin) {
     static_assert(RB % 4 == 0, "rows are handled in pairs, and pairs alternate between two LDS buffers");
     // Rides along: the first fin.n workgroups each finish the parameter gradients of one box from
     // the sums the preceding launch left (one wave's work; saves a launch of its own).
@@ -145,8 +150,12 @@ __global__ void __launch_bounds__(NT) grad_input_rows_kernel(SampleArgs<T> a, Fi
 #pragma unroll
         for (int k = 0; k < K; ++k) acc[r][k] = T(0);
 
+    // The box of the next filter is fetched while the current one is worked on (scalar loads
+    // whose latency would otherwise sit in front of every filter's first row loads).
+    BoxOfWorkgroup<T> bx_next = load_box(a.prm, c_in * a.F);
     for (int f = 0; f < a.F; ++f) {
-        const BoxOfWorkgroup<T> bx = load_box(a.prm, c_in * a.F + f);
+        const BoxOfWorkgroup<T> bx = bx_next;
+        bx_next = load_box(a.prm, c_in * a.F + min(f + 1, a.F - 1));
         const BoxSplit<T> s = split_grad_input(bx.xmin, bx.xmax, bx.ymin, bx.ymax);
         const T scale = a.normalize
             ? inverse_extent(bx.xmin, bx.xmax, bx.ymin, bx.ymax, EXACT, true, true) : T(1);
@@ -184,6 +193,20 @@ __global__ void __launch_bounds__(NT) grad_input_rows_kernel(SampleArgs<T> a, Fi
 #pragma unroll
             for (int k = 0; k < K; ++k) dst[k] = static_cast<T>(sum[k]);
         };
+        // The first six rows are requested before anything else that reads memory for this
+        // filter (the band offsets below wait for their own rows band by band): their latency
+        // then overlaps with those waits instead of following them.
+        // (Only with one or two columns per lane: with more, keeping six more rows in registers
+        // across the offset code lowers the occupancy, which costs more than the overlap gains.)
+        constexpr bool EARLY_ROWS = K <= 2;
+        T ta[K], bc[K], t0[K], t1[K], b1[K], b2[K];
+        auto first_rows = [&]() {
+            load_row<T, NT, K>(irows.row(first_t), q1, ta);
+            load_row<T, NT, K>(irows.row(first_b), q1, bc);
+            load_pair<T, NT, K, FULL>(irows, i0, s.xlo, s.xhi, h, q1, t0, t1, b1, b2);
+        };
+        if (EARLY_ROWS) first_rows();
+
         bool cross = false;
         T off_b[K];                                 // usual case: offset of bottom minus top rows
 #pragma unroll
@@ -218,10 +241,7 @@ __global__ void __launch_bounds__(NT) grad_input_rows_kernel(SampleArgs<T> a, Fi
                 }
             };
 
-            T ta[K], bc[K], t0[K], t1[K], b1[K], b2[K];
-            load_row<T, NT, K>(irows.row(first_t), q1, ta);
-            load_row<T, NT, K>(irows.row(first_b), q1, bc);
-            load_pair<T, NT, K, FULL>(irows, i0, s.xlo, s.xhi, h, q1, t0, t1, b1, b2);
+            if (!EARLY_ROWS) first_rows();
             correct(ta, first_t, band_t, last_t, off_t);
             correct(t0, clampi(i0 + s.xlo, 0, h), band_t, last_t, off_t);
             correct(t1, clampi(i0 + 1 + s.xlo, 0, h), band_t, last_t, off_t);

@@ -33,13 +33,12 @@ INTEGRAL_SHAPES = [
 ]
 
 
-@pytest.mark.parametrize("single_pass", ["where_faster", "wherever_possible"])
-@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+# (the single-pass kernel is float32 only)
+@pytest.mark.parametrize("dtype,single_pass", [(np.float32, "where_faster"), (np.float64, "where_faster"),
+                                               (np.float32, "wherever_possible")])
 @pytest.mark.parametrize("planes,h,w", INTEGRAL_SHAPES)
 def test_integral_image(hip, oracle, monkeypatch, planes, h, w, dtype, single_pass):
     if single_pass == "wherever_possible":
-        if dtype == np.float64:
-            pytest.skip("the single-pass kernel is float32 only")
         # by default that kernel serves only the shapes it is faster on; reach the others too
         monkeypatch.setenv("BOXCONV_INTEGRAL_LOOKBACK", "2")
     rng = np.random.default_rng(planes * 1000003 + h * 1009 + w)

@@ -459,37 +459,61 @@ band_scan_lookback_kernel(const TI* __restrict__ in, float* __restrict__ out, do
                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 
-    // -- column sums of the bands above
+    // -- column sums of the bands above, four bands per round trip: the first loads of a group
+    // are all in flight together; a band that was not published yet is then waited for on its own
     double colacc[4] = {0.0, 0.0, 0.0, 0.0};
-    for (int b = 0; b < band; ++b) {
-        const unsigned long long* theirs = sums + static_cast<int64_t>(b) * w + c0;
-        unsigned long long bits[4] = {0ull, 0ull, 0ull, 0ull};
-        bool have = false;
-        for (int it = 0; it < spin_limit; ++it) {
-            have = true;
+    constexpr int GROUP = 4;
+    for (int b0 = 0; b0 < band; b0 += GROUP) {
+        unsigned long long bits[GROUP][4];
+        bool have[GROUP];
 #pragma unroll
-            for (int v = 0; v < 4; ++v)
-                if (c0 + v < w) {
-                    bits[v] = __hip_atomic_load(theirs + v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    have = have && bits[v] != kNotPublished;
-                }
-            if (have) break;
-            __builtin_amdgcn_s_sleep(8);
-        }
-        if (have) {
+        for (int u = 0; u < GROUP; ++u) {
+            have[u] = false;
 #pragma unroll
-            for (int v = 0; v < 4; ++v)
-                colacc[v] += __longlong_as_double(static_cast<long long>(bits[v]));
-        } else {
-            double part[4] = {0.0, 0.0, 0.0, 0.0};
-            for (int r = b * R; r < (b + 1) * R; ++r) {      // bands above are complete bands
-                T t[4];
-                load_row(r, true, t);
+            for (int v = 0; v < 4; ++v) bits[u][v] = 0ull;
+            if (b0 + u < band && spin_limit > 0) {
+                const unsigned long long* theirs = sums + static_cast<int64_t>(b0 + u) * w + c0;
 #pragma unroll
-                for (int v = 0; v < 4; ++v) part[v] += static_cast<double>(t[v]);
+                for (int v = 0; v < 4; ++v)
+                    if (c0 + v < w)
+                        bits[u][v] = __hip_atomic_load(theirs + v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
+        }
 #pragma unroll
-            for (int v = 0; v < 4; ++v) colacc[v] += part[v];
+        for (int u = 0; u < GROUP; ++u) {
+            const int b = b0 + u;
+            if (b >= band) break;
+            if (spin_limit > 0) {
+                have[u] = true;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) have[u] = have[u] && bits[u][v] != kNotPublished;
+            }
+            const unsigned long long* theirs = sums + static_cast<int64_t>(b) * w + c0;
+            for (int it = 1; it < spin_limit && !have[u]; ++it) {
+                __builtin_amdgcn_s_sleep(8);
+                have[u] = true;
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    if (c0 + v < w) {
+                        bits[u][v] = __hip_atomic_load(theirs + v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        have[u] = have[u] && bits[u][v] != kNotPublished;
+                    }
+            }
+            if (have[u]) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    colacc[v] += __longlong_as_double(static_cast<long long>(bits[u][v]));
+            } else {
+                double part[4] = {0.0, 0.0, 0.0, 0.0};
+                for (int r = b * R; r < (b + 1) * R; ++r) {      // bands above are complete bands
+                    T t[4];
+                    load_row(r, true, t);
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) part[v] += static_cast<double>(t[v]);
+                }
+#pragma unroll
+                for (int v = 0; v < 4; ++v) colacc[v] += part[v];
+            }
         }
     }
 

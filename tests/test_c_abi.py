@@ -61,6 +61,21 @@ def test_argument_errors_are_reported_without_launching(lib):
     dummy16 = ctypes.c_void_p(256)
     rc = lib.boxconv_integral_image_half_f32(dummy16, 1, dummy16, 1, 4, 4096, null, 0, null)
     assert rc == -3 and b"2048" in lib.boxconv_last_error()
+    assert lib.boxconv_profile_arm_every(b"forward_rows", 0) == -1
+    assert lib.boxconv_profile_arm_every(None, 3) == 0
+    f64 = ctypes.c_double
+    rc = lib.boxconv_training_forward_f32(null, null, null, null, null, null, null, null, 1, 1, 1, 4, 4,
+                                          f64(8.0), f64(8.0), f64(4.0), f64(4.0), 1, 1, null, 0, null)
+    assert rc == -1 and b"null parameter pointer" in lib.boxconv_last_error()
+    rc = lib.boxconv_training_forward_f32(dummy16, dummy16, dummy16, dummy16, dummy16, dummy16, dummy16,
+                                          dummy16, 1, 1, 1, 4, 4, f64(0.0), f64(8.0), f64(4.0), f64(4.0),
+                                          1, 1, null, 0, null)
+    assert rc == -1 and b"positive" in lib.boxconv_last_error()
+    # several bands and no workspace: refused before anything is launched
+    rc = lib.boxconv_training_forward_f32(dummy16, dummy16, dummy16, dummy16, dummy16, dummy16, dummy16,
+                                          dummy16, 2, 16, 8, 512, 1024, f64(8.0), f64(8.0), f64(512.0),
+                                          f64(1024.0), 1, 1, null, 0, null)
+    assert rc == -2 and b"workspace" in lib.boxconv_last_error()
     # more than 2^31-1 elements
     rc = lib.boxconv_forward_f32(null, null, null, null, null, null, 64, 64, 64, 4096, 4096, 1, 1, null)
     assert rc == -3

@@ -188,3 +188,18 @@ def test_bottleneck_tail_in_one_launch(dtype):
         assert torch.allclose(got, want, rtol=1e-5, atol=1e-5)
     else:
         assert torch.all((got.float() - want_in).abs() <= HALF_ULP[dtype] * want_in.abs() + 1e-5)
+
+
+def test_forward_fused_modes_and_double_input():
+    """forward_fused follows the module's normalize / exact switches and takes float64 input
+    (integrated in float32, as the entry point works on a float32 integral image)."""
+    m = make_module(2, 3, 24, 40, 21).eval()
+    x = torch.randn(2, 2, 24, 40, device=DEV)
+    for normalize, exact in ((True, True), (False, True), (True, False), (False, False)):
+        m.normalize, m.exact = normalize, exact
+        with torch.no_grad():
+            want = m(x)
+        assert torch.equal(m.forward_fused(x), want)
+        got = m.forward_fused(x.double(), output_dtype=torch.float32)
+        assert torch.allclose(got, want, rtol=1e-5, atol=1e-5)
+    assert not m.forward_fused(x).requires_grad

@@ -434,13 +434,24 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
     const int i0 = band * a.R;
     const int i1 = min(h, i0 + a.R);
 
+    // The first two rows of grad_output are requested before anything else: they come from HBM
+    // and need nothing but the workgroup's coordinates, so their latency runs alongside the
+    // set-up below (LDS clearing, box parameters, column weights).
+    const int q1 = lane_q1<T>();
+    T g0[K], g1[K];
+    auto load_g = [&](int i, T (&dst)[K]) {
+        const RowRef r = grows.row(min(i, h - 1), i < i1);     // rows past the band read as zeros
+#pragma unroll
+        for (int k = 0; k < K; ++k) dst[k] = load_slot<T, NT, kCacheStream>(r, q1, k);
+    };
+    load_g(i0, g0);
+    load_g(i0 + 1, g1);
+
     // clear the grad_output rows once: pads and the columns beyond w stay zero for good
     for (int e = tid; e < 2 * glen; e += nt) lds.grow[e] = RowPair<T>{T(0), T(0)};
     if (SCAN && band == 0)
         for (int c = tid; c <= w; c += nt) lrows[c] = T(0);                    // integral row 0
     __syncthreads();
-
-    const int q1 = lane_q1<T>();
 
     // lane-constant LDS byte offsets of the pairs (grA, gr) and (gl, glA); the tail weights of the
     // lane's columns go to LDS (read back once per row pair: cheaper than K live registers)
@@ -477,19 +488,12 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
 #pragma unroll
     for (int k = 0; k < K; ++k) colacc[k] = T(0);
 
-    T ta[K], bc[K], t0[K], t1[K], b1[K], b2[K], g0[K], g1[K];
+    T ta[K], bc[K], t0[K], t1[K], b1[K], b2[K];
     if (PARAMS) {
         load_row<T, NT, K>(irows.row(clampi(i0 + s.xlo - 1, 0, h)), q1, ta);
         load_row<T, NT, K>(irows.row(clampi(i0 + s.xhi, 0, h)), q1, bc);
         load_pair<T, NT, K, FULL>(irows, i0, s.xlo, s.xhi, h, q1, t0, t1, b1, b2);
     }
-    auto load_g = [&](int i, T (&dst)[K]) {
-        const RowRef r = grows.row(min(i, h - 1), i < i1);     // rows past the band read as zeros
-#pragma unroll
-        for (int k = 0; k < K; ++k) dst[k] = load_slot<T, NT, kCacheStream>(r, q1, k);
-    };
-    load_g(i0, g0);
-    load_g(i0 + 1, g1);
 
     int flip = 0;
     auto row_pair = [&](int i, auto prefetch_tag) {

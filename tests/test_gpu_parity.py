@@ -70,8 +70,9 @@ def test_integral_image_single_pass_waits_are_bounded(hip, monkeypatch, planes, 
     x = torch.from_numpy(np.random.default_rng(h * w).random((planes, h, w), dtype=np.float32) - 0.3).cuda()
     monkeypatch.setenv("BOXCONV_INTEGRAL_LOOKBACK", "2")       # single pass for every shape it covers
     usual = hip.integral_image(x)
-    monkeypatch.setenv("BOXCONV_INTEGRAL_SPIN", "0")
-    assert torch.equal(hip.integral_image(x), usual)
+    for limit in ("0", "1", "2"):     # never wait / give up at once: a mix of both ways per launch
+        monkeypatch.setenv("BOXCONV_INTEGRAL_SPIN", limit)
+        assert torch.equal(hip.integral_image(x), usual)
     monkeypatch.delenv("BOXCONV_INTEGRAL_SPIN")
     monkeypatch.setenv("BOXCONV_INTEGRAL_LOOKBACK", "0")       # same bands, three launches
     three = hip.integral_image(x)

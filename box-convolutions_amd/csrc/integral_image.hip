@@ -678,16 +678,18 @@ IntegralPlan plan_integral(int64_t planes, int h, int w, int64_t want) {
     int nb = static_cast<int>(std::min<int64_t>(wanted, std::max(1, h / 32)));
     // Where planes get cut anyway and the single-pass kernel covers the width, cut them into
     // bands of at most 32 rows, which that kernel holds in registers.
-    // Measured against the three launches (8..256 planes): 0.6-0.9 of their time for rows of 256,
-    // 512 or 1024 columns (they fill a workgroup of 1, 2 or 4 waves exactly) and planes of up to 16
-    // bands, 1.1 with 64 planes; slower (1.1-1.4) for other widths, for 2048 columns (8 waves: one
-    // workgroup per CU) and for taller planes, where collecting the sums of many bands costs more
-    // than the pass it saves.
+    // Measured against the three launches: 0.6-0.95 of their time when all workgroups are on the
+    // chip at once (they then read, hand over and write in step, so the bands above are never
+    // late) or when there are several times more than fit (they fall out of step and reads overlap
+    // writes); 1.05-1.3 in between, for rows that do not fill the workgroup exactly, and for
+    // planes of more than 32 bands in the first case.
+    const int bands32 = (h + kLookbackRows - 1) / kLookbackRows;
+    const int64_t groups = planes * bands32;                          // workgroups of the launch
+    const int64_t resident = w > 0 ? 256 * (8 / std::max(1, w / 256)) : 0;   // two waves per SIMD each
+    const bool measured_faster = (w == 256 || w == 512 || w == 1024 || w == 2048) &&
+                                 ((groups <= resident && bands32 <= 32) || groups >= 4096);
     const bool single_pass = wanted >= 2 && h > kLookbackRows && scan_by_rows(h, w, sizeof(float)) &&
-                             (h + kLookbackRows - 1) / kLookbackRows <= kLookbackBands &&
-                             (lookback_any_shape() ||
-                              ((w == 256 || w == 512 || w == 1024) &&
-                               h <= 16 * kLookbackRows));
+                             bands32 <= kLookbackBands && (lookback_any_shape() || measured_faster);
     if (single_pass) nb = (h + kLookbackRows - 1) / kLookbackRows;
     nb = std::max(nb, (h + 255) / 256);
     nb = std::max(nb, 1);

@@ -166,20 +166,18 @@ grad_input_rows_kernel(SampleArgs<T> a, FinalizeArgs<T> fin) {
 
         // OFFS: the plane holds a band-local integral (bands of off_R rows, each restarting at
         // zero). Integral row r (1..h) belongs to band (r-1)/off_R; row 0 counts as band 0. The
-        // true integral is the stored row plus the bottom rows of all bands above it; relative to
-        // the reference band (that of the first row touched) only the bottom rows of the bands in
-        // between remain, summed in double.
-        //   Usual case: the RB+2 top rows lie in one band and so do the RB+2 bottom rows. Then
-        //   the top rows need nothing, the bottom rows share one offset vector, and since V only
-        //   contains differences, that vector is added to V once.
-        //   Otherwise (CROSS) every loaded row is corrected on its own; rows only move down, so
-        //   each side tracks the last row of its current band instead of dividing.
+        // true integral I[r] is the stored row L[r] plus base(band(r)), the sum of the bottom rows
+        // of all bands above. V only contains differences of rows, so only differences of base()
+        // matter. The RB+2 rows of a side (top: i+xlo-1 .., bottom: i+xhi ..) span fewer rows than
+        // a band, so each side starts in one band (band_t, band_b) and may cross into the next
+        // once. Relative to band_t:
+        //   I_t = L_t + c * E_t,             c = 1 for top rows beyond band_t, E_t = its bottom row
+        //   I_b = L_b + off_b + d * E_b,     d = 1 for bottom rows beyond band_b, E_b likewise,
+        //                                    off_b = base(band_b) - base(band_t), summed in double
+        // and V picks these up with the weights of its rows: off_b once, E_t and E_b with scalar
+        // weights that are 0 or -+1 except in the one row pair where the crossing happens.
         const int first_t = clampi(i0 + s.xlo - 1, 0, h), final_t = clampi(i0 + RB - 1 + s.xlo, 0, h);
         const int first_b = clampi(i0 + s.xhi, 0, h), final_b = clampi(i0 + RB + s.xhi, 0, h);
-        // reference band: that of the topmost row touched (a box given with min > max has its
-        // "bottom" rows above its "top" rows)
-        const int ref_band = OFFS ? max(min(first_t, first_b) - 1, 0) / a.off_R : 0;
-        const int ref_last = (ref_band + 1) * a.off_R;              // last row of the reference band
         auto bottoms_between = [&](int from_band, int to_band, T (&dst)[K]) {
             double sum[K];
 #pragma unroll
@@ -207,91 +205,80 @@ grad_input_rows_kernel(SampleArgs<T> a, FinalizeArgs<T> fin) {
         };
         if (EARLY_ROWS) first_rows();
 
-        bool cross = false;
-        T off_b[K];                                 // usual case: offset of bottom minus top rows
+        int last_t = h, last_b = h;                 // last row of the band each side starts in
+        bool crossing = false;
+        T off_b[K], e_t[K], e_b[K];
 #pragma unroll
-        for (int k = 0; k < K; ++k) off_b[k] = T(0);
+        for (int k = 0; k < K; ++k) { off_b[k] = T(0); e_t[k] = T(0); e_b[k] = T(0); }
         if (OFFS) {
-            int band_t = ref_band, last_t = ref_last, band_b = ref_band, last_b = ref_last;
-            while (first_t > last_t) { ++band_t; last_t += a.off_R; }
-            while (first_b > last_b) { ++band_b; last_b += a.off_R; }
-            cross = final_t > last_t || final_b > last_b;
-            if (!cross && band_b > band_t) bottoms_between(band_t, band_b, off_b);
-            if (!cross && band_b < band_t) {
+            const int band_t = max(first_t - 1, 0) / a.off_R, band_b = max(first_b - 1, 0) / a.off_R;
+            last_t = (band_t + 1) * a.off_R;
+            last_b = (band_b + 1) * a.off_R;
+            if (band_b > band_t) bottoms_between(band_t, band_b, off_b);
+            if (band_b < band_t) {                  // a box given with min > max
                 bottoms_between(band_b, band_t, off_b);
 #pragma unroll
                 for (int k = 0; k < K; ++k) off_b[k] = -off_b[k];
             }
+            const bool cross_t = final_t > last_t, cross_b = final_b > last_b;
+            crossing = cross_t || cross_b;
+            if (cross_t) load_row<T, NT, K>(irows.row(min(h, last_t)), q1, e_t);
+            if (cross_b) load_row<T, NT, K>(irows.row(min(h, last_b)), q1, e_b);
         }
+        if (!EARLY_ROWS) first_rows();
 
-        auto pass = [&](auto cross_tag) {
-            constexpr bool CROSS = decltype(cross_tag)::value;
-            int band_t = ref_band, band_b = ref_band, last_t = ref_last, last_b = ref_last;
-            T off_t[K];
+        // All RB rows are always computed (rows past the image read clamped, valid rows and
+        // are not stored) and the prefetch of the next pair is decided at compile time:
+        // straight-line code, so loads stay in flight across the barrier.
 #pragma unroll
-            for (int k = 0; k < K; ++k) off_t[k] = T(0);
-            auto correct = [&](T (&row)[K], int row_index, int& cached_band, int& cached_last, T (&cached)[K]) {
-                if constexpr (CROSS) {
-                    if (row_index > cached_last) {              // uniform: depends on the row only
-                        do { ++cached_band; cached_last += a.off_R; } while (row_index > cached_last);
-                        bottoms_between(ref_band, cached_band, cached);
-                    }
+        for (int r = 0; r < RB; r += 2) {
+            const int i = i0 + r;
+            T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {};
+            const bool more = r + 2 < RB;                            // known after unrolling
+            if (more)
+                load_pair<T, NT, K, FULL>(irows, i + 2, s.xlo, s.xhi, h, q1, n0, n1, n2, n3);
+            RowPair<T>* V = vbuf + (((r >> 1) & 1) ? vlen : 0);
+            T v0[K], v1[K];
 #pragma unroll
-                    for (int k = 0; k < K; ++k) row[k] += cached[k];
-                }
-            };
-
-            if (!EARLY_ROWS) first_rows();
-            correct(ta, first_t, band_t, last_t, off_t);
-            correct(t0, clampi(i0 + s.xlo, 0, h), band_t, last_t, off_t);
-            correct(t1, clampi(i0 + 1 + s.xlo, 0, h), band_t, last_t, off_t);
-            correct(bc, first_b, band_b, last_b, off_b);
-            correct(b1, clampi(i0 + 1 + s.xhi, 0, h), band_b, last_b, off_b);
-            correct(b2, clampi(i0 + 2 + s.xhi, 0, h), band_b, last_b, off_b);
-
-            // All RB rows are always computed (rows past the image read clamped, valid rows and
-            // are not stored) and the prefetch of the next pair is decided at compile time:
-            // straight-line code, so loads stay in flight across the barrier.
-#pragma unroll
-            for (int r = 0; r < RB; r += 2) {
-                const int i = i0 + r;
-                T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {};
-                const bool more = r + 2 < RB;                            // known after unrolling
-                if (more)
-                    load_pair<T, NT, K, FULL>(irows, i + 2, s.xlo, s.xhi, h, q1, n0, n1, n2, n3);
-                RowPair<T>* V = vbuf + (((r >> 1) & 1) ? vlen : 0);
-                T v0[K], v1[K];
+            for (int k = 0; k < K; ++k) {
+                v0[k] = blend<T, EXACT>(ta[k], t0[k], bc[k], b1[k], s.fxlo, s.fxhi);
+                v1[k] = blend<T, EXACT>(t0[k], t1[k], b1[k], b2[k], s.fxlo, s.fxhi);
+                if (OFFS) { v0[k] += off_b[k]; v1[k] += off_b[k]; }
+            }
+            if (OFFS && crossing) {                                  // uniform; one batch in four
+                // which of the pair's rows lie beyond their side's first band (scalars)
+                const T cA = T(clampi(i + s.xlo - 1, 0, h) > last_t), c0 = T(clampi(i + s.xlo, 0, h) > last_t),
+                        c1 = T(clampi(i + 1 + s.xlo, 0, h) > last_t);
+                const T dC = T(clampi(i + s.xhi, 0, h) > last_b), d1 = T(clampi(i + 1 + s.xhi, 0, h) > last_b),
+                        d2 = T(clampi(i + 2 + s.xhi, 0, h) > last_b);
+                // weights of E_b and E_t in blend(lo_adv, lo, hi, hi_adv)
+                const T fhi = EXACT ? s.fxhi : T(0), flo = EXACT ? s.fxlo : T(0);
+                const T wb0 = dC + fhi * (d1 - dC), wt0 = flo * (c0 - cA) - c0;
+                const T wb1 = d1 + fhi * (d2 - d1), wt1 = flo * (c1 - c0) - c1;
 #pragma unroll
                 for (int k = 0; k < K; ++k) {
-                    v0[k] = blend<T, EXACT>(ta[k], t0[k], bc[k], b1[k], s.fxlo, s.fxhi);
-                    v1[k] = blend<T, EXACT>(t0[k], t1[k], b1[k], b2[k], s.fxlo, s.fxhi);
-                    if (OFFS && !CROSS) { v0[k] += off_b[k]; v1[k] += off_b[k]; }
-                }
-                publish_rows<T, NT, K, FULL>(V, v0, v1, w, row_bytes, q1);
-                __syncthreads();
-#pragma unroll
-                for (int k = 0; k < K; ++k) {
-                    if (slot_valid<T, NT, FULL>(q1, k, row_bytes)) {
-                        const RowPair<T> o = sample_columns<T, EXACT>(V, lo[k], hi[k], s.fylo, s.fyhi);
-                        acc[r][k] += scale * o.r0;
-                        acc[r + 1][k] += scale * o.r1;
-                    }
-                }
-                if (more) {
-#pragma unroll
-                    for (int k = 0; k < K; ++k) {
-                        ta[k] = t1[k]; bc[k] = b2[k];
-                        t0[k] = n0[k]; t1[k] = n1[k]; b1[k] = n2[k]; b2[k] = n3[k];
-                    }
-                    correct(t0, clampi(i + 2 + s.xlo, 0, h), band_t, last_t, off_t);
-                    correct(t1, clampi(i + 3 + s.xlo, 0, h), band_t, last_t, off_t);
-                    correct(b1, clampi(i + 3 + s.xhi, 0, h), band_b, last_b, off_b);
-                    correct(b2, clampi(i + 4 + s.xhi, 0, h), band_b, last_b, off_b);
+                    v0[k] += wb0 * e_b[k] + wt0 * e_t[k];
+                    v1[k] += wb1 * e_b[k] + wt1 * e_t[k];
                 }
             }
-        };
-        if (OFFS && cross) pass(std::true_type{});
-        else pass(std::false_type{});
+            publish_rows<T, NT, K, FULL>(V, v0, v1, w, row_bytes, q1);
+            __syncthreads();
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                if (slot_valid<T, NT, FULL>(q1, k, row_bytes)) {
+                    const RowPair<T> o = sample_columns<T, EXACT>(V, lo[k], hi[k], s.fylo, s.fyhi);
+                    acc[r][k] += scale * o.r0;
+                    acc[r + 1][k] += scale * o.r1;
+                }
+            }
+            if (more) {
+#pragma unroll
+                for (int k = 0; k < K; ++k) {
+                    ta[k] = t1[k]; bc[k] = b2[k];
+                    t0[k] = n0[k]; t1[k] = n1[k]; b1[k] = n2[k]; b2[k] = n3[k];
+                }
+            }
+        }
     }
 
     // column slot q = j + 1 lands on pixel j; rows past the image get size 0

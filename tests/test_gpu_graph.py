@@ -46,3 +46,43 @@ def test_captured_step_replays_identically(hip, shape):
         torch.cuda.synchronize()
         for got, ref in zip(static_out, want):
             assert torch.equal(got, ref)
+
+
+def test_captured_training_step_replays_identically(hip):
+    """The same for the one-call training forward (clip and the marking of the single-pass
+    integral image's hand-over words in one launch, no memset) followed by the backward."""
+    B, C, F, h, w = 2, 3, 4, 96, 256                    # 3 bands: the single-pass kernel runs
+    rng = np.random.default_rng(7)
+    real = [torch.from_numpy(b).cuda() for b in make_boxes(rng, C, F, h, w, "inside")]
+    reparam_h, reparam_w = 2.5 * h, 2.5 * w
+    stored = [p / s for p, s in zip(real, (reparam_h, reparam_h, reparam_w, reparam_w))]
+
+    def step(x, g):
+        params = [p.clone() for p in stored]
+        integ, out, real_now = hip.training_forward(x, *params, reparam_h, reparam_w, h, w, True, True)
+        grads = hip.box_convolution_backward(integ, *real_now, g, None, reparam_h, reparam_w, True,
+                                             True, True, True, True, True, True)
+        return [out, integ] + list(grads) + list(real_now) + params
+
+    static_x = torch.randn(B, C, h, w, device="cuda")
+    static_g = torch.randn(B, C * F, h, w, device="cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step(static_x, static_g)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_out = step(static_x, static_g)
+
+    for _ in range(4):
+        x = torch.randn_like(static_x)
+        g = torch.randn_like(static_g)
+        want = step(x, g)
+        torch.cuda.synchronize()
+        static_x.copy_(x)
+        static_g.copy_(g)
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, ref in zip(static_out, want):
+            assert torch.equal(got, ref)

@@ -118,13 +118,20 @@ param_grad_finalize_kernel(FinalizeArgs<T> fa, BoxParams<T> prm) {
 // Registers: the float shapes that need about 128 registers per lane are held to 128 (four waves per
 // SIMD, i.e. two 512-thread workgroups per CU; one register more would halve that); the wider
 // shapes need far more and are left to the compiler.
-template <class T, int NT, int K, int RB, bool EXACT, bool FULL, bool OFFS>
-__global__ void __launch_bounds__(NT, (sizeof(T) == 4 && (K <= 2 || (K == 3 && !FULL)) ? 4 : 1))
+//
+// FS > 1 (narrow images, where a row needs one wave only): the workgroup holds FS such waves
+// (threadIdx.y), wave g visits filters g, g + FS, ..., and the FS partial sums are added in wave
+// order at the end. A workgroup of one wave that walks through all F filters is one long chain of
+// memory round trips; on small problems, which cannot fill the chip with workgroups, that chain
+// is the whole run time of the launch.
+template <class T, int NT, int K, int RB, bool EXACT, bool FULL, bool OFFS, int FS = 1>
+__global__ void __launch_bounds__(NT * FS, (FS == 1 && sizeof(T) == 4 && (K <= 2 || (K == 3 && !FULL)) ? 4 : 1))
 grad_input_rows_kernel(SampleArgs<T> a, FinalizeArgs<T> fin) {
     static_assert(RB % 4 == 0, "rows are handled in pairs, and pairs alternate between two LDS buffers");
     // Rides along: the first fin.n workgroups each finish the parameter gradients of one box from
     // the sums the preceding launch left (one wave's work; saves a launch of its own).
-    if (fin.acc != nullptr && blockIdx.x < static_cast<unsigned>(fin.n) && threadIdx.x < 64)
+    if (fin.acc != nullptr && blockIdx.x < static_cast<unsigned>(fin.n) && threadIdx.x < 64 &&
+        (FS == 1 || threadIdx.y == 0))
         finalize_box(fin, a.prm, static_cast<int>(blockIdx.x), static_cast<int>(threadIdx.x));
     unsigned vid = xcd_contiguous_id(a.per_xcd);
     if (vid >= a.total) return;
@@ -137,8 +144,10 @@ grad_input_rows_kernel(SampleArgs<T> a, FinalizeArgs<T> fin) {
     const unsigned row_bytes = static_cast<unsigned>(w) * sizeof(T);
     const int64_t pitch = w + 1;
     const int64_t ipl = static_cast<int64_t>(h + 1) * pitch;
-    RowPair<T>* vbuf = reinterpret_cast<RowPair<T>*>(smem_raw);
     const int vlen = w + 3;
+    // which share of the filters (one value per wave: kept scalar)
+    const int fgroup = FS > 1 ? __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.y)) : 0;
+    RowPair<T>* vbuf = reinterpret_cast<RowPair<T>*>(smem_raw) + fgroup * 2 * vlen;
     clear_row_pads(vbuf, vlen);
     const int i0 = band * RB;
 
@@ -152,10 +161,14 @@ grad_input_rows_kernel(SampleArgs<T> a, FinalizeArgs<T> fin) {
 
     // The box of the next filter is fetched while the current one is worked on (scalar loads
     // whose latency would otherwise sit in front of every filter's first row loads).
-    BoxOfWorkgroup<T> bx_next = load_box(a.prm, c_in * a.F);
-    for (int f = 0; f < a.F; ++f) {
+    // (FS > 1: every wave makes the same number of turns, as the barriers below are the
+    // workgroup's; a wave whose turn has no filter left repeats the last one and adds nothing.)
+    BoxOfWorkgroup<T> bx_next = load_box(a.prm, c_in * a.F + min(fgroup, a.F - 1));
+    for (int f0 = 0; f0 < a.F; f0 += FS) {
+        const int f = min(f0 + fgroup, a.F - 1);
+        const bool counts = f0 + fgroup < a.F;
         const BoxOfWorkgroup<T> bx = bx_next;
-        bx_next = load_box(a.prm, c_in * a.F + min(f + 1, a.F - 1));
+        bx_next = load_box(a.prm, c_in * a.F + min(f + FS, a.F - 1));
         const BoxSplit<T> s = split_grad_input(bx.xmin, bx.xmax, bx.ymin, bx.ymax);
         const T scale = a.normalize
             ? inverse_extent(bx.xmin, bx.xmax, bx.ymin, bx.ymax, EXACT, true, true) : T(1);
@@ -265,7 +278,7 @@ grad_input_rows_kernel(SampleArgs<T> a, FinalizeArgs<T> fin) {
             __syncthreads();
 #pragma unroll
             for (int k = 0; k < K; ++k) {
-                if (slot_valid<T, NT, FULL>(q1, k, row_bytes)) {
+                if (slot_valid<T, NT, FULL>(q1, k, row_bytes) && (FS == 1 || counts)) {
                     const RowPair<T> o = sample_columns<T, EXACT>(V, lo[k], hi[k], s.fylo, s.fyhi);
                     acc[r][k] += scale * o.r0;
                     acc[r + 1][k] += scale * o.r1;
@@ -279,6 +292,28 @@ grad_input_rows_kernel(SampleArgs<T> a, FinalizeArgs<T> fin) {
                 }
             }
         }
+    }
+
+    if constexpr (FS > 1) {
+        // partial sums of waves 1..FS-1 go through LDS (the row buffers are done with) and are
+        // added by wave 0 in wave order
+        T* part = reinterpret_cast<T*>(smem_raw);
+        __syncthreads();
+        if (fgroup > 0) {
+#pragma unroll
+            for (int r = 0; r < RB; ++r)
+#pragma unroll
+                for (int k = 0; k < K; ++k)
+                    part[(((fgroup - 1) * RB + r) * K + k) * NT + threadIdx.x] = acc[r][k];
+        }
+        __syncthreads();
+        if (fgroup > 0) return;
+        for (int g = 1; g < FS; ++g)
+#pragma unroll
+            for (int r = 0; r < RB; ++r)
+#pragma unroll
+                for (int k = 0; k < K; ++k)
+                    acc[r][k] += part[(((g - 1) * RB + r) * K + k) * NT + threadIdx.x];
     }
 
     // column slot q = j + 1 lands on pixel j; rows past the image get size 0
@@ -745,6 +780,15 @@ FinalizeArgs<T> finalize_args(const ParamFinish<T>& f) {
     return fa;
 }
 
+// BOXCONV_GI_SPLIT_FILTERS=0 keeps one wave per workgroup for narrow images (for comparison).
+inline bool split_filters_enabled() {
+    static const bool v = [] {
+        const char* e = std::getenv("BOXCONV_GI_SPLIT_FILTERS");
+        return e == nullptr || std::atoi(e) != 0;
+    }();
+    return v;
+}
+
 template <class T>
 hipError_t grad_input_launch(const T* gint, int band_rows, BoxParams<T> prm, T* grad_in, Dims d,
                              bool normalize, bool exact, hipStream_t stream,
@@ -773,6 +817,11 @@ hipError_t grad_input_launch(const T* gint, int band_rows, BoxParams<T> prm, T* 
     finish_args(a, d.planes * a.nb);
     const dim3 grid(static_cast<unsigned>(a.per_xcd * kXcds));
     const size_t lds = 4 * static_cast<size_t>(d.w + 3) * sizeof(T);
+    // Narrow images on a problem too small to fill the chip: eight waves per workgroup share the
+    // filters (see the kernel).
+    constexpr int FS = 8;
+    const bool split_filters = rc.nt == 64 && d.F >= 4 && a.total <= 4096 && split_filters_enabled();
+    const size_t lds_split = std::max(lds * FS, static_cast<size_t>(FS - 1) * RB * 64 * sizeof(T));
     FinalizeArgs<T> fin{};
     if (finish != nullptr && finish->acc != nullptr && grid.x >= static_cast<unsigned>(finish->n_boxes)) {
         fin = finalize_args(*finish);
@@ -781,7 +830,16 @@ hipError_t grad_input_launch(const T* gint, int band_rows, BoxParams<T> prm, T* 
 #define LAUNCH_GI(NT, KK, EX, FU) \
     if (band_rows > 0) BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, NT, KK, RB, EX, FU, true>), grid, dim3(NT), lds, stream, a, fin); \
     else BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, NT, KK, RB, EX, FU, false>), grid, dim3(NT), lds, stream, a, fin)
-    BOXCONV_DISPATCH_SHAPE_EXACT_FULL(LAUNCH_GI, rc, exact)
+#define LAUNCH_GI_SPLIT(EX, FU) \
+    if (band_rows > 0) BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, 64, 1, RB, EX, FU, true, FS>), grid, dim3(64, FS), lds_split, stream, a, fin); \
+    else BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, 64, 1, RB, EX, FU, false, FS>), grid, dim3(64, FS), lds_split, stream, a, fin)
+    if (split_filters) {
+        if (exact) { if (rc.full) { LAUNCH_GI_SPLIT(true, true); } else { LAUNCH_GI_SPLIT(true, false); } }
+        else       { if (rc.full) { LAUNCH_GI_SPLIT(false, true); } else { LAUNCH_GI_SPLIT(false, false); } }
+    } else {
+        BOXCONV_DISPATCH_SHAPE_EXACT_FULL(LAUNCH_GI, rc, exact)
+    }
+#undef LAUNCH_GI_SPLIT
 #undef LAUNCH_GI
     return hipGetLastError();
 }

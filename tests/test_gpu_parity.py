@@ -150,6 +150,9 @@ SMALL_CASES = [
     (1, 2, 2, 17, 65), (1, 1, 3, 40, 130), (1, 2, 2, 33, 300), (1, 1, 2, 20, 600),
     (1, 1, 2, 12, 1100), (1, 1, 1, 9, 2100), (1, 1, 2, 1, 1), (1, 1, 2, 1, 70), (1, 1, 2, 70, 1),
     (1, 1, 2, 12, 700), (1, 2, 1, 10, 768), (1, 1, 2, 11, 1300), (1, 1, 1, 9, 1536),   # three columns per lane
+    # narrow images with four filters or more: the waves of a grad-input workgroup share the
+    # filters (one turn with idle waves, two turns with the second partial, full-width rows)
+    (1, 2, 4, 9, 20), (1, 2, 11, 19, 33), (2, 1, 16, 12, 64),
 ]
 
 
@@ -194,6 +197,20 @@ def test_backward_across_row_bands(hip, oracle, h, w, kind):
         boxes[1] = (lo - rng.uniform(3.3, 0.5 * h, (C, F))).astype(np.float32)   # x_max < x_min
     cpu, gpu, sc = run_both(hip, oracle, x, tuple(boxes), 3.5 * h, 2.25 * w, False, True, g)
     assert_parity(cpu, gpu, np.float32, "%s %dx%d" % (kind, h, w), **sc)
+
+
+@pytest.mark.parametrize("kind", ["inside", "hanging"])
+def test_backward_across_row_bands_narrow_image(hip, oracle, kind):
+    """As above for an image one wave wide with many filters, where the waves of a grad-input
+    workgroup take the filters in turns."""
+    rng = np.random.default_rng(77 + len(kind))
+    B, C, F, h, w = 2, 2, 9, 150, 48
+    x = rng.standard_normal((B, C, h, w)).astype(np.float32)
+    g = (rng.standard_normal((B, C * F, h, w)) + 0.5).astype(np.float32)
+    boxes = make_boxes(rng, C, F, h, w, kind, away_from_integers=0.05)
+    for normalize in (False, True):
+        cpu, gpu, sc = run_both(hip, oracle, x, tuple(boxes), 3.5 * h, 2.25 * w, normalize, True, g)
+        assert_parity(cpu, gpu, np.float32, "%s normalize=%s" % (kind, normalize), **sc)
 
 
 def test_parameter_gradients_are_reproducible(hip):

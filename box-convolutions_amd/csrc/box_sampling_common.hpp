@@ -193,7 +193,7 @@ __device__ __forceinline__ T gather_box(const T* __restrict__ plane, const BoxSp
 
 // ---------------------------------------------------------------------------------------------
 // Workgroup shapes the row kernels are compiled for: (threads, columns per lane).
-//   (64,1) widths up to 64; (256,1..4) up to 256..1024; (512,1..4) up to 512..2048.
+//   (64,1) widths up to 64; (128,1) up to 128; (256,1..4) up to 256..1024; (512,1..4) up to 512..2048.
 // Each kernel has a preferred size (measured at width 1024: 512 threads for forward and grad
 // input, 256 for the grad_output pass); rows too wide for 4 columns per lane at that size take
 // 512 threads, which bounds the register footprint and the length of the per-lane float
@@ -206,8 +206,8 @@ inline int preferred_row_threads(const char* env_name, int fallback) {
 }
 inline RowConfig row_config(int w, int prefer) {
     RowConfig c;
-    if (w <= 64) {
-        c.nt = 64; c.K = 1;
+    if (w <= 128) {
+        c.nt = w <= 64 ? 64 : 128; c.K = 1;
     } else {
         // fewest column slots (K * threads) that cover the row; the preferred size wins ties
         const int other = prefer == 256 ? 512 : 256;
@@ -269,6 +269,7 @@ void finish_args(SampleArgs<T>& a, int64_t total) {
     }
 #define BOXCONV_DISPATCH_SHAPE(KERNEL, RC, ...)                                      \
     if ((RC).nt == 64)       { KERNEL(64, 1, __VA_ARGS__); }                         \
+    else if ((RC).nt == 128) { KERNEL(128, 1, __VA_ARGS__); }                        \
     else if ((RC).nt == 256) { BOXCONV_DISPATCH_K(KERNEL, 256, (RC).K, __VA_ARGS__) } \
     else                     { BOXCONV_DISPATCH_K(KERNEL, 512, (RC).K, __VA_ARGS__) }
 #define BOXCONV_DISPATCH_SHAPE_EXACT_FULL(KERNEL, RC, EXACT)                         \

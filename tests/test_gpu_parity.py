@@ -153,6 +153,7 @@ SMALL_CASES = [
     # narrow images with four filters or more: the waves of a grad-input workgroup share the
     # filters (one turn with idle waves, two turns with the second partial, full-width rows)
     (1, 2, 4, 9, 20), (1, 2, 11, 19, 33), (2, 1, 16, 12, 64),
+    (1, 2, 2, 12, 128), (1, 1, 3, 35, 100),          # two waves per row, full and partial
 ]
 
 

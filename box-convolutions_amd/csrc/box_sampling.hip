@@ -119,9 +119,9 @@ param_grad_finalize_kernel(FinalizeArgs<T> fa, BoxParams<T> prm) {
 // SIMD, i.e. two 512-thread workgroups per CU; one register more would halve that); the wider
 // shapes need far more and are left to the compiler.
 //
-// FS > 1 (narrow images, where a row needs one wave only): the workgroup holds FS such waves
-// (threadIdx.y), wave g visits filters g, g + FS, ..., and the FS partial sums are added in wave
-// order at the end. A workgroup of one wave that walks through all F filters is one long chain of
+// FS > 1 (narrow images, one column per lane): the workgroup holds FS sets of NT threads
+// (threadIdx.y), set g visits filters g, g + FS, ..., and the FS partial sums are added in that
+// order at the end. A small workgroup that walks through all F filters is one long chain of
 // memory round trips; on small problems, which cannot fill the chip with workgroups, that chain
 // is the whole run time of the launch.
 template <class T, int NT, int K, int RB, bool EXACT, bool FULL, bool OFFS, int FS = 1>
@@ -817,11 +817,14 @@ hipError_t grad_input_launch(const T* gint, int band_rows, BoxParams<T> prm, T* 
     finish_args(a, d.planes * a.nb);
     const dim3 grid(static_cast<unsigned>(a.per_xcd * kXcds));
     const size_t lds = 4 * static_cast<size_t>(d.w + 3) * sizeof(T);
-    // Narrow images on a problem too small to fill the chip: eight waves per workgroup share the
+    // One column per lane on a problem too small to fill the chip: the workgroup is widened to
+    // 512 (one or two waves per row) or 1024 threads (four waves per row) and its waves share the
     // filters (see the kernel).
-    constexpr int FS = 8;
-    const bool split_filters = rc.nt == 64 && d.F >= 4 && a.total <= 4096 && split_filters_enabled();
-    const size_t lds_split = std::max(lds * FS, static_cast<size_t>(FS - 1) * RB * 64 * sizeof(T));
+    const int waves_per_row = rc.nt / 64;
+    const bool split_filters = rc.K == 1 && rc.nt <= 256 && d.F >= 4 &&
+                               a.total * waves_per_row <= 4096 && split_filters_enabled();
+    const int fs = rc.nt == 64 ? 8 : 4;
+    const size_t lds_split = std::max(lds * fs, static_cast<size_t>(fs - 1) * RB * rc.nt * sizeof(T));
     FinalizeArgs<T> fin{};
     if (finish != nullptr && finish->acc != nullptr && grid.x >= static_cast<unsigned>(finish->n_boxes)) {
         fin = finalize_args(*finish);
@@ -830,15 +833,20 @@ hipError_t grad_input_launch(const T* gint, int band_rows, BoxParams<T> prm, T* 
 #define LAUNCH_GI(NT, KK, EX, FU) \
     if (band_rows > 0) BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, NT, KK, RB, EX, FU, true>), grid, dim3(NT), lds, stream, a, fin); \
     else BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, NT, KK, RB, EX, FU, false>), grid, dim3(NT), lds, stream, a, fin)
-#define LAUNCH_GI_SPLIT(EX, FU) \
-    if (band_rows > 0) BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, 64, 1, RB, EX, FU, true, FS>), grid, dim3(64, FS), lds_split, stream, a, fin); \
-    else BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, 64, 1, RB, EX, FU, false, FS>), grid, dim3(64, FS), lds_split, stream, a, fin)
+#define LAUNCH_GI_SPLIT(NT, FS, EX, FU) \
+    if (band_rows > 0) BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, NT, 1, RB, EX, FU, true, FS>), grid, dim3(NT, FS), lds_split, stream, a, fin); \
+    else BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, NT, 1, RB, EX, FU, false, FS>), grid, dim3(NT, FS), lds_split, stream, a, fin)
+#define LAUNCH_GI_SPLIT_SHAPE(EX, FU) \
+    if (rc.nt == 64) { LAUNCH_GI_SPLIT(64, 8, EX, FU); } \
+    else if (rc.nt == 128) { LAUNCH_GI_SPLIT(128, 4, EX, FU); } \
+    else { LAUNCH_GI_SPLIT(256, 4, EX, FU); }
     if (split_filters) {
-        if (exact) { if (rc.full) { LAUNCH_GI_SPLIT(true, true); } else { LAUNCH_GI_SPLIT(true, false); } }
-        else       { if (rc.full) { LAUNCH_GI_SPLIT(false, true); } else { LAUNCH_GI_SPLIT(false, false); } }
+        if (exact) { if (rc.full) { LAUNCH_GI_SPLIT_SHAPE(true, true) } else { LAUNCH_GI_SPLIT_SHAPE(true, false) } }
+        else       { if (rc.full) { LAUNCH_GI_SPLIT_SHAPE(false, true) } else { LAUNCH_GI_SPLIT_SHAPE(false, false) } }
     } else {
         BOXCONV_DISPATCH_SHAPE_EXACT_FULL(LAUNCH_GI, rc, exact)
     }
+#undef LAUNCH_GI_SPLIT_SHAPE
 #undef LAUNCH_GI_SPLIT
 #undef LAUNCH_GI
     return hipGetLastError();

@@ -154,6 +154,8 @@ SMALL_CASES = [
     # filters (one turn with idle waves, two turns with the second partial, full-width rows)
     (1, 2, 4, 9, 20), (1, 2, 11, 19, 33), (2, 1, 16, 12, 64),
     (1, 2, 2, 12, 128), (1, 1, 3, 35, 100),          # two waves per row, full and partial
+    # the same sharing of filters for rows of two and four waves
+    (1, 2, 5, 20, 100), (1, 1, 6, 12, 128), (1, 1, 4, 20, 200), (1, 2, 7, 9, 256),
 ]
 
 
@@ -200,12 +202,13 @@ def test_backward_across_row_bands(hip, oracle, h, w, kind):
     assert_parity(cpu, gpu, np.float32, "%s %dx%d" % (kind, h, w), **sc)
 
 
+@pytest.mark.parametrize("w", [48, 100, 200])
 @pytest.mark.parametrize("kind", ["inside", "hanging"])
-def test_backward_across_row_bands_narrow_image(hip, oracle, kind):
-    """As above for an image one wave wide with many filters, where the waves of a grad-input
-    workgroup take the filters in turns."""
-    rng = np.random.default_rng(77 + len(kind))
-    B, C, F, h, w = 2, 2, 9, 150, 48
+def test_backward_across_row_bands_narrow_image(hip, oracle, kind, w):
+    """As above for images one, two and four waves wide with many filters, where the waves of a
+    grad-input workgroup take the filters in turns."""
+    rng = np.random.default_rng(77 + len(kind) + w)
+    B, C, F, h = 2, 2, 9, 150
     x = rng.standard_normal((B, C, h, w)).astype(np.float32)
     g = (rng.standard_normal((B, C * F, h, w)) + 0.5).astype(np.float32)
     boxes = make_boxes(rng, C, F, h, w, kind, away_from_integers=0.05)

@@ -551,8 +551,8 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
                 const T dt1 = t1[k] - t0[k], db1 = b2[k] - b1[k];
                 T v0 = bc[k] - t0[k], v1 = b1[k] - t1[k];
                 if (EXACT) {
-                    v0 += s.fxhi * db0 + s.fxlo * dt0;
-                    v1 += s.fxhi * db1 + s.fxlo * dt1;
+                    v0 += s.fxhi * db0; v0 += s.fxlo * dt0;
+                    v1 += s.fxhi * db1; v1 += s.fxlo * dt1;
                 }
                 X0[0] = v0; X0[1] = dt0; X0[2] = db0;
                 X1[0] = v1; X1[1] = dt1; X1[2] = db1;
@@ -568,8 +568,8 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
                 const T dt1 = t1[k] - t0[k], db1 = b2[k] - b1[k];
                 T v0 = bc[k] - t0[k], v1 = b1[k] - t1[k];
                 if (EXACT) {
-                    v0 += s.fxhi * db0 + s.fxlo * dt0;
-                    v1 += s.fxhi * db1 + s.fxlo * dt1;
+                    v0 += s.fxhi * db0; v0 += s.fxlo * dt0;
+                    v1 += s.fxhi * db1; v1 += s.fxlo * dt1;
                 }
                 const RowPair<T>* R = at_bytes(G, ir[k]);
                 const RowPair<T>* L = at_bytes(G, il[k]);
@@ -577,7 +577,7 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
                 {
                     const T dr = grA.r0 - gr.r0, dl = gl.r0 - glA.r0;
                     T wq = gr.r0 - gl.r0;
-                    if (EXACT) wq += s.fyhi * dr + s.fylo * dl;
+                    if (EXACT) { wq += s.fyhi * dr; wq += s.fylo * dl; }
                     sum[4] += v0 * wq;
                     sum[1] += db0 * wq;
                     sum[0] -= dt0 * wq;
@@ -587,7 +587,7 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
                 {
                     const T dr = grA.r1 - gr.r1, dl = gl.r1 - glA.r1;
                     T wq = gr.r1 - gl.r1;
-                    if (EXACT) wq += s.fyhi * dr + s.fylo * dl;
+                    if (EXACT) { wq += s.fyhi * dr; wq += s.fylo * dl; }
                     sum[4] += v1 * wq;
                     sum[1] += db1 * wq;
                     sum[0] -= dt1 * wq;

@@ -98,8 +98,13 @@ __device__ __forceinline__ void load_pair(const LoadRows<T>& rows, int i, int xl
 
 template <class T, bool EXACT>
 __device__ __forceinline__ T blend(T lo_adv, T lo, T hi, T hi_adv, T flo, T fhi) {
+    // two fused multiply-adds onto the main difference (written as one sum of two products it
+    // costs a multiply, a fused multiply-add and an add)
     T v = hi - lo;
-    if (EXACT) v += fhi * (hi_adv - hi) + flo * (lo - lo_adv);
+    if (EXACT) {
+        v += fhi * (hi_adv - hi);
+        v += flo * (lo - lo_adv);
+    }
     return v;
 }
 

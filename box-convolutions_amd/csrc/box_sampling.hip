@@ -780,13 +780,11 @@ FinalizeArgs<T> finalize_args(const ParamFinish<T>& f) {
     return fa;
 }
 
-// BOXCONV_GI_SPLIT_FILTERS=0 keeps one wave per workgroup for narrow images (for comparison).
+// BOXCONV_GI_SPLIT_FILTERS=0 keeps the workgroups of narrow images at one row's width (for
+// comparison; read at every call, so that a test can switch it within one process).
 inline bool split_filters_enabled() {
-    static const bool v = [] {
-        const char* e = std::getenv("BOXCONV_GI_SPLIT_FILTERS");
-        return e == nullptr || std::atoi(e) != 0;
-    }();
-    return v;
+    const char* e = std::getenv("BOXCONV_GI_SPLIT_FILTERS");
+    return e == nullptr || std::atoi(e) != 0;
 }
 
 template <class T>

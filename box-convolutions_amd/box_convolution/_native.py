@@ -43,6 +43,7 @@ for _s in ("f32", "f64"):
     _SIGNATURES["boxconv_training_forward_" + _s] = (
         _i, [_vp] * 8 + [_i] * 5 + [_d] * 4 + [_i, _i] + [_vp, _sz, _vp])
 
+_SIGNATURES["boxconv_integral_image_static_f32"] = (_i, [_vp, _vp, _i64, _i, _i, _vp])
 _SIGNATURES["boxconv_integral_image_half_f32"] = (_i, [_vp, _i, _vp, _i64, _i, _i, _vp, _sz, _vp])
 _SIGNATURES["boxconv_forward_fused_f32"] = (_i, [_vp] * 6 + [_i] + [_vp] * 3 + [_i] * 8 + [_vp])
 

@@ -181,6 +181,62 @@ int integral_image_impl(const T* in, T* out, int64_t planes, int h, int w, void*
                       "integral image launch");
 }
 
+// ---- integral image without a caller-provided workspace ----------------------------------------
+// The band column sums (and the hand-over words of the single-pass kernel) live in a fixed array
+// in device memory instead of a workspace argument, for callers that cannot allocate one. Every
+// GPU holds its own copy of the array at its own address; `scratch` itself is only the host-side
+// name of the symbol, so the address is looked up once per device and kept.
+static __device__ __align__(256) unsigned char scratch[BOXCONV_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Address of `scratch` on the current device (null + error message on failure).
+void* static_scratch(int* rc) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) { *rc = hip_result(e, "hipGetDevice"); return nullptr; }
+    if (dev < 0 || dev >= kMaxDevices) {
+        *rc = fail(BOXCONV_E_INVALID_ARGUMENT, "device index %d outside 0..%d", dev, kMaxDevices - 1);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr) {
+            *rc = e != hipSuccess ? hip_result(e, "hipGetSymbolAddress(scratch)")
+                                  : fail(BOXCONV_E_WORKSPACE, "hipGetSymbolAddress(scratch) returned null");
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = ptr;
+    }
+    *rc = 0;
+    return g_scratch_ptr[dev];
+}
+
+int integral_image_static_impl(const float* in, float* out, int64_t planes, int h, int w, void* stream) {
+    if (planes < 0 || h < 1 || w < 1)
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "integral image: invalid sizes planes=%lld h=%d w=%d",
+                    static_cast<long long>(planes), h, w);
+    if (planes == 0) return 0;
+    const size_t need = boxconv_integral_image_workspace_bytes(planes, h, w);
+    if (need > BOXCONV_STATIC_SCRATCH_BYTES)
+        return fail(BOXCONV_E_TOO_LARGE,
+                    "integral image without workspace: planes=%lld h=%d w=%d needs %zu bytes of scratch, "
+                    "the built-in array holds %zu; use boxconv_integral_image_f32 with a workspace",
+                    static_cast<long long>(planes), h, w, need,
+                    static_cast<size_t>(BOXCONV_STATIC_SCRATCH_BYTES));
+    int rc = 0;
+    void* ws = need > 0 ? static_scratch(&rc) : nullptr;
+    if (rc != 0) return rc;
+    // Same checks and launches as the entry point with a workspace argument; the kernels rewrite
+    // every scratch word they later read (column sums, or the hand-over markers, which a fill
+    // kernel resets at every call), so nothing of the previous call is ever seen.
+    return integral_image_impl<float>(in, out, planes, h, w, ws, need, stream);
+}
+
 // BoxConv2d.forward in training mode, natively: clip (+ stored -> real units), integral image,
 // forward sampling; the clip rides on the launch that prepares the integral image's workspace.
 template <class T>
@@ -418,6 +474,11 @@ int boxconv_integral_image_f32(const float* in, float* out, int64_t planes, int 
 int boxconv_integral_image_f64(const double* in, double* out, int64_t planes, int h, int w,
                                void* workspace, size_t workspace_bytes, void* stream) {
     return integral_image_impl<double>(in, out, planes, h, w, workspace, workspace_bytes, stream);
+}
+
+int boxconv_integral_image_static_f32(const float* in, float* out, int64_t planes, int h, int w,
+                                      void* stream) {
+    return integral_image_static_impl(in, out, planes, h, w, stream);
 }
 
 int boxconv_forward_f32(const float* input_integrated, const float* x_min, const float* x_max,

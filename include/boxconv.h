@@ -72,6 +72,21 @@ int boxconv_integral_image_f32(const float* in, float* out, int64_t planes, int 
 int boxconv_integral_image_f64(const double* in, double* out, int64_t planes, int h, int w,
                                void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same integral image for callers that cannot allocate or pass a workspace (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc). It has no counterpart in
+ * the reference. Same kernels and bit-identical results as boxconv_integral_image_f32; the band
+ * column sums go to an array of BOXCONV_STATIC_SCRATCH_BYTES bytes that the library holds in the
+ * memory of every GPU it is loaded on until the process ends. The call allocates and frees
+ * nothing (the first call on a device looks the array's address up once; make that call before
+ * starting a graph capture).
+ * Shapes with boxconv_integral_image_workspace_bytes(planes, h, w) > BOXCONV_STATIC_SCRATCH_BYTES
+ * are refused with BOXCONV_E_TOO_LARGE (the headline shape, 32 planes of 512 x 1024, needs 3.75 MiB).
+ * All calls on one GPU share the one array: two calls that overlap in time on the same GPU (two
+ * streams, two threads) race; calls on one stream are ordered and safe. */
+#define BOXCONV_STATIC_SCRATCH_BYTES (8u << 20)
+int boxconv_integral_image_static_f32(const float* in, float* out, int64_t planes, int h, int w,
+                                      void* stream);
+
 /* Element type codes of the entry points that read or write half precision. */
 #define BOXCONV_F32 0
 #define BOXCONV_F16 1  /* IEEE binary16 */

@@ -28,7 +28,7 @@ sys.path.insert(0, os.path.join(ROOT, "box-convolutions_amd"))
 
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E
 EVENT_EVERY = 5     # launches of the dominant kernel per HIP-event pair in the timed region
-TIMED_KERNELS = ("grad_output_stream", "band_scan", "band_colsum", "forward_rows", "grad_input_rows")
+TIMED_KERNELS = ("grad_output_stream", "band_scan", "band_colsum", "forward_rows", "grad_input_cols")
 METRIC = "BoxConv2d fwd+bwd ms/iter + effective HBM GB/s (% peak) at 2x16ch 512x1024 fp32"
 
 
@@ -41,7 +41,7 @@ def kernel_algorithmic_bytes(ab, elem=4):
         "band_scan": elem * (ab["n_in"] + ab["n_int"]),          # read input, write its integral
         "band_colsum": elem * ab["n_in"],                        # pre-pass over the input
         "forward_rows": elem * (ab["n_int"] + ab["n_out"]),      # read integral, write output
-        "grad_input_rows": elem * (ab["n_gint"] + ab["n_in"]),   # read integral of grad_output, write grad_input
+        "grad_input_cols": elem * (ab["n_gint"] + ab["n_in"]),   # read integral of grad_output, write grad_input
     }
 
 

@@ -441,7 +441,7 @@ def training_forward(input, x_min, x_max, y_min, y_max, reparametrization_h, rep
 
 
 KERNEL_NAMES = ("band_colsum", "band_prefix", "band_scan", "forward_rows", "grad_output_stream",
-                "grad_input_rows", "param_grad_finalize", "fill_zero", "fill_marker", "clip",
+                "grad_input_cols", "param_grad_finalize", "fill_zero", "fill_marker", "clip",
                 "forward_gather", "grad_input_gather", "grad_params_gather")
 
 

@@ -107,204 +107,153 @@ param_grad_finalize_kernel(FinalizeArgs<T> fa, BoxParams<T> prm) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Gradient w.r.t. the input. Work item = (plane p = (b,c), band of RB rows); the F mirrored boxes
-// are visited in order and summed in registers, so no [B,C,F,h,w] temporary exists.
+// Gradient w.r.t. the input from the column workspace M that grad_output_stream_kernel leaves:
+//   M[pf][r][c], r = 0..h, rows `mpitch` elements apart (a multiple of 4: rows are 16-byte aligned)
+//   M[pf][r][c] = sum over the rows i' of the band that row r lies in, i' < r, of A(i')[c],
+// A(i')[c] being row i' of grad_output filtered along the row with the mirrored box (the adjoint
+// of the forward's column formula). Integral row r (1..h) belongs to band (r-1)/off_R and row 0
+// to band 0; each band restarts at zero. The running sum over ALL rows above r is therefore
+// I[r] = M[r] + base(band(r)), base(b) = sum of the bottom rows M[(b'+1)*off_R] of the bands b' < b,
+// and
+//   grad_input(i, c) = sum_f scale_f * ((I[b] - I[t]) + fxhi*(I[bAdv] - I[b]) + fxlo*(I[t] - I[tAdv]))[c]
+// with t = clamp(i+xlo), tAdv = clamp(i+xlo-1), b = clamp(i+xhi), bAdv = clamp(i+xhi+1) in [0,h]
+// from the split of the mirrored box (reference src/box_convolution.cpp:51-67, :286-456; the sum
+// over filters is tmpArray.sum(2), src/box_convolution_interface.cpp:274).
 //
-// OFFS: `src` holds BAND-LOCAL integral images (see grad_output_stream_kernel). A box sum only
-// involves differences between rows, so a row is corrected relative to a reference band (that of
-// the first row this workgroup touches for the filter): the bulk of the integral cancels before
-// it is ever added.
+// Everything is local to a column: no LDS, no barriers, any tiling. A lane owns 4 consecutive
+// columns (one 16-byte load per row); 2^LQ lanes side by side cover a strip of 4*2^LQ columns
+// and RB consecutive output rows; a workgroup holds NTX / 2^LQ such row groups (one for rows of
+// 256 columns and more: then every row index is wave-uniform and stays in scalar registers).
+// Per filter a lane loads the RB+1 rows i0+xlo-1 .. and the RB+1 rows i0+xhi .. (all in flight
+// together); both runs are shorter than a band, so each starts in one band and crosses into the
+// next at most once:
+//   I_t[r] = M_t[r] + [row beyond the first band of the run] * E_t          (relative to that band)
+//   I_b[r] = M_b[r] + off_b + [row beyond ...] * E_b,   off_b = base(band_b) - base(band_t),
+// E = bottom row of the band being left; off_b is summed in double.
 //
-// Registers: the float shapes that need about 128 registers per lane are held to 128 (four waves per
-// SIMD, i.e. two 512-thread workgroups per CU; one register more would halve that); the wider
-// shapes need far more and are left to the compiler.
-//
-// FS > 1 (narrow images, one column per lane): the workgroup holds FS sets of NT threads
-// (threadIdx.y), set g visits filters g, g + FS, ..., and the FS partial sums are added in that
-// order at the end. A small workgroup that walks through all F filters is one long chain of
-// memory round trips; on small problems, which cannot fill the chip with workgroups, that chain
-// is the whole run time of the launch.
-template <class T, int NT, int K, int RB, bool EXACT, bool FULL, bool OFFS, int FS = 1>
-__global__ void __launch_bounds__(NT * FS, (FS == 1 && sizeof(T) == 4 && (K <= 2 || (K == 3 && !FULL)) ? 4 : 1))
-grad_input_rows_kernel(SampleArgs<T> a, FinalizeArgs<T> fin) {
-    static_assert(RB % 4 == 0, "rows are handled in pairs, and pairs alternate between two LDS buffers");
+// FS > 1 (small problems): threadIdx.y selects one of FS sets of threads; set g visits the
+// filters g, g + FS, ... and the FS partial sums are added in that order through LDS at the end.
+// A small launch cannot fill the chip with workgroups, and a workgroup that walks through all F
+// filters alone is one chain of F memory round trips.
+template <class T>
+struct alignas(16) Quad {
+    T v[4];
+};
+
+template <class T, int LQ, int RB, bool EXACT, int FS>
+__global__ void __launch_bounds__((LQ > 6 ? (1 << LQ) : 64) * FS)
+grad_input_cols_kernel(SampleArgs<T> a, FinalizeArgs<T> fin) {
+    constexpr int NTX = LQ > 6 ? (1 << LQ) : 64;
+    constexpr int RG = NTX >> LQ;                    // row groups per workgroup
     // Rides along: the first fin.n workgroups each finish the parameter gradients of one box from
     // the sums the preceding launch left (one wave's work; saves a launch of its own).
     if (fin.acc != nullptr && blockIdx.x < static_cast<unsigned>(fin.n) && threadIdx.x < 64 &&
-        (FS == 1 || threadIdx.y == 0))
+        threadIdx.y == 0)
         finalize_box(fin, a.prm, static_cast<int>(blockIdx.x), static_cast<int>(threadIdx.x));
     unsigned vid = xcd_contiguous_id(a.per_xcd);
     if (vid >= a.total) return;
     if (a.reverse) vid = static_cast<unsigned>(a.total) - 1u - vid;
+    const int h = a.h, w = a.w;
+    const unsigned strips = static_cast<unsigned>((w + (4 << LQ) - 1) / (4 << LQ));
+    const int strip = static_cast<int>(vid % strips);
+    vid /= strips;
     const unsigned nbands = a.nb;
     const int band = static_cast<int>(vid % nbands);
     const int64_t p = vid / nbands;
     const int c_in = static_cast<int>(static_cast<unsigned>(a.plane0 + p) % static_cast<unsigned>(a.C));
-    const int h = a.h, w = a.w;
-    const unsigned row_bytes = static_cast<unsigned>(w) * sizeof(T);
-    const int64_t pitch = w + 1;
-    const int64_t ipl = static_cast<int64_t>(h + 1) * pitch;
-    const int vlen = w + 3;
-    // which share of the filters (one value per wave: kept scalar)
+    const int tid = threadIdx.x;
+    const int rg = RG > 1 ? tid >> LQ : 0;
+    const int i0 = (band * RG + rg) * RB;
+    const int c0 = strip * (4 << LQ) + 4 * (tid & ((1 << LQ) - 1));
+    const bool lane_in = c0 < w;
+    const int cl = lane_in ? c0 : 0;                 // idle lanes read column 0 and store nothing
+    const int64_t mpitch = a.mpitch;
+    const int64_t mplane = static_cast<int64_t>(h + 1) * mpitch;
     const int fgroup = FS > 1 ? __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.y)) : 0;
-    RowPair<T>* vbuf = reinterpret_cast<RowPair<T>*>(smem_raw) + fgroup * 2 * vlen;
-    clear_row_pads(vbuf, vlen);
-    const int i0 = band * RB;
+    const int R = a.off_R;
 
-    const int q1 = lane_q1<T>();
-
-    T acc[RB][K];
+    T acc[RB][4];
 #pragma unroll
     for (int r = 0; r < RB; ++r)
 #pragma unroll
-        for (int k = 0; k < K; ++k) acc[r][k] = T(0);
+        for (int v = 0; v < 4; ++v) acc[r][v] = T(0);
 
-    // The box of the next filter is fetched while the current one is worked on (scalar loads
-    // whose latency would otherwise sit in front of every filter's first row loads).
-    // (FS > 1: every wave makes the same number of turns, as the barriers below are the
-    // workgroup's; a wave whose turn has no filter left repeats the last one and adds nothing.)
-    BoxOfWorkgroup<T> bx_next = load_box(a.prm, c_in * a.F + min(fgroup, a.F - 1));
-    for (int f0 = 0; f0 < a.F; f0 += FS) {
-        const int f = min(f0 + fgroup, a.F - 1);
-        const bool counts = f0 + fgroup < a.F;
-        const BoxOfWorkgroup<T> bx = bx_next;
-        bx_next = load_box(a.prm, c_in * a.F + min(f + FS, a.F - 1));
+#pragma unroll 1
+    for (int f = fgroup; f < a.F; f += FS) {
+        const BoxOfWorkgroup<T> bx = load_box(a.prm, c_in * a.F + f);
         const BoxSplit<T> s = split_grad_input(bx.xmin, bx.xmax, bx.ymin, bx.ymax);
         const T scale = a.normalize
             ? inverse_extent(bx.xmin, bx.xmax, bx.ymin, bx.ymax, EXACT, true, true) : T(1);
-        const LoadRows<T> irows(a.src + (p * a.F + f) * ipl, pitch, w + 1, h + 1);
-
-        unsigned lo[K], hi[K];
-        column_taps<T, NT, K>(lo, hi, s.ylo, s.yhi, w);
-
-        // OFFS: the plane holds a band-local integral (bands of off_R rows, each restarting at
-        // zero). Integral row r (1..h) belongs to band (r-1)/off_R; row 0 counts as band 0. The
-        // true integral I[r] is the stored row L[r] plus base(band(r)), the sum of the bottom rows
-        // of all bands above. V only contains differences of rows, so only differences of base()
-        // matter. The RB+2 rows of a side (top: i+xlo-1 .., bottom: i+xhi ..) span fewer rows than
-        // a band, so each side starts in one band (band_t, band_b) and may cross into the next
-        // once. Relative to band_t:
-        //   I_t = L_t + c * E_t,             c = 1 for top rows beyond band_t, E_t = its bottom row
-        //   I_b = L_b + off_b + d * E_b,     d = 1 for bottom rows beyond band_b, E_b likewise,
-        //                                    off_b = base(band_b) - base(band_t), summed in double
-        // and V picks these up with the weights of its rows: off_b once, E_t and E_b with scalar
-        // weights that are 0 or -+1 except in the one row pair where the crossing happens.
-        const int first_t = clampi(i0 + s.xlo - 1, 0, h), final_t = clampi(i0 + RB - 1 + s.xlo, 0, h);
-        const int first_b = clampi(i0 + s.xhi, 0, h), final_b = clampi(i0 + RB + s.xhi, 0, h);
-        auto bottoms_between = [&](int from_band, int to_band, T (&dst)[K]) {
-            double sum[K];
-#pragma unroll
-            for (int k = 0; k < K; ++k) sum[k] = 0.0;
-            for (int b = from_band; b < to_band; ++b) {
-                T bottom[K];
-                load_row<T, NT, K>(irows.row(min(h, (b + 1) * a.off_R)), q1, bottom);
-#pragma unroll
-                for (int k = 0; k < K; ++k) sum[k] += static_cast<double>(bottom[k]);
-            }
-#pragma unroll
-            for (int k = 0; k < K; ++k) dst[k] = static_cast<T>(sum[k]);
+        const T* plane = a.src + (p * a.F + f) * mplane + cl;
+        auto load_row = [&](int row) {
+            return *reinterpret_cast<const Quad<T>*>(plane + static_cast<int64_t>(row) * mpitch);
         };
-        // The first six rows are requested before anything else that reads memory for this
-        // filter (the band offsets below wait for their own rows band by band): their latency
-        // then overlaps with those waits instead of following them.
-        // (Only with one or two columns per lane: with more, keeping six more rows in registers
-        // across the offset code lowers the occupancy, which costs more than the overlap gains.)
-        constexpr bool EARLY_ROWS = K <= 2;
-        T ta[K], bc[K], t0[K], t1[K], b1[K], b2[K];
-        auto first_rows = [&]() {
-            load_row<T, NT, K>(irows.row(first_t), q1, ta);
-            load_row<T, NT, K>(irows.row(first_b), q1, bc);
-            load_pair<T, NT, K, FULL>(irows, i0, s.xlo, s.xhi, h, q1, t0, t1, b1, b2);
-        };
-        if (EARLY_ROWS) first_rows();
 
-        int last_t = h, last_b = h;                 // last row of the band each side starts in
-        bool crossing = false;
-        T off_b[K], e_t[K], e_b[K];
+        // rows of the two runs; rt[r+1], rb[r] are the plain and rt[r], rb[r+1] the advanced rows
+        // of output row i0 + r
+        int rt[RB + 1], rb[RB + 1];
+        Quad<T> Tq[RB + 1], Bq[RB + 1];
 #pragma unroll
-        for (int k = 0; k < K; ++k) { off_b[k] = T(0); e_t[k] = T(0); e_b[k] = T(0); }
-        if (OFFS) {
-            const int band_t = max(first_t - 1, 0) / a.off_R, band_b = max(first_b - 1, 0) / a.off_R;
-            last_t = (band_t + 1) * a.off_R;
-            last_b = (band_b + 1) * a.off_R;
-            if (band_b > band_t) bottoms_between(band_t, band_b, off_b);
-            if (band_b < band_t) {                  // a box given with min > max
-                bottoms_between(band_b, band_t, off_b);
-#pragma unroll
-                for (int k = 0; k < K; ++k) off_b[k] = -off_b[k];
-            }
-            const bool cross_t = final_t > last_t, cross_b = final_b > last_b;
-            crossing = cross_t || cross_b;
-            if (cross_t) load_row<T, NT, K>(irows.row(min(h, last_t)), q1, e_t);
-            if (cross_b) load_row<T, NT, K>(irows.row(min(h, last_b)), q1, e_b);
+        for (int r = 0; r <= RB; ++r) {
+            rt[r] = clampi(i0 + r + s.xlo - 1, 0, h);
+            rb[r] = clampi(i0 + r + s.xhi, 0, h);
+            Tq[r] = load_row(rt[r]);
+            Bq[r] = load_row(rb[r]);
         }
-        if (!EARLY_ROWS) first_rows();
 
-        // All RB rows are always computed (rows past the image read clamped, valid rows and
-        // are not stored) and the prefetch of the next pair is decided at compile time:
-        // straight-line code, so loads stay in flight across the barrier.
+        T off_b[4] = {T(0), T(0), T(0), T(0)};
+        if (R > 0) {
+            const int band_t = max(rt[0] - 1, 0) / R, band_b = max(rb[0] - 1, 0) / R;
+            const int last_t = (band_t + 1) * R, last_b = (band_b + 1) * R;   // last row of each first band
+            if (band_t != band_b) {
+                double sum[4] = {0.0, 0.0, 0.0, 0.0};
+                for (int b = min(band_t, band_b); b < max(band_t, band_b); ++b) {
+                    const Quad<T> bottom = load_row(min(h, (b + 1) * R));
 #pragma unroll
-        for (int r = 0; r < RB; r += 2) {
-            const int i = i0 + r;
-            T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {};
-            const bool more = r + 2 < RB;                            // known after unrolling
-            if (more)
-                load_pair<T, NT, K, FULL>(irows, i + 2, s.xlo, s.xhi, h, q1, n0, n1, n2, n3);
-            RowPair<T>* V = vbuf + (((r >> 1) & 1) ? vlen : 0);
-            T v0[K], v1[K];
+                    for (int v = 0; v < 4; ++v) sum[v] += static_cast<double>(bottom.v[v]);
+                }
 #pragma unroll
-            for (int k = 0; k < K; ++k) {
-                v0[k] = blend<T, EXACT>(ta[k], t0[k], bc[k], b1[k], s.fxlo, s.fxhi);
-                v1[k] = blend<T, EXACT>(t0[k], t1[k], b1[k], b2[k], s.fxlo, s.fxhi);
-                if (OFFS) { v0[k] += off_b[k]; v1[k] += off_b[k]; }
+                for (int v = 0; v < 4; ++v) off_b[v] = static_cast<T>(band_b > band_t ? sum[v] : -sum[v]);
             }
-            if (OFFS && crossing) {                                  // uniform; one batch in four
-                // which of the pair's rows lie beyond their side's first band (scalars)
-                const T cA = T(clampi(i + s.xlo - 1, 0, h) > last_t), c0 = T(clampi(i + s.xlo, 0, h) > last_t),
-                        c1 = T(clampi(i + 1 + s.xlo, 0, h) > last_t);
-                const T dC = T(clampi(i + s.xhi, 0, h) > last_b), d1 = T(clampi(i + 1 + s.xhi, 0, h) > last_b),
-                        d2 = T(clampi(i + 2 + s.xhi, 0, h) > last_b);
-                // weights of E_b and E_t in blend(lo_adv, lo, hi, hi_adv)
-                const T fhi = EXACT ? s.fxhi : T(0), flo = EXACT ? s.fxlo : T(0);
-                const T wb0 = dC + fhi * (d1 - dC), wt0 = flo * (c0 - cA) - c0;
-                const T wb1 = d1 + fhi * (d2 - d1), wt1 = flo * (c1 - c0) - c1;
+            if (rt[RB] > last_t) {                   // the top run crosses into the next band
+                const Quad<T> e = load_row(min(h, last_t));
 #pragma unroll
-                for (int k = 0; k < K; ++k) {
-                    v0[k] += wb0 * e_b[k] + wt0 * e_t[k];
-                    v1[k] += wb1 * e_b[k] + wt1 * e_t[k];
+                for (int r = 0; r <= RB; ++r) {
+                    const T c = T(rt[r] > last_t);
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) Tq[r].v[v] += c * e.v[v];
                 }
             }
-            publish_rows<T, NT, K, FULL>(V, v0, v1, w, row_bytes, q1);
-            __syncthreads();
+            if (rb[RB] > last_b) {
+                const Quad<T> e = load_row(min(h, last_b));
 #pragma unroll
-            for (int k = 0; k < K; ++k) {
-                if (slot_valid<T, NT, FULL>(q1, k, row_bytes) && (FS == 1 || counts)) {
-                    const RowPair<T> o = sample_columns<T, EXACT>(V, lo[k], hi[k], s.fylo, s.fyhi);
-                    acc[r][k] += scale * o.r0;
-                    acc[r + 1][k] += scale * o.r1;
-                }
-            }
-            if (more) {
+                for (int r = 0; r <= RB; ++r) {
+                    const T c = T(rb[r] > last_b);
 #pragma unroll
-                for (int k = 0; k < K; ++k) {
-                    ta[k] = t1[k]; bc[k] = b2[k];
-                    t0[k] = n0[k]; t1[k] = n1[k]; b1[k] = n2[k]; b2[k] = n3[k];
+                    for (int v = 0; v < 4; ++v) Bq[r].v[v] += c * e.v[v];
                 }
             }
         }
+
+#pragma unroll
+        for (int r = 0; r < RB; ++r)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                T val = blend<T, EXACT>(Tq[r].v[v], Tq[r + 1].v[v], Bq[r].v[v], Bq[r + 1].v[v], s.fxlo, s.fxhi);
+                val += off_b[v];
+                acc[r][v] += scale * val;
+            }
     }
 
     if constexpr (FS > 1) {
-        // partial sums of waves 1..FS-1 go through LDS (the row buffers are done with) and are
-        // added by wave 0 in wave order
+        // partial sums of the sets 1..FS-1 go through LDS and are added by set 0 in set order
         T* part = reinterpret_cast<T*>(smem_raw);
-        __syncthreads();
         if (fgroup > 0) {
 #pragma unroll
             for (int r = 0; r < RB; ++r)
 #pragma unroll
-                for (int k = 0; k < K; ++k)
-                    part[(((fgroup - 1) * RB + r) * K + k) * NT + threadIdx.x] = acc[r][k];
+                for (int v = 0; v < 4; ++v)
+                    part[(((fgroup - 1) * RB + r) * 4 + v) * NTX + tid] = acc[r][v];
         }
         __syncthreads();
         if (fgroup > 0) return;
@@ -312,18 +261,28 @@ grad_input_rows_kernel(SampleArgs<T> a, FinalizeArgs<T> fin) {
 #pragma unroll
             for (int r = 0; r < RB; ++r)
 #pragma unroll
-                for (int k = 0; k < K; ++k)
-                    acc[r][k] += part[(((g - 1) * RB + r) * K + k) * NT + threadIdx.x];
+                for (int v = 0; v < 4; ++v)
+                    acc[r][v] += part[(((g - 1) * RB + r) * 4 + v) * NTX + tid];
     }
 
-    // column slot q = j + 1 lands on pixel j; rows past the image get size 0
-    const Rows<T, FULL> orows(a.dst + p * static_cast<int64_t>(h) * w - 1, w, w + 1, h);
+    if (!lane_in) return;
+    T* out = a.dst + p * static_cast<int64_t>(h) * w + c0;
+    const bool wide_store = a.vec_out != 0 && c0 + 4 <= w;
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
         const int i = i0 + r;
-        const RowRef ob = orows.row(min(i, h - 1), i < h);
+        if (i >= h) break;
+        T* orow = out + static_cast<int64_t>(i) * w;
+        if (wide_store) {
+            Quad<T> q;
 #pragma unroll
-        for (int k = 0; k < K; ++k) store_slot<T, NT, kCacheDefault>(acc[r][k], ob, q1, k);
+            for (int v = 0; v < 4; ++v) q.v[v] = acc[r][v];
+            *reinterpret_cast<Quad<T>*>(orow) = q;
+        } else {
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                if (c0 + v < w) orow[v] = acc[r][v];
+        }
     }
 }
 
@@ -366,32 +325,49 @@ __device__ __forceinline__ void block_accumulate5(const double (&v)[5], double* 
 //          dS/dymin = -sum_q V[q]*(gl - glA) - V[w]*g[w-ylo+1].
 // Column 0 of the integral image is zero, so clamping at the left edge needs no correction.
 //
-// (SCAN) the BAND-LOCAL integral image of grad_output: L[i+1][c+1] = sum of grad_output over rows
-// band_start..i and columns 0..c. Bands do not depend on each other, so nothing has to be known
-// about the rows above: the true integral is L plus the bottom rows of the bands above, which
-// the grad-input kernel adds when it loads a row. Lanes own K consecutive columns for this part
-// (read back from the LDS row) and store them as one run, so a wave writes 64*K contiguous
-// elements per row.
+// (SCAN) what the gradient w.r.t. the input needs from grad_output, the column workspace M:
+//   A(i)[c] = sum_j g(i)[j] * (weight of input column c in the box of output pixel j)
+//           = sum_{q > c} W[q] + tail            (the adjoint of the forward's column formula:
+//             the input row enters through its prefix X[q] = sum_{c < q} x[c], so the weight of
+//             x[c] is the sum of the W[q] of all prefixes that contain it; `tail` belongs to q = w),
+//   M[i+1][c] = sum of A(i')[c] over the rows i' <= i of this band          (band-local running sum)
+// with the same W[q] as above, so the four grad_output taps per column are shared with PARAMS.
+// W(i), W(i+1) go to LDS as a row pair, are read back K consecutive columns per lane, and
+// A = (sum of all W + tail) - (exclusive prefix of W) is a lane prefix, a DPP wave scan and the
+// totals of the waves to the left. Bands do not depend on each other, so nothing has to be known
+// about the rows above: the grad-input kernel adds the bottom rows of the bands above when it
+// loads a row. A lane stores its K consecutive columns as one run into 16-byte aligned rows
+// (pitch rounded up to 4 elements), so a wave writes 64*K contiguous elements per row.
+// The boxes behind W are those of the parameter-gradient split; the reference's grad-input
+// pass splits the mirrored box (src/box_convolution.cpp:51-67), whose whole-pixel part can
+// differ when x_min - 1 rounds in T (it is then one pixel off with a border weight that makes up
+// for it in exact mode only). A workgroup whose box is such a case computes a second set of
+// weights for M from the mirrored split.
 //
 // LDS: [2 buffers][K*nt + 8] RowPair grad_output rows (4 zero pairs in front, >= 4 behind),
-//      [2][2][4] X[w] triples, [K*nt] tail weights, [8*5] doubles, [2][8] wave totals.
+//      [2][2][4] X[w] triples, [K*nt] tail weights, [K*nt] RowPair W rows, [8*5] doubles,
+//      [2][8] wave totals, [2][8] wave tails.
 constexpr int kGPad = 4;
 
 template <class T>
 struct StreamLds {
     RowPair<T>* grow;   // [2][glen]
+    RowPair<T>* wrow;   // [K*nt] W(i), W(i+1) by pixel column
     T* xw;              // [2][2][4]
     T* delta;           // [K*nt] tail weight of pixel column j
     double* red;        // [5 * kMaxRowWaves]
     T* wave_tot;        // [2][kMaxRowWaves]
+    T* wave_tail;       // [2][kMaxRowWaves]
     int glen;
 };
 
-__host__ __device__ inline size_t stream_lds_bytes(int K, int nt, size_t elem) {
+__host__ __device__ inline size_t stream_lds_elems(int K, int nt) {
     const size_t glen = static_cast<size_t>(K) * nt + 8;
-    size_t b = (4 * glen + 16 + static_cast<size_t>(K) * nt) * elem;
-    b = (b + 15) / 16 * 16;
-    return b + (2 * kMaxRowWaves + 5 * kMaxRowWaves) * sizeof(double);
+    return 4 * glen + 2 * static_cast<size_t>(K) * nt + 16 + static_cast<size_t>(K) * nt;
+}
+__host__ __device__ inline size_t stream_lds_bytes(int K, int nt, size_t elem) {
+    const size_t b = (stream_lds_elems(K, nt) * elem + 15) / 16 * 16;
+    return b + (4 * kMaxRowWaves + 5 * kMaxRowWaves) * sizeof(double);
 }
 
 template <class T>
@@ -399,25 +375,16 @@ __device__ __forceinline__ StreamLds<T> carve_stream_lds(int K, int nt) {
     StreamLds<T> l;
     l.glen = K * nt + 8;
     l.grow = reinterpret_cast<RowPair<T>*>(smem_raw);
-    l.xw = reinterpret_cast<T*>(l.grow + 2 * l.glen);
+    l.wrow = l.grow + 2 * l.glen;
+    l.xw = reinterpret_cast<T*>(l.wrow + K * nt);
     l.delta = l.xw + 16;
-    size_t b = (4 * static_cast<size_t>(l.glen) + 16 + static_cast<size_t>(K) * nt) * sizeof(T);
-    b = (b + 15) / 16 * 16;
+    const size_t b = (stream_lds_elems(K, nt) * sizeof(T) + 15) / 16 * 16;
     l.red = reinterpret_cast<double*>(smem_raw + b);
     l.wave_tot = reinterpret_cast<T*>(l.red + 5 * kMaxRowWaves);
+    l.wave_tail = reinterpret_cast<T*>(l.red + 7 * kMaxRowWaves);
     return l;
 }
 
-template <class T, int WV>
-__device__ __forceinline__ void add_waves_left(const T* wave_tot, int wave, T& carry0, T& carry1) {
-    if constexpr (WV < kMaxRowWaves - 1) {
-        if (wave > WV) {
-            carry0 += wave_tot[WV];
-            carry1 += wave_tot[kMaxRowWaves + WV];
-            add_waves_left<T, WV + 1>(wave_tot, wave, carry0, carry1);
-        }
-    }
-}
 
 template <class T, int NT, int K, bool EXACT, bool FULL, bool PARAMS, bool SCAN>
 __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a) {
@@ -439,17 +406,18 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
     const BoxSplit<T> s = split_grad_params(bx.xmin, bx.xmax, bx.ymin, bx.ymax);
 
     const int64_t pitch = w + 1;
+    const int64_t mpitch = a.mpitch;
     // integral of the input; grad_output (one element early: column slot q = j + 1 is pixel j);
-    // band-local integral of grad_output
+    // column workspace M of this (plane, filter)
     const LoadRows<T> irows(a.src + p * static_cast<int64_t>(h + 1) * pitch, pitch, w + 1, h + 1);
     const LoadRows<T> grows(a.grad_out + pf * static_cast<int64_t>(h) * w - 1, w, w + 1, h);
-    T* lrows = SCAN ? a.dst + pf * static_cast<int64_t>(h + 1) * pitch : nullptr;
+    T* mrows = SCAN ? a.dst + pf * static_cast<int64_t>(h + 1) * mpitch : nullptr;
     // The bands an XCD writes last (the final keep_tail bytes of its range) are stored with the
     // ordinary cache policy, everything before them non-temporally: see the store below.
     const unsigned from_end = static_cast<unsigned>(a.per_xcd) - 1u - vid % static_cast<unsigned>(a.per_xcd);
     const bool keep_in_cache =
-        static_cast<uint64_t>(from_end) * a.R * pitch * sizeof(T) < static_cast<uint64_t>(a.keep_tail);
-    const Rows<T, FULL> lout(lrows, pitch, w + 1, h + 1);
+        static_cast<uint64_t>(from_end) * a.R * mpitch * sizeof(T) < static_cast<uint64_t>(a.keep_tail);
+    const Rows<T, FULL> mout(mrows, mpitch, static_cast<int>(mpitch), h + 1);
     const StreamLds<T> lds = carve_stream_lds<T>(K, nt);
     const int glen = lds.glen;
 
@@ -469,37 +437,57 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
     load_g(i0, g0);
     load_g(i0 + 1, g1);
 
-    // clear the grad_output rows once: pads and the columns beyond w stay zero for good
+    // clear the grad_output rows once: pads and the columns beyond w stay zero for good; the
+    // same for the W rows
     for (int e = tid; e < 2 * glen; e += nt) lds.grow[e] = RowPair<T>{T(0), T(0)};
-    if (SCAN && band == 0)
-        for (int c = tid; c <= w; c += nt) lrows[c] = T(0);                    // integral row 0
+    if (SCAN) {
+        for (int e = tid; e < K * nt; e += nt) lds.wrow[e] = RowPair<T>{T(0), T(0)};
+        if (band == 0)
+            for (int c = tid; c < mpitch; c += nt) mrows[c] = T(0);            // row 0
+    }
     __syncthreads();
 
-    // lane-constant LDS byte offsets of the pairs (grA, gr) and (gl, glA); the tail weights of the
-    // lane's columns go to LDS (read back once per row pair: cheaper than K live registers)
+    // tail weight of pixel column j for a box with these column offsets and border weights
+    auto tail_weight = [&](int j, int ylo, int yhi, T fylo, T fyhi) {
+        const T one = T(1);
+        return (EXACT ? (one - fyhi) : one) * T(j > w - yhi)
+             + (EXACT ? fyhi : T(0)) * T(j > w - yhi - 1)
+             - (EXACT ? (one - fylo) : one) * T(j > w - ylo)
+             - (EXACT ? fylo : T(0)) * T(j > w - ylo + 1);
+    };
+    // LDS byte offsets of the pairs (grA, gr) and (gl, glA) of column slot q
+    auto tap_r = [&](int q, int yhi) {
+        return static_cast<unsigned>(clampi(q - yhi - 1, -2, w) + kGPad) * static_cast<unsigned>(sizeof(RowPair<T>));
+    };
+    auto tap_l = [&](int q, int ylo) {
+        return static_cast<unsigned>(clampi(q - ylo, -2, w) + kGPad) * static_cast<unsigned>(sizeof(RowPair<T>));
+    };
+
+    // lane-constant tap offsets; the tail weights of the lane's columns go to LDS (read back
+    // once per row pair: cheaper than K live registers)
     unsigned ir[K], il[K];
     unsigned idx_ymax = 0, idx_ymin = 0;
-    if (PARAMS) {
+    bool wave_has_tail = false;
 #pragma unroll
-        for (int k = 0; k < K; ++k) {
-            const int j = tid + nt * k;
-            const int q = j + 1;
-            ir[k] = static_cast<unsigned>(clampi(q - s.yhi - 1, -2, w) + kGPad) * static_cast<unsigned>(sizeof(RowPair<T>));
-            il[k] = static_cast<unsigned>(clampi(q - s.ylo, -2, w) + kGPad) * static_cast<unsigned>(sizeof(RowPair<T>));
-            T d = T(0);
-            if (FULL || j < w) {
-                const T one = T(1);
-                d = (EXACT ? (one - s.fyhi) : one) * T(j > w - s.yhi)
-                  + (EXACT ? s.fyhi : T(0)) * T(j > w - s.yhi - 1)
-                  - (EXACT ? (one - s.fylo) : one) * T(j > w - s.ylo)
-                  - (EXACT ? s.fylo : T(0)) * T(j > w - s.ylo + 1);
-            }
-            lds.delta[j] = d;
-        }
+    for (int k = 0; k < K; ++k) {
+        const int j = tid + nt * k;
+        ir[k] = tap_r(j + 1, s.yhi);
+        il[k] = tap_l(j + 1, s.ylo);
+        const T d = (FULL || j < w) ? tail_weight(j, s.ylo, s.yhi, s.fylo, s.fyhi) : T(0);
+        lds.delta[j] = d;
+        wave_has_tail = wave_has_tail || d != T(0);
+    }
+    if (PARAMS) {
         const int j_ymax = w - s.yhi, j_ymin = w - s.ylo + 1;
         idx_ymax = (j_ymax >= 0 && j_ymax < w) ? j_ymax + kGPad : 0;          // index 0 holds a zero
         idx_ymin = (j_ymin >= 0 && j_ymin < w) ? j_ymin + kGPad : 0;
     }
+    // SCAN: the whole-pixel column offsets of the reference's mirrored split, turned back to the
+    // orientation of W; they differ from s.ylo / s.yhi only when y_min - 1 rounds in T
+    const BoxSplit<T> sm = split_grad_input(bx.xmin, bx.xmax, bx.ymin, bx.ymax);
+    const int ylo_m = 1 - sm.yhi, yhi_m = 1 - sm.ylo;
+    const bool own_w = SCAN && (ylo_m != s.ylo || yhi_m != s.yhi);               // workgroup-uniform
+    wave_has_tail = __any(wave_has_tail) != 0 || own_w;                          // wave-uniform
 
     // The five sums are added up in T only within one row pair of one lane (2*K products each);
     // from there on in double. The products are large against the final sums (V grows along the
@@ -541,7 +529,7 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
         for (int k = 0; k < K; ++k) {
             if (slot_valid<T, NT, FULL>(q1, k, row_bytes))
                 *at_bytes(G + kGPad - 1 + NT * k, 2 * q1) = RowPair<T>{g0[k], g1[k]};
-            if (PARAMS) {
+            {
                 const T dlt = *at_bytes(lds.delta - 1 + NT * k, q1);
                 tail0 += dlt * g0[k];
                 tail1 += dlt * g1[k];
@@ -560,109 +548,152 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
         }
         __syncthreads();                                                     // rows are in LDS
 
-        if (PARAMS) {
+        // W(i)[q], W(i+1)[q] of the lane's column slots
+        T wq0[K], wq1[K];
+        {
             T sum[5] = {T(0), T(0), T(0), T(0), T(0)};
 #pragma unroll
             for (int k = 0; k < K; ++k) {
-                const T dt0 = t0[k] - ta[k], db0 = b1[k] - bc[k];
-                const T dt1 = t1[k] - t0[k], db1 = b2[k] - b1[k];
-                T v0 = bc[k] - t0[k], v1 = b1[k] - t1[k];
-                if (EXACT) {
-                    v0 += s.fxhi * db0; v0 += s.fxlo * dt0;
-                    v1 += s.fxhi * db1; v1 += s.fxlo * dt1;
-                }
                 const RowPair<T>* R = at_bytes(G, ir[k]);
                 const RowPair<T>* L = at_bytes(G, il[k]);
                 const RowPair<T> grA = R[0], gr = R[1], gl = L[0], glA = L[1];
-                {
-                    const T dr = grA.r0 - gr.r0, dl = gl.r0 - glA.r0;
-                    T wq = gr.r0 - gl.r0;
-                    if (EXACT) { wq += s.fyhi * dr; wq += s.fylo * dl; }
-                    sum[4] += v0 * wq;
-                    sum[1] += db0 * wq;
-                    sum[0] -= dt0 * wq;
-                    sum[3] += v0 * dr;
-                    sum[2] -= v0 * dl;
+                const T dr0 = grA.r0 - gr.r0, dl0 = gl.r0 - glA.r0;
+                const T dr1 = grA.r1 - gr.r1, dl1 = gl.r1 - glA.r1;
+                wq0[k] = gr.r0 - gl.r0;
+                wq1[k] = gr.r1 - gl.r1;
+                if (EXACT) {
+                    wq0[k] += s.fyhi * dr0; wq0[k] += s.fylo * dl0;
+                    wq1[k] += s.fyhi * dr1; wq1[k] += s.fylo * dl1;
                 }
-                {
-                    const T dr = grA.r1 - gr.r1, dl = gl.r1 - glA.r1;
-                    T wq = gr.r1 - gl.r1;
-                    if (EXACT) { wq += s.fyhi * dr; wq += s.fylo * dl; }
-                    sum[4] += v1 * wq;
-                    sum[1] += db1 * wq;
-                    sum[0] -= dt1 * wq;
-                    sum[3] += v1 * dr;
-                    sum[2] -= v1 * dl;
+                if (PARAMS) {
+                    const T dt0 = t0[k] - ta[k], db0 = b1[k] - bc[k];
+                    const T dt1 = t1[k] - t0[k], db1 = b2[k] - b1[k];
+                    T v0 = bc[k] - t0[k], v1 = b1[k] - t1[k];
+                    if (EXACT) {
+                        v0 += s.fxhi * db0; v0 += s.fxlo * dt0;
+                        v1 += s.fxhi * db1; v1 += s.fxlo * dt1;
+                    }
+                    sum[4] += v0 * wq0[k];
+                    sum[1] += db0 * wq0[k];
+                    sum[0] -= dt0 * wq0[k];
+                    sum[3] += v0 * dr0;
+                    sum[2] -= v0 * dl0;
+                    sum[4] += v1 * wq1[k];
+                    sum[1] += db1 * wq1[k];
+                    sum[0] -= dt1 * wq1[k];
+                    sum[3] += v1 * dr1;
+                    sum[2] -= v1 * dl1;
                 }
             }
-            const T vw0 = X0[0], dtw0 = X0[1], dbw0 = X0[2];
-            const T vw1 = X1[0], dtw1 = X1[1], dbw1 = X1[2];
-            sum[4] += vw0 * tail0 + vw1 * tail1;
-            sum[1] += dbw0 * tail0 + dbw1 * tail1;
-            sum[0] -= dtw0 * tail0 + dtw1 * tail1;
-            if (tid == 0) {
-                const RowPair<T> gmax = G[idx_ymax], gmin = G[idx_ymin];
-                sum[3] += vw0 * gmax.r0 + vw1 * gmax.r1;
-                sum[2] -= vw0 * gmin.r0 + vw1 * gmin.r1;
-            }
+            if (PARAMS) {
+                const T vw0 = X0[0], dtw0 = X0[1], dbw0 = X0[2];
+                const T vw1 = X1[0], dtw1 = X1[1], dbw1 = X1[2];
+                sum[4] += vw0 * tail0 + vw1 * tail1;
+                sum[1] += dbw0 * tail0 + dbw1 * tail1;
+                sum[0] -= dtw0 * tail0 + dtw1 * tail1;
+                if (tid == 0) {
+                    const RowPair<T> gmax = G[idx_ymax], gmin = G[idx_ymin];
+                    sum[3] += vw0 * gmax.r0 + vw1 * gmax.r1;
+                    sum[2] -= vw0 * gmin.r0 + vw1 * gmin.r1;
+                }
 #pragma unroll
-            for (int n = 0; n < 5; ++n) total[n] += static_cast<double>(sum[n]);
+                for (int n = 0; n < 5; ++n) total[n] += static_cast<double>(sum[n]);
+            }
         }
 
         if (SCAN) {
-            // lane owns columns K*tid .. K*tid+K-1; two rows of the band-local integral. A band
-            // restarts at zero and the row prefix is a tree (inside the lane, across the wave,
-            // across waves), so plain T arithmetic loses a few ulps of the band-local value only.
-            T loc0[K], loc1[K];
-            T carry0, carry1;
+            if (own_w) {
+                // rare: the mirrored split cuts the box at other whole pixels; weights and tails
+                // of M from that split, tap offsets worked out on the spot
+                tail0 = T(0); tail1 = T(0);
+#pragma unroll
+                for (int k = 0; k < K; ++k) {
+                    const int j = tid + nt * k;
+                    const RowPair<T>* R = at_bytes(G, tap_r(j + 1, yhi_m));
+                    const RowPair<T>* L = at_bytes(G, tap_l(j + 1, ylo_m));
+                    const RowPair<T> grA = R[0], gr = R[1], gl = L[0], glA = L[1];
+                    wq0[k] = gr.r0 - gl.r0;
+                    wq1[k] = gr.r1 - gl.r1;
+                    if (EXACT) {
+                        wq0[k] += sm.fylo * (grA.r0 - gr.r0); wq0[k] += sm.fyhi * (gl.r0 - glA.r0);
+                        wq1[k] += sm.fylo * (grA.r1 - gr.r1); wq1[k] += sm.fyhi * (gl.r1 - glA.r1);
+                    }
+                    const T dlt = (FULL || j < w) ? tail_weight(j, ylo_m, yhi_m, sm.fyhi, sm.fylo) : T(0);
+                    tail0 += dlt * g0[k];
+                    tail1 += dlt * g1[k];
+                }
+            }
+            // W rows by pixel column c = q - 1, and the wave's share of the tails
+#pragma unroll
+            for (int k = 0; k < K; ++k)
+                if (slot_valid<T, NT, FULL>(q1, k, row_bytes))
+                    *at_bytes(lds.wrow - 1 + NT * k, 2 * q1) = RowPair<T>{wq0[k], wq1[k]};
+            T wt0 = T(0), wt1 = T(0);
+            if (wave_has_tail) {
+                wt0 = wave_sum_to_last(tail0);
+                wt1 = wave_sum_to_last(tail1);
+            }
+            if (lane == 63) { lds.wave_tail[wave] = wt0; lds.wave_tail[kMaxRowWaves + wave] = wt1; }
+            __syncthreads();                                                 // W rows are in LDS
+
+            // the lane's K consecutive columns K*tid .. K*tid+K-1: exclusive prefix of W inside
+            // the lane, the lanes to the left by a wave scan
+            T ex0[K], ex1[K];
+            T base0, base1;
             {
-                const RowPair<T>* r = G + kGPad + K * tid;
+                const RowPair<T>* r = lds.wrow + K * tid;
                 T run0 = T(0), run1 = T(0);
 #pragma unroll
                 for (int k = 0; k < K; ++k) {
-                    const RowPair<T> g = r[k];
-                    colacc[k] += g.r0;
-                    run0 += colacc[k];
-                    loc0[k] = run0;
-                    colacc[k] += g.r1;
-                    run1 += colacc[k];
-                    loc1[k] = run1;
+                    const RowPair<T> wv = r[k];
+                    ex0[k] = run0; run0 += wv.r0;
+                    ex1[k] = run1; run1 += wv.r1;
                 }
                 const T inc0 = wave_inclusive_scan(run0);
                 const T inc1 = wave_inclusive_scan(run1);
-                carry0 = inc0 - run0;
-                carry1 = inc1 - run1;
+                base0 = run0 - inc0;                                         // -(lanes to the left)
+                base1 = run1 - inc1;
                 if (lane == 63) { lds.wave_tot[wave] = inc0; lds.wave_tot[kMaxRowWaves + wave] = inc1; }
             }
             __syncthreads();                                                 // wave totals visible
             {
-                // totals of the waves to the left; `wave` is scalar, so these are scalar branches
-                // and wave n takes n + 1 of them
-                add_waves_left<T, 0>(lds.wave_tot, wave, carry0, carry1);
-                // the lane's K consecutive columns K*tid+1 .. K*tid+K of integral rows i+1, i+2:
-                // a wave stores one contiguous run of 64*K elements per row. The grad-input
-                // kernel starts with the planes written last and finds them still in the
-                // memory-side cache if they were stored with the ordinary policy; the rest is
-                // stored non-temporally so that it does not push the integral plane of the
+                // A[c] = (sum of all W + tail) - (W of the columns before c)
+                //      = totals of this wave and the waves to the right + all tails - lanes to
+                //        the left - columns to the left inside the lane.
+                // `wave` is scalar, so the conditions below are scalar.
+#pragma unroll
+                for (int wv = 0; wv < NT / 64; ++wv) {
+                    base0 += lds.wave_tail[wv];
+                    base1 += lds.wave_tail[kMaxRowWaves + wv];
+                    if (wv >= wave) {
+                        base0 += lds.wave_tot[wv];
+                        base1 += lds.wave_tot[kMaxRowWaves + wv];
+                    }
+                }
+                // M rows i+1, i+2: a wave stores one contiguous run of 64*K elements per row. The
+                // grad-input kernel starts with the planes written last and finds them still in
+                // the memory-side cache if they were stored with the ordinary policy; the rest
+                // is stored non-temporally so that it does not push the integral plane of the
                 // input, which all filters of a plane re-read, out of the L2.
-                T* o0 = lrows + static_cast<int64_t>(i + 1) * pitch;
                 const bool second = i + 1 < i1;
-                const RowRef ob0 = lout.row(i + 1);
-                const RowRef ob1 = lout.row(min(i + 2, h), second);
+                const RowRef ob0 = mout.row(i + 1);
+                const RowRef ob1 = mout.row(min(i + 2, h), second);
                 T out0[K], out1[K];
 #pragma unroll
-                for (int k = 0; k < K; ++k) { out0[k] = carry0 + loc0[k]; out1[k] = carry1 + loc1[k]; }
-                const int first = (1 + K * tid) * static_cast<int>(sizeof(T));
-                if (keep_in_cache) {
-                    buffer_store_run<kCacheDefault, FULL>(out0, ob0, first, static_cast<int>(row_bytes + sizeof(T)));
-                    buffer_store_run<kCacheDefault, FULL>(out1, ob1, first, static_cast<int>(row_bytes + sizeof(T)));
-                } else {
-                    buffer_store_run<kCacheStream, FULL>(out0, ob0, first, static_cast<int>(row_bytes + sizeof(T)));
-                    buffer_store_run<kCacheStream, FULL>(out1, ob1, first, static_cast<int>(row_bytes + sizeof(T)));
+                for (int k = 0; k < K; ++k) {
+                    colacc[k] += base0 - ex0[k];
+                    out0[k] = colacc[k];
+                    colacc[k] += base1 - ex1[k];
+                    out1[k] = colacc[k];
                 }
-                if (tid == 0) {
-                    o0[0] = T(0);
-                    if (second) o0[pitch] = T(0);
+                const int first = K * tid * static_cast<int>(sizeof(T));
+                const int limit = static_cast<int>(mpitch * sizeof(T));
+                if (keep_in_cache) {
+                    buffer_store_run<kCacheDefault, FULL>(out0, ob0, first, limit);
+                    buffer_store_run<kCacheDefault, FULL>(out1, ob1, first, limit);
+                } else {
+                    buffer_store_run<kCacheStream, FULL>(out0, ob0, first, limit);
+                    buffer_store_run<kCacheStream, FULL>(out1, ob1, first, limit);
                 }
             }
         }
@@ -780,11 +811,38 @@ FinalizeArgs<T> finalize_args(const ParamFinish<T>& f) {
     return fa;
 }
 
-// BOXCONV_GI_SPLIT_FILTERS=0 keeps the workgroups of narrow images at one row's width (for
-// comparison; read at every call, so that a test can switch it within one process).
+// BOXCONV_GI_SPLIT_FILTERS=0: every workgroup of the grad-input kernel walks through all
+// filters itself (for comparison; read at every call, so that a test can switch it within one
+// process).
 inline bool split_filters_enabled() {
     const char* e = std::getenv("BOXCONV_GI_SPLIT_FILTERS");
     return e == nullptr || std::atoi(e) != 0;
+}
+
+// Shape of the grad-input launch for an image of h x w with F filters per plane: 2^lq lanes
+// (4 columns each) side by side, rb output rows per lane, fs sets of threads sharing the filters.
+struct ColsConfig { int lq, rb, fs; };
+inline ColsConfig cols_config(int64_t planes, int F, int h, int w, bool allow_split) {
+    ColsConfig c;
+    const int quads = (w + 3) / 4;
+    c.lq = 3;
+    while (c.lq < 8 && (1 << c.lq) < quads) ++c.lq;          // 8 .. 256 lanes per row group
+    c.rb = 8;
+    c.fs = 1;
+    // Small problems: more, shorter-lived waves (2 rows per lane), and the filters of a plane
+    // spread over several sets of threads. "Small": fewer waves than the chip holds at once.
+    auto waves = [&](int rb) {
+        const int ntx = std::max(64, 1 << c.lq), rg = ntx >> c.lq;
+        const int64_t strips = (w + (4 << c.lq) - 1) / (4 << c.lq);
+        return planes * ((h + rb * rg - 1) / (rb * rg)) * strips * (ntx / 64);
+    };
+    if (waves(8) < 2048) c.rb = 2;
+    if (allow_split && F >= 4 && c.rb == 2 && waves(c.rb) <= 4096 && c.lq <= 6) {
+        c.fs = F >= 16 ? 8 : 4;
+        while (c.fs > 1 && waves(c.rb) * c.fs > 16384) c.fs /= 2;
+        if (c.fs == 2) c.fs = 1;
+    }
+    return c;
 }
 
 template <class T>
@@ -796,10 +854,9 @@ hipError_t grad_input_launch(const T* gint, int band_rows, BoxParams<T> prm, T* 
     SampleArgs<T> a = base_args(prm, d);
     a.src = gint; a.dst = grad_in; a.normalize = normalize ? 1 : 0;
     a.off_R = band_rows;
-    a.reverse = (band_rows > 0 && reverse_grad_input()) ? 1 : 0;
 
-    if (!row_kernels_apply(d.h, d.w, sizeof(T))) {
-        if (band_rows > 0) return hipErrorInvalidValue;         // the gather kernel needs a true integral
+    if (band_rows == 0) {
+        // true integral images: one thread per pixel (any width)
         finish_args(a, d.planes * d.hw());
         const dim3 grid(static_cast<unsigned>((a.total + 255) / 256));
         if (exact) BOXCONV_LAUNCH("grad_input_gather", (grad_input_gather_kernel<T, true>), grid, dim3(256), 0, stream, a);
@@ -807,46 +864,51 @@ hipError_t grad_input_launch(const T* gint, int band_rows, BoxParams<T> prm, T* 
         return hipGetLastError();
     }
 
-    constexpr int RB = 8;
-    static const int gi_threads = preferred_row_threads("BOXCONV_GI_THREADS", 512);
-    const RowConfig rc = row_config(d.w, gi_threads);
-    a.nb = (d.h + RB - 1) / RB;
-    a.R = RB;
-    finish_args(a, d.planes * a.nb);
+    a.reverse = reverse_grad_input() ? 1 : 0;
+    a.mpitch = column_workspace_pitch(d.w);
+    a.vec_out = (d.w % 4 == 0 && reinterpret_cast<uintptr_t>(grad_in) % (4 * sizeof(T)) == 0) ? 1 : 0;
+    const ColsConfig cc = cols_config(d.planes, d.F, d.h, d.w, split_filters_enabled());
+    const int ntx = std::max(64, 1 << cc.lq), rg = ntx >> cc.lq;
+    const int64_t strips = (d.w + (4 << cc.lq) - 1) / (4 << cc.lq);
+    a.nb = (d.h + cc.rb * rg - 1) / (cc.rb * rg);
+    a.R = cc.rb;
+    if (band_rows < cc.rb + 1 && band_rows < d.h) return hipErrorInvalidValue;   // a run may cross one band edge only
+    finish_args(a, d.planes * a.nb * strips);
     const dim3 grid(static_cast<unsigned>(a.per_xcd * kXcds));
-    const size_t lds = 4 * static_cast<size_t>(d.w + 3) * sizeof(T);
-    // One column per lane on a problem too small to fill the chip: the workgroup is widened to
-    // 512 (one or two waves per row) or 1024 threads (four waves per row) and its waves share the
-    // filters (see the kernel).
-    const int waves_per_row = rc.nt / 64;
-    const bool split_filters = rc.K == 1 && rc.nt <= 256 && d.F >= 4 &&
-                               a.total * waves_per_row <= 4096 && split_filters_enabled();
-    const int fs = rc.nt == 64 ? 8 : 4;
-    const size_t lds_split = std::max(lds * fs, static_cast<size_t>(fs - 1) * RB * rc.nt * sizeof(T));
+    const size_t lds = cc.fs > 1 ? static_cast<size_t>(cc.fs - 1) * cc.rb * 4 * ntx * sizeof(T) : 0;
     FinalizeArgs<T> fin{};
     if (finish != nullptr && finish->acc != nullptr && grid.x >= static_cast<unsigned>(finish->n_boxes)) {
         fin = finalize_args(*finish);
         if (finish_done != nullptr) *finish_done = true;
     }
-#define LAUNCH_GI(NT, KK, EX, FU) \
-    if (band_rows > 0) BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, NT, KK, RB, EX, FU, true>), grid, dim3(NT), lds, stream, a, fin); \
-    else BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, NT, KK, RB, EX, FU, false>), grid, dim3(NT), lds, stream, a, fin)
-#define LAUNCH_GI_SPLIT(NT, FS, EX, FU) \
-    if (band_rows > 0) BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, NT, 1, RB, EX, FU, true, FS>), grid, dim3(NT, FS), lds_split, stream, a, fin); \
-    else BOXCONV_LAUNCH("grad_input_rows", (grad_input_rows_kernel<T, NT, 1, RB, EX, FU, false, FS>), grid, dim3(NT, FS), lds_split, stream, a, fin)
-#define LAUNCH_GI_SPLIT_SHAPE(EX, FU) \
-    if (rc.nt == 64) { LAUNCH_GI_SPLIT(64, 8, EX, FU); } \
-    else if (rc.nt == 128) { LAUNCH_GI_SPLIT(128, 4, EX, FU); } \
-    else { LAUNCH_GI_SPLIT(256, 4, EX, FU); }
-    if (split_filters) {
-        if (exact) { if (rc.full) { LAUNCH_GI_SPLIT_SHAPE(true, true) } else { LAUNCH_GI_SPLIT_SHAPE(true, false) } }
-        else       { if (rc.full) { LAUNCH_GI_SPLIT_SHAPE(false, true) } else { LAUNCH_GI_SPLIT_SHAPE(false, false) } }
-    } else {
-        BOXCONV_DISPATCH_SHAPE_EXACT_FULL(LAUNCH_GI, rc, exact)
+#define LAUNCH_GC(LQ, RB, FS)                                                                          \
+    do {                                                                                               \
+        constexpr int NTX_ = (LQ) > 6 ? (1 << (LQ)) : 64;                                              \
+        if (exact) BOXCONV_LAUNCH("grad_input_cols", (grad_input_cols_kernel<T, LQ, RB, true, FS>), grid, dim3(NTX_, FS), lds, stream, a, fin); \
+        else       BOXCONV_LAUNCH("grad_input_cols", (grad_input_cols_kernel<T, LQ, RB, false, FS>), grid, dim3(NTX_, FS), lds, stream, a, fin); \
+    } while (0)
+#define LAUNCH_GC_FS(LQ, RB)                                                                           \
+    do {                                                                                               \
+        if (cc.fs == 8) LAUNCH_GC(LQ, RB, 8);                                                          \
+        else if (cc.fs == 4) LAUNCH_GC(LQ, RB, 4);                                                     \
+        else LAUNCH_GC(LQ, RB, 1);                                                                     \
+    } while (0)
+#define LAUNCH_GC_RB(LQ)                                                                               \
+    do {                                                                                               \
+        if (cc.rb == 2) LAUNCH_GC_FS(LQ, 2);                                                           \
+        else LAUNCH_GC(LQ, 8, 1);                                                                      \
+    } while (0)
+    switch (cc.lq) {
+        case 3: LAUNCH_GC_RB(3); break;
+        case 4: LAUNCH_GC_RB(4); break;
+        case 5: LAUNCH_GC_RB(5); break;
+        case 6: LAUNCH_GC_RB(6); break;
+        case 7: if (cc.rb == 2) LAUNCH_GC(7, 2, 1); else LAUNCH_GC(7, 8, 1); break;
+        default: if (cc.rb == 2) LAUNCH_GC(8, 2, 1); else LAUNCH_GC(8, 8, 1); break;
     }
-#undef LAUNCH_GI_SPLIT_SHAPE
-#undef LAUNCH_GI_SPLIT
-#undef LAUNCH_GI
+#undef LAUNCH_GC_RB
+#undef LAUNCH_GC_FS
+#undef LAUNCH_GC
     return hipGetLastError();
 }
 
@@ -882,14 +944,15 @@ inline int64_t cached_tail_bytes() {
 
 template <class T>
 hipError_t grad_output_stream_launch(const T* integ, const T* grad_out, BoxParams<T> prm,
-                                     double* acc, int acc_slots, T* local_integral,
+                                     double* acc, int acc_slots, T* column_workspace,
                                      const StreamPlan& sp, Dims d, bool exact, hipStream_t stream) {
     const int64_t planes_f = d.planes * d.F;
     if (planes_f == 0 || d.hw() == 0) return hipSuccess;
-    const bool params = acc != nullptr, scan = local_integral != nullptr;
+    const bool params = acc != nullptr, scan = column_workspace != nullptr;
     if (!sp.usable || (!params && !scan)) return hipErrorInvalidValue;
     SampleArgs<T> a = base_args(prm, d);
-    a.src = integ; a.grad_out = grad_out; a.acc = acc; a.acc_slots = acc_slots; a.dst = local_integral;
+    a.src = integ; a.grad_out = grad_out; a.acc = acc; a.acc_slots = acc_slots; a.dst = column_workspace;
+    a.mpitch = column_workspace_pitch(d.w);
     if (acc_slots != 0 && acc_slots != sp.nb) return hipErrorInvalidValue;
     a.nb = sp.nb; a.R = sp.R;
     a.keep_tail = scan ? cached_tail_bytes() / kXcds : 0;

@@ -27,11 +27,13 @@ template <class T>
 struct SampleArgs {
     const T* src;         // integral planes, (h+1) x (w+1) each, contiguous
     BoxParams<T> prm;
-    T* dst;               // forward: [planes,F,h,w]; grad input: [planes,h,w]
+    T* dst;               // forward: [planes,F,h,w]; grad input: [planes,h,w]; grad_output pass: M
     const T* grad_out;    // param grads only: [planes,F,h,w]
     double* acc;          // param grads only: [C*F*5], or [planes*F*acc_slots*5] workgroup slots
     int acc_slots;        // param grads only: slots per (plane, filter), 0 = atomics on [C*F*5]
-    int off_R;                // grad input only: rows per band of a band-local integral, 0 = true integral
+    int off_R;            // grad input only: rows per band of the column workspace M (each band restarts at zero)
+    int64_t mpitch;       // elements between rows of M (a multiple of 4)
+    int vec_out;          // grad input only: rows of dst are 16-byte aligned
     int C, F, h, w;
     int nb, R;            // bands per plane and rows per band
     int64_t plane0;       // global index of the first plane (selects the boxes)

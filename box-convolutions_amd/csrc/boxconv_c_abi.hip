@@ -109,7 +109,8 @@ bool reverse_second_pass() {
 }
 
 // Workspace of the backward pass:
-//   [integral of grad_output: chunk*F planes of (h+1)(w+1)]   only if grad_input is wanted
+//   [column workspace M of grad_output: chunk*F planes of (h+1) rows, or their integral images
+//    of (h+1)(w+1) where the streaming pass does not apply]     only if grad_input is wanted
 //   [aux doubles: band column sums, three-pass fallback only]
 //   [acc: C*F*5 doubles, times batch*bands when every streaming workgroup has its own slot]
 //                                                              only if parameter gradients are wanted
@@ -137,8 +138,12 @@ BackwardLayout backward_layout(int batch, int in_planes, int num_filters, int h,
     L.gint_off = off;
     L.aux_off = off;
     if (need_input) {
+        // streaming: the column workspace M; else true integral images of (h+1) x (w+1)
+        const size_t per_plane = L.streaming
+            ? static_cast<size_t>(boxconv::column_workspace_plane(h, w))
+            : static_cast<size_t>(h + 1) * (w + 1);
         off += align_up(static_cast<size_t>(std::min(L.chunk, std::max<int64_t>(planes, 1))) *
-                        num_filters * (h + 1) * (w + 1) * elem_size, 256);
+                        num_filters * per_plane * elem_size, 256);
         L.aux_off = off;
         const int64_t aux = max_over_chunks(std::max<int64_t>(planes, 1), L.chunk, [&](int64_t np) {
             return L.streaming ? int64_t(0)

@@ -256,6 +256,15 @@ __device__ __forceinline__ void buffer_store(bf16_t v, const RowRef& r, int off)
 // dword alignment suffices); the at most one lane per row whose run straddles the end goes
 // element by element, each store checked against the row size. WHOLE: every lane's run lies
 // inside the row, nothing to test.
+//
+// A buffer store of more than 8 bytes per lane reads its data registers over several cycles
+// after issue. The compiler keeps the next write to those registers one wait state away only
+// when the store has no scalar offset register; with one (the stacked descriptors of `Rows` above) it
+// assumes no hazard, and a conversion to double placed right behind such a store was observed
+// to replace the first two dwords of the data in the lanes the store reads last. Two wait
+// states behind every wide store rule that out at a cost of two cycles.
+__device__ __forceinline__ void settle_wide_store() { asm volatile("s_nop 1"); }
+
 template <int POLICY, int K>
 __device__ __forceinline__ void buffer_store_wide(const float (&v)[K], const RowRef& r, int off) {
     typedef unsigned v4u __attribute__((__vector_size__(16)));
@@ -268,10 +277,12 @@ __device__ __forceinline__ void buffer_store_wide(const float (&v)[K], const Row
                               __builtin_bit_cast(unsigned, v[k + 2]), __builtin_bit_cast(unsigned, v[k + 3])};
             __builtin_amdgcn_raw_buffer_store_b128(pack, r.rs, off + 4 * k, r.soff, POLICY);
         }
+        settle_wide_store();
     } else if constexpr (K == 3) {
         const v3u pack = {__builtin_bit_cast(unsigned, v[0]), __builtin_bit_cast(unsigned, v[1]),
                           __builtin_bit_cast(unsigned, v[2])};
         __builtin_amdgcn_raw_buffer_store_b96(pack, r.rs, off, r.soff, POLICY);
+        settle_wide_store();
     } else if constexpr (K == 2) {
         const v2u pack = {__builtin_bit_cast(unsigned, v[0]), __builtin_bit_cast(unsigned, v[1])};
         __builtin_amdgcn_raw_buffer_store_b64(pack, r.rs, off, r.soff, POLICY);

@@ -79,8 +79,16 @@ struct ParamFinish {
     bool normalize, exact;
 };
 
-// band_rows: 0 when `gint` holds true integral images; otherwise `gint` holds band-local
-// integrals (each band of band_rows rows restarts at zero).
+// The column workspace M of the backward pass (written by grad_output_stream_launch, read by
+// grad_input_launch): per (plane, filter) h+1 rows of column_workspace_pitch(w) elements, so
+// that every row starts 16-byte aligned.
+inline int64_t column_workspace_pitch(int w) { return (static_cast<int64_t>(w) + 3) / 4 * 4; }
+inline int64_t column_workspace_plane(int h, int w) {
+    return (static_cast<int64_t>(h) + 1) * column_workspace_pitch(w);
+}
+
+// band_rows: 0 when `gint` holds true integral images, (h+1) x (w+1) per (plane, filter);
+// otherwise `gint` is the column workspace M in bands of band_rows rows, each restarting at zero.
 // finish (may be null): parameter-gradient sums that are complete when this launch starts; the
 // row kernel then finishes them on the side (no launch of its own) and *finish_done is set.
 template <class T>
@@ -99,11 +107,11 @@ StreamPlan plan_grad_output_stream(int64_t planes_f, int h, int w, size_t elem_s
 // and every workgroup stores its five partial sums in its own slot (nothing to clear, no atomics,
 // results reproducible bit for bit); with acc_slots == 0 it is [C*F*5] doubles, cleared by
 // grad_params_begin, and workgroups add atomically. grad_params_finish takes the same two values.
-// local_integral ([planes*F, h+1, w+1]) may be null: no integral. At least one of the two must
-// be given.
+// column_workspace ([planes*F] planes of column_workspace_plane(h, w) elements) may be null: no
+// workspace for the gradient w.r.t. the input. At least one of the two must be given.
 template <class T>
 hipError_t grad_output_stream_launch(const T* integ, const T* grad_out, BoxParams<T> prm,
-                                     double* acc, int acc_slots, T* local_integral,
+                                     double* acc, int acc_slots, T* column_workspace,
                                      const StreamPlan& sp, Dims d, bool exact, hipStream_t stream);
 
 hipError_t grad_params_begin(double* acc, int n_boxes, hipStream_t stream);

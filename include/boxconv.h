@@ -47,7 +47,7 @@ const char* boxconv_last_error(void);
  * boxconv_profile_arm(name): from now on every launch of the kernel called `name` is bracketed by
  * a pair of HIP events recorded on the stream it is launched on (so the time is that kernel's
  * alone, whatever else the entry point launches). Names: "band_colsum", "band_prefix",
- * "band_scan", "forward_rows", "grad_output_stream", "grad_input_rows",
+ * "band_scan", "forward_rows", "grad_output_stream", "grad_input_cols",
  * "param_grad_finalize", "fill_zero", "fill_marker", "clip", "forward_gather", "grad_input_gather",
  * "grad_params_gather".
  * NULL or "" disarms. Arming discards earlier measurements.

@@ -103,7 +103,7 @@ def test_workspace_sizes(lib):
     full = lib.boxconv_backward_workspace_bytes(2, 16, 8, 512, 1024, 4, 1, 1)
     only_params = lib.boxconv_backward_workspace_bytes(2, 16, 8, 512, 1024, 4, 0, 1)
     only_input = lib.boxconv_backward_workspace_bytes(2, 16, 8, 512, 1024, 4, 1, 0)
-    gint = 2 * 16 * 8 * 513 * 1025 * 4
+    gint = 2 * 16 * 8 * 513 * 1024 * 4     # column workspace: h+1 rows of w (rounded up to 4) per (plane, filter)
     # per-box sums: five doubles per (batch item, box, row band), 256-byte granules
     assert only_params % 256 == 0 and only_params >= 2 * 16 * 8 * 5 * 8
     assert only_params % (2 * 16 * 8 * 5 * 8) == 0

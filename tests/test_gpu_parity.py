@@ -150,6 +150,7 @@ SMALL_CASES = [
     (1, 2, 2, 17, 65), (1, 1, 3, 40, 130), (1, 2, 2, 33, 300), (1, 1, 2, 20, 600),
     (1, 1, 2, 12, 1100), (1, 1, 1, 9, 2100), (1, 1, 2, 1, 1), (1, 1, 2, 1, 70), (1, 1, 2, 70, 1),
     (1, 1, 2, 12, 700), (1, 2, 1, 10, 768), (1, 1, 2, 11, 1300), (1, 1, 1, 9, 1536),   # three columns per lane
+    (1, 1, 2, 40, 2048), (1, 2, 2, 21, 1800), (1, 1, 1, 10, 2047),      # 512 threads, four columns per lane
     # narrow images with four filters or more: the waves of a grad-input workgroup share the
     # filters (one turn with idle waves, two turns with the second partial, full-width rows)
     (1, 2, 4, 9, 20), (1, 2, 11, 19, 33), (2, 1, 16, 12, 64),

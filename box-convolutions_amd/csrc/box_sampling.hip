@@ -361,33 +361,40 @@ struct StreamLds {
     int glen;
 };
 
-__host__ __device__ inline size_t stream_lds_elems(int K, int nt) {
+__host__ __device__ constexpr size_t stream_lds_elems(int K, int nt) {
     const size_t glen = static_cast<size_t>(K) * nt + 8;
     return 4 * glen + 2 * static_cast<size_t>(K) * nt + 16 + static_cast<size_t>(K) * nt;
 }
-__host__ __device__ inline size_t stream_lds_bytes(int K, int nt, size_t elem) {
+__host__ __device__ constexpr size_t stream_lds_bytes(int K, int nt, size_t elem) {
     const size_t b = (stream_lds_elems(K, nt) * elem + 15) / 16 * 16;
     return b + (4 * kMaxRowWaves + 5 * kMaxRowWaves) * sizeof(double);
 }
 
+// `lds_base`: the kernel's own statically sized array, so that every LDS address is a lane
+// offset plus a compile-time constant (a dynamically sized array has a link-time base that costs
+// an addition per access).
 template <class T>
-__device__ __forceinline__ StreamLds<T> carve_stream_lds(int K, int nt) {
+__device__ __forceinline__ StreamLds<T> carve_stream_lds(unsigned char* lds_base, int K, int nt) {
     StreamLds<T> l;
     l.glen = K * nt + 8;
-    l.grow = reinterpret_cast<RowPair<T>*>(smem_raw);
+    l.grow = reinterpret_cast<RowPair<T>*>(lds_base);
     l.wrow = l.grow + 2 * l.glen;
     l.xw = reinterpret_cast<T*>(l.wrow + K * nt);
     l.delta = l.xw + 16;
     const size_t b = (stream_lds_elems(K, nt) * sizeof(T) + 15) / 16 * 16;
-    l.red = reinterpret_cast<double*>(smem_raw + b);
+    l.red = reinterpret_cast<double*>(lds_base + b);
     l.wave_tot = reinterpret_cast<T*>(l.red + 5 * kMaxRowWaves);
     l.wave_tail = reinterpret_cast<T*>(l.red + 7 * kMaxRowWaves);
     return l;
 }
 
 
+// Register budget: with three or four columns per lane the kernel needs more registers than
+// three waves per SIMD leave (170); told so, the compiler takes the 256 of two waves per SIMD
+// instead of spilling.
 template <class T, int NT, int K, bool EXACT, bool FULL, bool PARAMS, bool SCAN>
-__global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a) {
+__global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu((K >= 3 && PARAMS && SCAN) ? 2 : 1, (K >= 3 && PARAMS && SCAN) ? 2 : 8)))
+grad_output_stream_kernel(SampleArgs<T> a) {
     const unsigned vid = xcd_contiguous_id(a.per_xcd);
     if (vid >= a.total) return;                      // whole workgroup leaves together
     const unsigned nbands = a.nb, nfilt = a.F;
@@ -418,7 +425,8 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
     const bool keep_in_cache =
         static_cast<uint64_t>(from_end) * a.R * mpitch * sizeof(T) < static_cast<uint64_t>(a.keep_tail);
     const Rows<T, FULL> mout(mrows, mpitch, static_cast<int>(mpitch), h + 1);
-    const StreamLds<T> lds = carve_stream_lds<T>(K, nt);
+    __shared__ __align__(16) unsigned char lds_bytes[stream_lds_bytes(K, NT, sizeof(T))];
+    const StreamLds<T> lds = carve_stream_lds<T>(lds_bytes, K, nt);
     const int glen = lds.glen;
 
     const int i0 = band * a.R;
@@ -427,12 +435,19 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
     // The first two rows of grad_output are requested before anything else: they come from HBM
     // and need nothing but the workgroup's coordinates, so their latency runs alongside the
     // set-up below (LDS clearing, box parameters, column weights).
-    const int q1 = lane_q1<T>();
+    // Column slots: a wave owns 64*K consecutive columns, lane l of wave v the pixel columns
+    // jbase + 64*k, jbase = v*64*K + l (integral columns q = j + 1). Loads are lane-consecutive
+    // dwords as with workgroup-wide slots, and the columns a lane owns in the second part of a row
+    // pair (K consecutive ones, K*tid ..) belong to the same wave, so that the change of ownership
+    // goes through LDS without a workgroup barrier.
+    constexpr int CH = 64 * K;
+    const int jbase = wave * CH + lane;
+    const int q1 = (1 + jbase) * static_cast<int>(sizeof(T));
     T g0[K], g1[K];
     auto load_g = [&](int i, T (&dst)[K]) {
         const RowRef r = grows.row(min(i, h - 1), i < i1);     // rows past the band read as zeros
 #pragma unroll
-        for (int k = 0; k < K; ++k) dst[k] = load_slot<T, NT, kCacheStream>(r, q1, k);
+        for (int k = 0; k < K; ++k) dst[k] = load_slot<T, 64, kCacheStream>(r, q1, k);
     };
     load_g(i0, g0);
     load_g(i0 + 1, g1);
@@ -470,7 +485,7 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
     bool wave_has_tail = false;
 #pragma unroll
     for (int k = 0; k < K; ++k) {
-        const int j = tid + nt * k;
+        const int j = jbase + 64 * k;
         ir[k] = tap_r(j + 1, s.yhi);
         il[k] = tap_l(j + 1, s.ylo);
         const T d = (FULL || j < w) ? tail_weight(j, s.ylo, s.yhi, s.fylo, s.fyhi) : T(0);
@@ -500,22 +515,24 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
 
     T ta[K], bc[K], t0[K], t1[K], b1[K], b2[K];
     if (PARAMS) {
-        load_row<T, NT, K>(irows.row(clampi(i0 + s.xlo - 1, 0, h)), q1, ta);
-        load_row<T, NT, K>(irows.row(clampi(i0 + s.xhi, 0, h)), q1, bc);
-        load_pair<T, NT, K, FULL>(irows, i0, s.xlo, s.xhi, h, q1, t0, t1, b1, b2);
+        load_row<T, 64, K>(irows.row(clampi(i0 + s.xlo - 1, 0, h)), q1, ta);
+        load_row<T, 64, K>(irows.row(clampi(i0 + s.xhi, 0, h)), q1, bc);
+        load_pair<T, 64, K, FULL>(irows, i0, s.xlo, s.xhi, h, q1, t0, t1, b1, b2);
     }
 
-    int flip = 0;
-    auto row_pair = [&](int i, auto prefetch_tag) {
-        constexpr bool PREFETCH = decltype(prefetch_tag)::value;   // see forward_rows_kernel
-        // (the LDS buffer alternates at run time here: unrolling this loop over both buffers, as
-        // the forward kernel does, costs more registers than the kernel can afford)
-        const int FLIP = flip;
-        flip ^= 1;
+    // PREFETCH and the LDS buffer are compile-time tags (see forward_rows_kernel): the loop below
+    // is unrolled over both buffers, so LDS addresses are lane constants plus immediates and the
+    // sliding rows rotate by renaming instead of moves.
+    // OWN_W: the rare box whose mirrored split differs (see above); a tag as well, so that the
+    // common case carries none of its code.
+    auto row_pair = [&](int i, auto prefetch_tag, auto flip_tag, auto own_w_tag) {
+        constexpr bool PREFETCH = decltype(prefetch_tag)::value;
+        constexpr int FLIP = decltype(flip_tag)::value;
+        constexpr bool OWN_W = decltype(own_w_tag)::value;
         T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {}, m0[K] = {}, m1[K] = {};
         if (PREFETCH) {
             if (PARAMS)
-                load_pair<T, NT, K, FULL>(irows, i + 2, s.xlo, s.xhi, h, q1, n0, n1, n2, n3);
+                load_pair<T, 64, K, FULL>(irows, i + 2, s.xlo, s.xhi, h, q1, n0, n1, n2, n3);
             load_g(i + 2, m0);
             load_g(i + 3, m1);
         }
@@ -527,14 +544,14 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
         T tail0 = T(0), tail1 = T(0);
 #pragma unroll
         for (int k = 0; k < K; ++k) {
-            if (slot_valid<T, NT, FULL>(q1, k, row_bytes))
-                *at_bytes(G + kGPad - 1 + NT * k, 2 * q1) = RowPair<T>{g0[k], g1[k]};
+            if (slot_valid<T, 64, FULL>(q1, k, row_bytes))
+                *at_bytes(G + kGPad - 1 + 64 * k, 2 * q1) = RowPair<T>{g0[k], g1[k]};
             {
-                const T dlt = *at_bytes(lds.delta - 1 + NT * k, q1);
+                const T dlt = *at_bytes(lds.delta - 1 + 64 * k, q1);
                 tail0 += dlt * g0[k];
                 tail1 += dlt * g1[k];
             }
-            if (PARAMS && (FULL ? (k == K - 1 && tid == nt - 1) : (q1 + slot_bytes<T, NT>(k) == row_bytes))) {   // owner of column q = w
+            if (PARAMS && (FULL ? (k == K - 1 && tid == nt - 1) : (q1 + slot_bytes<T, 64>(k) == row_bytes))) {   // owner of column q = w
                 const T dt0 = t0[k] - ta[k], db0 = b1[k] - bc[k];
                 const T dt1 = t1[k] - t0[k], db1 = b2[k] - b1[k];
                 T v0 = bc[k] - t0[k], v1 = b1[k] - t1[k];
@@ -602,13 +619,13 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
         }
 
         if (SCAN) {
-            if (own_w) {
+            if (OWN_W) {
                 // rare: the mirrored split cuts the box at other whole pixels; weights and tails
                 // of M from that split, tap offsets worked out on the spot
                 tail0 = T(0); tail1 = T(0);
 #pragma unroll
                 for (int k = 0; k < K; ++k) {
-                    const int j = tid + nt * k;
+                    const int j = jbase + 64 * k;
                     const RowPair<T>* R = at_bytes(G, tap_r(j + 1, yhi_m));
                     const RowPair<T>* L = at_bytes(G, tap_l(j + 1, ylo_m));
                     const RowPair<T> grA = R[0], gr = R[1], gl = L[0], glA = L[1];
@@ -626,15 +643,19 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
             // W rows by pixel column c = q - 1, and the wave's share of the tails
 #pragma unroll
             for (int k = 0; k < K; ++k)
-                if (slot_valid<T, NT, FULL>(q1, k, row_bytes))
-                    *at_bytes(lds.wrow - 1 + NT * k, 2 * q1) = RowPair<T>{wq0[k], wq1[k]};
+                if (slot_valid<T, 64, FULL>(q1, k, row_bytes))
+                    *at_bytes(lds.wrow - 1 + 64 * k, 2 * q1) = RowPair<T>{wq0[k], wq1[k]};
             T wt0 = T(0), wt1 = T(0);
             if (wave_has_tail) {
                 wt0 = wave_sum_to_last(tail0);
                 wt1 = wave_sum_to_last(tail1);
             }
-            if (lane == 63) { lds.wave_tail[wave] = wt0; lds.wave_tail[kMaxRowWaves + wave] = wt1; }
-            __syncthreads();                                                 // W rows are in LDS
+            // The columns written above and the columns read below belong to this wave: LDS
+            // serves a wave's accesses in order, so only the compiler has to be kept from moving
+            // the reads up.
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
             // the lane's K consecutive columns K*tid .. K*tid+K-1: exclusive prefix of W inside
             // the lane, the lanes to the left by a wave scan
@@ -653,7 +674,10 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
                 const T inc1 = wave_inclusive_scan(run1);
                 base0 = run0 - inc0;                                         // -(lanes to the left)
                 base1 = run1 - inc1;
-                if (lane == 63) { lds.wave_tot[wave] = inc0; lds.wave_tot[kMaxRowWaves + wave] = inc1; }
+                if (lane == 63) {
+                    lds.wave_tot[wave] = inc0; lds.wave_tot[kMaxRowWaves + wave] = inc1;
+                    lds.wave_tail[wave] = wt0; lds.wave_tail[kMaxRowWaves + wave] = wt1;
+                }
             }
             __syncthreads();                                                 // wave totals visible
             {
@@ -678,22 +702,20 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
                 const bool second = i + 1 < i1;
                 const RowRef ob0 = mout.row(i + 1);
                 const RowRef ob1 = mout.row(min(i + 2, h), second);
-                T out0[K], out1[K];
+                T out0[K];
 #pragma unroll
                 for (int k = 0; k < K; ++k) {
-                    colacc[k] += base0 - ex0[k];
-                    out0[k] = colacc[k];
-                    colacc[k] += base1 - ex1[k];
-                    out1[k] = colacc[k];
+                    out0[k] = colacc[k] + (base0 - ex0[k]);
+                    colacc[k] = out0[k] + (base1 - ex1[k]);
                 }
                 const int first = K * tid * static_cast<int>(sizeof(T));
                 const int limit = static_cast<int>(mpitch * sizeof(T));
                 if (keep_in_cache) {
                     buffer_store_run<kCacheDefault, FULL>(out0, ob0, first, limit);
-                    buffer_store_run<kCacheDefault, FULL>(out1, ob1, first, limit);
+                    buffer_store_run<kCacheDefault, FULL>(colacc, ob1, first, limit);
                 } else {
                     buffer_store_run<kCacheStream, FULL>(out0, ob0, first, limit);
-                    buffer_store_run<kCacheStream, FULL>(out1, ob1, first, limit);
+                    buffer_store_run<kCacheStream, FULL>(colacc, ob1, first, limit);
                 }
             }
         }
@@ -712,9 +734,25 @@ __global__ void __launch_bounds__(NT) grad_output_stream_kernel(SampleArgs<T> a)
         // only add live registers
         __builtin_amdgcn_sched_barrier(0);
     };
-    int i = i0;
-    for (; i + 2 < i1; i += 2) row_pair(i, std::true_type{});
-    row_pair(i, std::false_type{});
+    // (written out twice rather than through another lambda: arrays captured through two levels
+    // of closures end up in scratch memory)
+#define BOXCONV_ALL_PAIRS(OWN_W_TAG)                                         \
+    {                                                                        \
+        int i = i0;                                                          \
+        for (; i + 4 < i1; i += 4) {                                         \
+            row_pair(i, std::true_type{}, Flip0{}, OWN_W_TAG{});             \
+            row_pair(i + 2, std::true_type{}, Flip1{}, OWN_W_TAG{});         \
+        }                                                                    \
+        if (i + 2 < i1) {                                                    \
+            row_pair(i, std::true_type{}, Flip0{}, OWN_W_TAG{});             \
+            row_pair(i + 2, std::false_type{}, Flip1{}, OWN_W_TAG{});        \
+        } else {                                                             \
+            row_pair(i, std::false_type{}, Flip0{}, OWN_W_TAG{});            \
+        }                                                                    \
+    }
+    if (own_w) BOXCONV_ALL_PAIRS(std::true_type)
+    else BOXCONV_ALL_PAIRS(std::false_type)
+#undef BOXCONV_ALL_PAIRS
 
     if (PARAMS) {
         __syncthreads();
@@ -959,7 +997,7 @@ hipError_t grad_output_stream_launch(const T* integ, const T* grad_out, BoxParam
     finish_args(a, planes_f * a.nb);
     const RowConfig rc = stream_row_config(d.w);
     const dim3 grid(static_cast<unsigned>(a.per_xcd * kXcds));
-    const size_t lds = stream_lds_bytes(rc.K, rc.nt, sizeof(T));
+    const size_t lds = 0;                              // the kernel's LDS is statically sized
 #define LAUNCH_GS(NT, KK, EX, FU) \
     if (params && scan) BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_kernel<T, NT, KK, EX, FU, true, true>), grid, dim3(NT), lds, stream, a); \
     else if (params)    BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_kernel<T, NT, KK, EX, FU, true, false>), grid, dim3(NT), lds, stream, a); \

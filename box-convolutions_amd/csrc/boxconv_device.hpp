@@ -122,6 +122,22 @@ __device__ __forceinline__ A wave_inclusive_scan(A x) {
     return x;
 }
 
+// The same for float with the two row broadcasts written as single instructions: an addition
+// whose first operand comes through DPP and which leaves the rows outside the row mask
+// untouched. (From the generic form above the compiler makes a zeroed register, a DPP move and
+// an addition for each of them.) The wait states a DPP read needs after the write of its source
+// are part of the statement, since the compiler does not look inside it.
+template <>
+__device__ __forceinline__ float wave_inclusive_scan<float>(float x) {
+    x += dpp_move<0x111, 0xf>(x, x);
+    x += dpp_move<0x112, 0xf>(x, x);
+    x += dpp_move<0x114, 0xf>(x, x);
+    x += dpp_move<0x118, 0xf>(x, x);
+    asm volatile("s_nop 1\n\tv_add_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf" : "+v"(x));
+    asm volatile("s_nop 1\n\tv_add_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf" : "+v"(x));
+    return x;
+}
+
 // Sum over the wave, valid in lane 63 (and only there). All lanes must be active.
 template <class A>
 __device__ __forceinline__ A wave_sum_to_last(A x) { return wave_inclusive_scan(x); }

@@ -1,11 +1,14 @@
 """The five BASELINE workloads at full size on the GPU, through BoxConv2d (training mode, all
 five gradients), against the CPU oracle.
 
-Workloads 1, 2 and 4 are compared in full. Workloads 3 and 5 are compared on their first input
-planes (box convolution is independent per input plane, and a parameter gradient only sums over
-the batch, so the oracle restricted to planes [0, c) reproduces exactly those slices of the full
+Workloads 1 to 4 are compared in full. Workload 5 is compared on its first 16 of 128 input planes
+(box convolution is independent per input plane, and a parameter gradient only sums over the
+batch, so the oracle restricted to planes [0, c) reproduces exactly those slices of the full
 result), plus a size-independent property on the whole tensors: the adjoint identity
 <boxconv(x), g> = <x, grad_input(g)>.
+
+Every run prints its measured errors; with BOXCONV_PARITY_REPORT=<file> they are appended to that
+file as well (this is how profiles/parity_errors.txt is made).
 
 Tolerances: forward, grad_input 1e-4; parameter gradients 1e-3 (max|gpu-cpu| / max|cpu|).
 
@@ -14,9 +17,13 @@ the precision limit of the float32 reference itself: its parameter gradients are
 two nearly equal terms (for a constant image the gradient of a normalised box vanishes), and the
 reference's float32 result deviates from the same algorithm run in float64 by about 2e-3
 (measured: y_max 1.8e-3), the GPU result by about 3e-4. There the GPU is held to 1e-3 against
-the float64 oracle, must be at least as close to it as the float32 oracle is, and to 4e-3
-against the float32 oracle.
+the float64 oracle and must be at least as close to it as the float32 oracle is; its distance to
+the float32 oracle is held to 1e-3 or, where the float32 oracle itself is further than that from
+float64, to the sum of the two distances to float64 (nothing but the reference's own rounding
+error may separate them).
 """
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -27,7 +34,15 @@ from helpers import param_grad_floor, rel_err
 pytestmark = pytest.mark.gpu
 
 # planes the oracle is run on (None = all)
-ORACLE_PLANES = {1: None, 2: None, 3: 2, 4: None, 5: 1}
+ORACLE_PLANES = {1: None, 2: None, 3: None, 4: None, 5: 16}
+
+
+def report(line):
+    print(line)
+    path = os.environ.get("BOXCONV_PARITY_REPORT")
+    if path:
+        with open(path, "a") as fh:
+            fh.write(line + "\n")
 
 
 def run_gpu(wl):
@@ -72,7 +87,10 @@ def test_baseline_workload(oracle, k):
     e_gin = rel_err(gin[:, :c].cpu().numpy(), grads_c[0])
     floor = param_grad_floor(grads_c[1:])
     e_par = [rel_err(gp[:c].cpu().numpy(), gc, floor) for gp, gc in zip(gpar, grads_c[1:])]
-    print("workload %d: forward %.2e grad_input %.2e grad_params %s" % (k, e_out, e_gin, ["%.2e" % e for e in e_par]))
+    report("workload %d (%s), oracle on %d of %d input planes: adjoint identity |lhs-rhs|/sum|terms| %.2e; "
+           "max|gpu-cpu|/max|cpu|: forward %.2e grad_input %.2e grad_x_min %.2e grad_x_max %.2e "
+           "grad_y_min %.2e grad_y_max %.2e"
+           % (k, wl.name, c, wl.C, abs(lhs - rhs) / scale, e_out, e_gin, *e_par))
     assert e_out <= 1e-4
     assert e_gin <= 1e-4
     if k != 5:
@@ -89,8 +107,9 @@ def test_baseline_workload(oracle, k):
     floor64 = param_grad_floor(grads64[1:])
     e_gpu64 = [rel_err(gp[:c].cpu().numpy(), g64, floor64) for gp, g64 in zip(gpar, grads64[1:])]
     e_cpu64 = [rel_err(gc, g64, floor64) for gc, g64 in zip(grads_c[1:], grads64[1:])]
-    print("workload 5 vs float64 oracle: gpu %s  float32 oracle %s"
-          % (["%.2e" % e for e in e_gpu64], ["%.2e" % e for e in e_cpu64]))
+    report("workload 5 parameter gradients vs the float64 oracle (x_min x_max y_min y_max): gpu %s ; "
+           "float32 cpu oracle %s" % (" ".join("%.2e" % e for e in e_gpu64), " ".join("%.2e" % e for e in e_cpu64)))
     assert max(e_gpu64) <= 1e-3
     assert max(e_gpu64) <= max(max(e_cpu64), 1e-4)
-    assert max(e_par) <= 4e-3
+    for e, eg, ec in zip(e_par, e_gpu64, e_cpu64):
+        assert e <= max(1e-3, 1.05 * (eg + ec))

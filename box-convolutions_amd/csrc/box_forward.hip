@@ -189,7 +189,10 @@ hipError_t forward_launch_any(const T* integ, BoxParams<T> prm, ForwardTail<TO> 
     SampleArgs<T> a = base_args(prm, d);
     a.src = integ; a.normalize = normalize ? 1 : 0;
 
-    if (!row_kernels_apply(d.h, d.w, sizeof(T))) {
+    // (the row kernel keeps two row pairs of w + 3 columns in LDS: float64 rows of 2046 columns
+    // and more would ask for more than a launch gets without opting in)
+    if (!row_kernels_apply(d.h, d.w, sizeof(T)) ||
+        4 * static_cast<size_t>(d.w + 3) * sizeof(T) > kMaxDynamicLds) {
         finish_args(a, planes_f * d.hw());
         const dim3 grid(static_cast<unsigned>((a.total + 255) / 256));
         if (exact) BOXCONV_LAUNCH("forward_gather", (forward_gather_kernel<T, TO, true, TAIL>), grid, dim3(256), 0, stream, a, tail);

@@ -1,6 +1,7 @@
 // extern "C" entry points of libboxconv_hip.so (declared in include/boxconv.h): argument checks on
 // the host, workspace carving, kernel launches. No torch types, no allocation, no synchronisation.
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -18,7 +19,8 @@ namespace boxconv {
 // ---- per-kernel timing ------------------------------------------------------------------------
 namespace {
 std::mutex g_prof_mutex;
-std::string g_prof_name;                                   // empty: disarmed
+std::atomic<bool> g_prof_armed{false};                     // read without the lock by every launch
+std::string g_prof_name;                                   // empty: disarmed; guarded by the mutex
 std::vector<std::pair<hipEvent_t, hipEvent_t>> g_prof_events;
 hipEvent_t g_prof_open = nullptr;
 int g_prof_every = 1;                                      // bracket one launch in this many
@@ -27,7 +29,7 @@ constexpr size_t kMaxProfiledLaunches = 1 << 16;
 }  // namespace
 
 void profile_before(const char* name, hipStream_t stream) {
-    if (g_prof_name.empty()) return;                       // unlocked fast path: not armed
+    if (!g_prof_armed.load(std::memory_order_acquire)) return;   // fast path: not armed
     std::lock_guard<std::mutex> lock(g_prof_mutex);
     if (g_prof_name != name || g_prof_events.size() >= kMaxProfiledLaunches) return;
     if (g_prof_seen++ % g_prof_every != 0) return;
@@ -38,7 +40,7 @@ void profile_before(const char* name, hipStream_t stream) {
 }
 
 void profile_after(const char* name, hipStream_t stream) {
-    if (g_prof_name.empty()) return;
+    if (!g_prof_armed.load(std::memory_order_acquire)) return;
     std::lock_guard<std::mutex> lock(g_prof_mutex);
     if (g_prof_open == nullptr || g_prof_name != name) return;
     hipEvent_t stop = nullptr;
@@ -87,18 +89,6 @@ int check_dims(int batch, int in_planes, int num_filters, int h, int w) {
     return 0;
 }
 
-// The backward pass can walk the (batch, plane) pairs in chunks so that the integral image of a
-// chunk of grad_output is consumed while it is still cache resident; the chunk (in planes) comes
-// from BOXCONV_BWD_CHUNK_PLANES, default: everything in one go.
-int64_t backward_chunk_planes(int64_t planes) {
-    static const long env = [] {
-        const char* e = std::getenv("BOXCONV_BWD_CHUNK_PLANES");
-        return e ? std::atol(e) : 0L;
-    }();
-    if (env > 0 && env < planes) return env;
-    return planes;
-}
-
 // Walk the planes last to first in the second pass over a tensor (see integral_image_launch).
 bool reverse_second_pass() {
     static const bool v = [] {
@@ -109,53 +99,38 @@ bool reverse_second_pass() {
 }
 
 // Workspace of the backward pass:
-//   [column workspace M of grad_output: chunk*F planes of (h+1) rows, or their integral images
+//   [column workspace M of grad_output: planes*F planes of (h+1) rows, or their integral images
 //    of (h+1)(w+1) where the streaming pass does not apply]     only if grad_input is wanted
-//   [aux doubles: band column sums, three-pass fallback only]
+//   [aux doubles: band column sums of that integral image; gather path only]
 //   [acc: C*F*5 doubles, times batch*bands when every streaming workgroup has its own slot]
 //                                                              only if parameter gradients are wanted
 struct BackwardLayout {
     size_t gint_off, aux_off, acc_off, total;
-    int64_t chunk;        // planes per chunk
     int acc_slots;        // > 0: per-workgroup accumulation slots per (plane, filter), see grad_output_stream_launch
     bool streaming;       // grad_output_stream_kernel usable for this shape
 };
 
-template <class F>
-int64_t max_over_chunks(int64_t planes, int64_t chunk, F f) {
-    int64_t m = f(std::min(chunk, planes));
-    if (const int64_t rest = planes % chunk) m = std::max(m, f(rest));   // shorter last chunk
-    return m;
-}
-
 BackwardLayout backward_layout(int batch, int in_planes, int num_filters, int h, int w,
                                int elem_size, bool need_input, bool need_params) {
     BackwardLayout L{};
-    const int64_t planes = static_cast<int64_t>(batch) * in_planes;
-    L.chunk = std::max<int64_t>(backward_chunk_planes(planes), 1);
-    L.streaming = boxconv::plan_grad_output_stream(L.chunk * num_filters, h, w, elem_size).usable;
+    const int64_t planes = std::max<int64_t>(static_cast<int64_t>(batch) * in_planes, 1);
+    const boxconv::StreamPlan sp = boxconv::plan_grad_output_stream(planes * num_filters, h, w, elem_size);
+    L.streaming = sp.usable;
     size_t off = 0;
     L.gint_off = off;
     L.aux_off = off;
     if (need_input) {
-        // streaming: the column workspace M; else true integral images of (h+1) x (w+1)
         const size_t per_plane = L.streaming
             ? static_cast<size_t>(boxconv::column_workspace_plane(h, w))
             : static_cast<size_t>(h + 1) * (w + 1);
-        off += align_up(static_cast<size_t>(std::min(L.chunk, std::max<int64_t>(planes, 1))) *
-                        num_filters * per_plane * elem_size, 256);
+        off += align_up(static_cast<size_t>(planes) * num_filters * per_plane * elem_size, 256);
         L.aux_off = off;
-        const int64_t aux = max_over_chunks(std::max<int64_t>(planes, 1), L.chunk, [&](int64_t np) {
-            return L.streaming ? int64_t(0)
-                               : boxconv::plan_integral(np * num_filters, h, w).aux_doubles;
-        });
+        const int64_t aux = L.streaming ? int64_t(0)
+                                        : boxconv::plan_integral(planes * num_filters, h, w).aux_doubles;
         off += align_up(static_cast<size_t>(aux) * 8, 256);
     }
     L.acc_off = off;
-    // one accumulation slot per streaming workgroup when the whole batch goes in one chunk
-    L.acc_slots = 0;
-    if (need_params && L.streaming && L.chunk >= planes)
-        L.acc_slots = boxconv::plan_grad_output_stream(planes * num_filters, h, w, elem_size).nb;
+    L.acc_slots = (need_params && L.streaming) ? sp.nb : 0;
     if (need_params)
         off += align_up(static_cast<size_t>(in_planes) * num_filters * 5 * 8 *
                         (L.acc_slots > 0 ? static_cast<size_t>(batch) * L.acc_slots : 1), 256);
@@ -354,50 +329,39 @@ int backward_impl(const T* integ, const T* x_min, const T* x_max, const T* y_min
                                          n_boxes, reparam_h, reparam_w, normalize != 0, exact != 0};
     bool finished = false;
     const int64_t planes = static_cast<int64_t>(batch) * in_planes;
-    const int64_t hw = static_cast<int64_t>(h) * w;
-    const int64_t ipl = static_cast<int64_t>(h + 1) * (w + 1);
-    for (int64_t p0 = 0; p0 < planes; p0 += L.chunk) {
-        const int64_t np = std::min(L.chunk, planes - p0);
-        boxconv::Dims d{in_planes, num_filters, h, w, np, p0};
-        const T* go_chunk = grad_output + p0 * num_filters * hw;
-        const T* integ_chunk = integ ? integ + p0 * ipl : nullptr;
-        T* gin_chunk = need_input ? grad_input + p0 * hw : nullptr;
-        if (L.streaming) {
-            // one pass over grad_output: parameter sums + band-local integral, then grad_input
-            const boxconv::StreamPlan sp =
-                boxconv::plan_grad_output_stream(np * num_filters, h, w, sizeof(T));
-            if (int rc = hip_result(boxconv::grad_output_stream_launch<T>(
-                    integ_chunk, go_chunk, prm, acc, L.acc_slots, gint, sp, d, exact != 0, s),
-                    "grad_output streaming launch"))
+    const boxconv::Dims d{in_planes, num_filters, h, w, planes, 0};
+    if (L.streaming) {
+        // one pass over grad_output: parameter sums + column workspace, then grad_input, whose
+        // launch finishes the parameter gradients on the side
+        const boxconv::StreamPlan sp = boxconv::plan_grad_output_stream(planes * num_filters, h, w, sizeof(T));
+        if (int rc = hip_result(boxconv::grad_output_stream_launch<T>(
+                integ, grad_output, prm, acc, L.acc_slots, gint, sp, d, exact != 0, s),
+                "grad_output streaming launch"))
+            return rc;
+        if (need_input)
+            if (int rc = hip_result(boxconv::grad_input_launch<T>(
+                    gint, sp.R, prm, grad_input, d, normalize != 0, exact != 0, s,
+                    need_params ? &finish : nullptr, &finished),
+                    "input-gradient launch"))
                 return rc;
-            // (the sums of all chunks are complete once the last chunk's pass over grad_output
-            // is: its grad-input launch finishes the parameter gradients on the side)
-            const bool last = p0 + np == planes;
-            if (need_input)
-                if (int rc = hip_result(boxconv::grad_input_launch<T>(
-                        gint, sp.R, prm, gin_chunk, d, normalize != 0, exact != 0, s,
-                        need_params && last ? &finish : nullptr, &finished),
-                        "input-gradient launch"))
-                    return rc;
-        } else {
-            // any width: gather kernels on true integral images
-            if (need_params)
-                if (int rc = hip_result(boxconv::grad_params_gather_launch<T>(
-                        integ_chunk, go_chunk, prm, acc, d, exact != 0, s),
-                        "parameter-gradient launch"))
-                    return rc;
-            if (need_input) {
-                const boxconv::IntegralPlan plan = boxconv::plan_integral(np * num_filters, h, w);
-                if (int rc = hip_result(boxconv::integral_image_launch<T>(
-                        go_chunk, gint, np * num_filters, h, w, aux, plan, false,
-                        need_params && reverse_second_pass(), s),
-                        "grad_output integral image launch"))
-                    return rc;
-                if (int rc = hip_result(boxconv::grad_input_launch<T>(
-                        gint, 0, prm, gin_chunk, d, normalize != 0, exact != 0, s),
-                        "input-gradient launch"))
-                    return rc;
-            }
+    } else {
+        // any width: gather kernels on true integral images
+        if (need_params)
+            if (int rc = hip_result(boxconv::grad_params_gather_launch<T>(
+                    integ, grad_output, prm, acc, d, exact != 0, s),
+                    "parameter-gradient launch"))
+                return rc;
+        if (need_input) {
+            const boxconv::IntegralPlan plan = boxconv::plan_integral(planes * num_filters, h, w);
+            if (int rc = hip_result(boxconv::integral_image_launch<T>(
+                    grad_output, gint, planes * num_filters, h, w, aux, plan, false,
+                    need_params && reverse_second_pass(), s),
+                    "grad_output integral image launch"))
+                return rc;
+            if (int rc = hip_result(boxconv::grad_input_launch<T>(
+                    gint, 0, prm, grad_input, d, normalize != 0, exact != 0, s),
+                    "input-gradient launch"))
+                return rc;
         }
     }
     if (need_params && !finished)
@@ -441,6 +405,7 @@ int boxconv_profile_arm_every(const char* kernel_name, int every) {
     }
     boxconv::g_prof_events.clear();
     boxconv::g_prof_name = kernel_name ? kernel_name : "";
+    boxconv::g_prof_armed.store(!boxconv::g_prof_name.empty(), std::memory_order_release);
     return 0;
 }
 
@@ -460,6 +425,7 @@ int boxconv_profile_collect(double* total_ms, int* launches) {
     }
     boxconv::g_prof_events.clear();
     boxconv::g_prof_name.clear();
+    boxconv::g_prof_armed.store(false, std::memory_order_release);
     if (total_ms) *total_ms = sum;
     if (launches) *launches = n;
     return rc;

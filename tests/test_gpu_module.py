@@ -89,6 +89,47 @@ def test_integral_image_like_reference_test():
         assert integral_image(x).allclose(want.float())        # default rtol/atol, reference test.py:53
 
 
+def test_native_module_stand_in_on_the_gpu(oracle):
+    """The four functions of `box_convolution_cpp_cuda` called the way the reference's Python layer
+    calls them (box_convolution_function.py:44-46,59-62; box_convolution_module.py:203-206),
+    against the CPU oracle; gradients that were not asked for come back as 0-element tensors
+    (reference src/box_convolution_interface.cpp:181-183,394)."""
+    import box_convolution_cpp_cuda as cpp_cuda
+    from helpers import make_boxes
+    rng = np.random.default_rng(31)
+    B, C, F, h, w = 2, 3, 2, 21, 34
+    x = rng.standard_normal((B, C, h, w)).astype(np.float32)
+    g = rng.standard_normal((B, C * F, h, w)).astype(np.float32)
+    boxes = make_boxes(rng, C, F, h, w, "hanging")
+    dev_boxes = [torch.from_numpy(b).to(DEV) for b in boxes]
+    integ = cpp_cuda.integral_image(torch.from_numpy(x).to(DEV))
+    out = cpp_cuda.box_convolution_forward(integ, *dev_boxes, True, True)
+    integ_c = oracle.integral_image(x)
+    out_c = oracle.box_forward(integ_c, *boxes, True, True)
+    assert np.abs(out.cpu().numpy() - out_c).max() <= 1e-4 * np.abs(out_c).max()
+    for needs in [(True, True, True, True, True), (True, False, False, False, False),
+                  (False, True, False, False, True), (False, False, True, True, False)]:
+        grads = cpp_cuda.box_convolution_backward(integ, *dev_boxes, torch.from_numpy(g).to(DEV), out,
+                                                  3.0, 5.0, True, True, *needs)
+        grads_c = oracle.box_backward(integ_c, *boxes, g, out_c, 3.0, 5.0, True, True, needs)
+        assert len(grads) == 5
+        scale = max(np.abs(gc).max() for gc in grads_c[1:] if gc is not None) if any(needs[1:]) else 1.0
+        for i, (got, want, need) in enumerate(zip(grads, grads_c, needs)):
+            if not need:
+                assert isinstance(got, torch.Tensor) and got.numel() == 0
+                continue
+            tol = 1e-4 * np.abs(want).max() if i == 0 else 1e-3 * max(np.abs(want).max(), 1e-2 * scale)
+            assert got.shape == want.shape and np.abs(got.cpu().numpy() - want).max() <= tol, (needs, i)
+    # clip_parameters: in place on the stored parameters, bit for bit as the oracle
+    stored = [torch.from_numpy((b / s).astype(np.float32)).to(DEV)
+              for b, s in zip(boxes, (8.0 * h, 8.0 * h, 8.0 * w, 8.0 * w))]
+    host = [p.cpu().numpy().copy() for p in stored]
+    assert cpp_cuda.clip_parameters(*stored, 8.0 * h, 8.0 * w, float(h), float(w), True) is None
+    oracle.clip_parameters(*host, 8.0 * h, 8.0 * w, float(h), float(w), True)
+    for p, q in zip(stored, host):
+        assert np.array_equal(p.cpu().numpy(), q)
+
+
 @pytest.mark.parametrize("seed", range(12))
 def test_module_against_conv2d_like_reference_test(seed):
     rng = random.Random(1546545757 + seed)

@@ -113,6 +113,11 @@ def main():
     ap.add_argument("--workload", type=int, default=3, choices=[1, 2, 3, 4, 5])
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--phases", action="store_true", help="also print per-kernel times to stderr")
+    ap.add_argument("--graph", action="store_true",
+                    help="time replays of a captured HIP graph of the step's native calls (training "
+                         "forward + backward through the C ABI) instead of the eager module step: "
+                         "the same kernels without Python, autograd and launch latency, which bound "
+                         "the small workloads")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
                     help="after the timed steps, run torch.neg on a float tensor of this many MiB "
                          "(reads MIB, writes MIB): the plain streaming kernel of known size that "
@@ -144,12 +149,14 @@ def main():
     g = wl.grad_output.to(dev)
     params = list(module.parameters())
 
-    def step():
+    def eager_step():
         x.grad = None
         for p in params:
             p.grad = None
         out = module(x)
         out.backward(g)
+
+    step = eager_step
 
     before = [p.detach().clone() for p in params]
     for _ in range(args.warmup):
@@ -178,14 +185,39 @@ def main():
             break
         last = cur
 
-    # which kernel takes the most time per step (one untimed step per candidate)
+    # which kernel takes the most time per step (three untimed eager steps per candidate)
     per_kernel = {}
     for name in TIMED_KERNELS:
         _native.profile_arm(name)
-        step()
+        for _ in range(3):
+            eager_step()
         ms, launches = _native.profile_collect()
-        per_kernel[name] = (ms, launches)
+        per_kernel[name] = (ms / 3, launches // 3, ms / max(launches, 1))
     dominant = max(per_kernel, key=lambda n: per_kernel[n][0])
+
+    if args.graph:
+        # the native calls of one step, captured once: clip + integral image + forward, backward
+        stored = [p.detach() for p in (module.x_min, module.x_max, module.y_min, module.y_max)]
+        x_static = x.detach()
+
+        def native_step():
+            integ, out, real = _native.training_forward(
+                x_static, *stored, wl.reparametrization_h, wl.reparametrization_w, wl.h, wl.w, True, True)
+            return out, _native.box_convolution_backward(
+                integ, *real, g, None, wl.reparametrization_h, wl.reparametrization_w, True, True,
+                True, True, True, True, True)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            native_step()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            keep_alive = native_step()
+        step = graph.replay
+        for _ in range(max(args.warmup, 5)):
+            step()
+        torch.cuda.synchronize()
     if args.phases:
         print("per-kernel ms per step:", {k: round(v[0], 4) for k, v in per_kernel.items()},
               file=sys.stderr)
@@ -196,9 +228,14 @@ def main():
     # An event pair around a kernel costs about 2.5 us of GPU time each side on this machine,
     # 1 % of a step: the dominant kernel is bracketed at one launch in EVENT_EVERY, so that the
     # whole-step figure is perturbed by a fraction of that.
-    _native.profile_arm(dominant, every=EVENT_EVERY)
+    if not args.graph:
+        _native.profile_arm(dominant, every=EVENT_EVERY)
     regions = [timed_block(args.steps) for _ in range(REPEATS)]
-    dom_ms, dom_launches = _native.profile_collect()
+    if args.graph:
+        # launches inside a replayed graph cannot be bracketed: the eager measurement above stands in
+        dom_ms, dom_launches = per_kernel[dominant][2] * 3, 3
+    else:
+        dom_ms, dom_launches = _native.profile_collect()
     elapsed = sorted(regions)[len(regions) // 2]
 
     if args.copy_probe > 0:
@@ -236,6 +273,7 @@ def main():
             "workload": "%s: BoxConv2d(%d,%d,%d,%d) fwd+bwd, input [%d,%d,%d,%d], normalize, exact, "
                         "grads to input and 4 box parameters" % (
                             wl.name, wl.C, wl.F, wl.h, wl.w, wl.B, wl.C, wl.h, wl.w),
+            "mode": "captured HIP graph of the step's native calls" if args.graph else "eager module step",
             "algorithmic_bytes_per_step": ab["alg"],
             "io_bytes_per_step": ab["io"],
             "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),

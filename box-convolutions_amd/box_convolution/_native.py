@@ -43,6 +43,8 @@ for _s in ("f32", "f64"):
     _SIGNATURES["boxconv_training_forward_" + _s] = (
         _i, [_vp] * 8 + [_i] * 5 + [_d] * 4 + [_i, _i] + [_vp, _sz, _vp])
 
+_SIGNATURES["boxconv_backward_half_f32"] = (
+    _i, [_vp] * 6 + [_i, _f, _f, _i, _i] + [_vp] * 5 + [_i] * 5 + [_vp, _sz, _vp])
 _SIGNATURES["boxconv_integral_image_static_f32"] = (_i, [_vp, _vp, _i64, _i, _i, _vp])
 _SIGNATURES["boxconv_integral_image_half_f32"] = (_i, [_vp, _i, _vp, _i64, _i, _i, _vp, _sz, _vp])
 _SIGNATURES["boxconv_forward_fused_f32"] = (_i, [_vp] * 6 + [_i] + [_vp] * 3 + [_i] * 8 + [_vp])
@@ -302,34 +304,63 @@ def box_convolution_backward(input_integrated, x_min, x_max, y_min, y_max, grad_
     F = x_min.size(1)
     if tuple(grad_output.shape) != (B, C * F, h, w):
         raise RuntimeError("box_convolution: sizes of grad_output and input_integrated don't match")
-    sfx = _suffix(grad_output, "grad_output")
-    if input_integrated.device != grad_output.device or input_integrated.dtype != grad_output.dtype:
+    half = grad_output.dtype in _FUSED_OUTPUT and grad_output.dtype != torch.float32
+    if half:
+        # float16 / bfloat16 grad_output with the float32 integral image the forward saved: read
+        # directly by the kernels (grad_input comes back in the same half type, the parameter
+        # gradients in float32); rows too wide for that go through float32 copies
+        if input_integrated.dtype != torch.float32:
+            raise RuntimeError("box_convolution: half-precision grad_output needs a float32 "
+                               "input_integrated, got %s" % input_integrated.dtype)
+        if w > _MAX_WIDENING_WIDTH or (h + 1) * (w + 1) * 4 >= 2 ** 31:
+            grads = box_convolution_backward(
+                input_integrated, x_min, x_max, y_min, y_max, grad_output.float(), output,
+                reparametrization_h, reparametrization_w, normalize, exact, input_needs_grad,
+                x_min_needs_grad, x_max_needs_grad, y_min_needs_grad, y_max_needs_grad)
+            if grads[0] is not None:
+                grads[0] = grads[0].to(grad_output.dtype)
+            return grads
+        sfx = "half_f32"
+    else:
+        sfx = _suffix(grad_output, "grad_output")
+        if input_integrated.dtype != grad_output.dtype:
+            raise RuntimeError("box_convolution: grad_output and input_integrated differ in device or dtype")
+    if input_integrated.device != grad_output.device:
         raise RuntimeError("box_convolution: grad_output and input_integrated differ in device or dtype")
     lib = load()
     grad_output = grad_output.contiguous()
     input_integrated = input_integrated.contiguous()
-    x_min, x_max, y_min, y_max = _same_kind((x_min, x_max, y_min, y_max), grad_output, "grad_output")
-    dev, dt = grad_output.device, grad_output.dtype
+    x_min, x_max, y_min, y_max = _same_kind((x_min, x_max, y_min, y_max), input_integrated, "input_integrated")
+    dev, dt = grad_output.device, input_integrated.dtype
     needs_p = (x_min_needs_grad, x_max_needs_grad, y_min_needs_grad, y_max_needs_grad)
 
     grad_input = None
     if input_needs_grad:
-        grad_input = (torch.empty if F > 0 else torch.zeros)((B, C, h, w), dtype=dt, device=dev)
+        grad_input = (torch.empty if F > 0 else torch.zeros)((B, C, h, w), dtype=grad_output.dtype, device=dev)
     grads = [torch.empty((C, F), dtype=dt, device=dev) if n else None for n in needs_p]
     want_input = input_needs_grad and grad_input.numel() > 0 and F > 0
     want_params = any(needs_p) and C * F > 0
     if want_input or want_params:
         with _on_device(dev):
             nbytes = lib.boxconv_backward_workspace_bytes(
-                B, C, F, h, w, grad_output.element_size(), int(want_input), int(want_params))
+                B, C, F, h, w, input_integrated.element_size(), int(want_input), int(want_params))
             ws = _workspace(nbytes, dev)
-            rc = getattr(lib, "boxconv_backward_" + sfx)(
-                _ptr(input_integrated), _ptr(x_min), _ptr(x_max), _ptr(y_min), _ptr(y_max),
-                _ptr(grad_output), _ptr(output) if output is not None and output.numel() else None,
-                float(reparametrization_h), float(reparametrization_w), int(bool(normalize)),
-                int(bool(exact)), _ptr(grad_input) if want_input else None,
-                *[_ptr(g) if want_params else None for g in grads],
-                B, C, F, h, w, _ptr(ws), nbytes, _stream(dev))
+            if half:
+                rc = lib.boxconv_backward_half_f32(
+                    _ptr(input_integrated), _ptr(x_min), _ptr(x_max), _ptr(y_min), _ptr(y_max),
+                    _ptr(grad_output), _FUSED_OUTPUT[grad_output.dtype],
+                    float(reparametrization_h), float(reparametrization_w), int(bool(normalize)),
+                    int(bool(exact)), _ptr(grad_input) if want_input else None,
+                    *[_ptr(g) if want_params else None for g in grads],
+                    B, C, F, h, w, _ptr(ws), nbytes, _stream(dev))
+            else:
+                rc = getattr(lib, "boxconv_backward_" + sfx)(
+                    _ptr(input_integrated), _ptr(x_min), _ptr(x_max), _ptr(y_min), _ptr(y_max),
+                    _ptr(grad_output), _ptr(output) if output is not None and output.numel() else None,
+                    float(reparametrization_h), float(reparametrization_w), int(bool(normalize)),
+                    int(bool(exact)), _ptr(grad_input) if want_input else None,
+                    *[_ptr(g) if want_params else None for g in grads],
+                    B, C, F, h, w, _ptr(ws), nbytes, _stream(dev))
         _check(rc, "box_convolution_backward")
     return [grad_input] + grads
 
@@ -348,6 +379,16 @@ def clip_parameters(x_min, x_max, y_min, y_max, reparametrization_h, reparametri
                 or not p.is_contiguous()):
             raise RuntimeError("box_convolution: clip_parameters needs four contiguous tensors of "
                                "one shape, dtype and device")
+    if x_min.dtype in (torch.float16, torch.bfloat16):
+        # half-precision parameters (module.half()): clipped in float32, as the kernel's
+        # arithmetic is double anyway, and rounded back once
+        with torch.no_grad():
+            staged = [p.detach().float() for p in params]
+            clip_parameters(*staged, reparametrization_h, reparametrization_w, max_input_h,
+                            max_input_w, exact)
+            for p, s in zip(params, staged):
+                p.detach().copy_(s)
+        return
     sfx = _suffix(x_min, "parameters")
     n = x_min.numel()
     if n == 0:

@@ -52,7 +52,22 @@ class BoxConvolutionFunction(torch.autograd.Function):
         ctx.reparametrization_w = reparametrization_w
         ctx.exact = exact
 
-        if clip_to is not None:
+        ctx.param_dtype = x_min.dtype
+        if input.dtype in (torch.float16, torch.bfloat16):
+            # half-precision input: float32 integral image and sums, read and written by the
+            # kernels in the half type (no float32 copies of input, output or their gradients);
+            # the bounds are used in float32
+            if clip_to is not None:
+                _native.clip_parameters(x_min.detach(), x_max.detach(), y_min.detach(), y_max.detach(),
+                                        reparametrization_h, reparametrization_w, clip_to[0],
+                                        clip_to[1], exact)
+            x_min, x_max, y_min, y_max = reparametrize(
+                x_min.float(), x_max.float(), y_min.float(), y_max.float(),
+                reparametrization_h, reparametrization_w, inverse=True)
+            input_integrated = _native.integral_image(input)
+            output = _native.box_convolution_forward_fused(
+                input_integrated, x_min, x_max, y_min, y_max, normalize, exact, input.dtype)
+        elif clip_to is not None:
             input_integrated, output, (x_min, x_max, y_min, y_max) = _native.training_forward(
                 input, x_min.detach(), x_max.detach(), y_min.detach(), y_max.detach(),
                 reparametrization_h, reparametrization_w, clip_to[0], clip_to[1], normalize, exact)
@@ -76,5 +91,7 @@ class BoxConvolutionFunction(torch.autograd.Function):
             input_integrated, x_min, x_max, y_min, y_max, grad_output, None,
             ctx.reparametrization_h, ctx.reparametrization_w,
             ctx.normalize, ctx.exact, *ctx.needs_input_grad[:5])
+        if ctx.param_dtype != input_integrated.dtype:     # half-precision parameters
+            grads = [grads[0]] + [None if g is None else g.to(ctx.param_dtype) for g in grads[1:]]
         # no gradients for reparametrization_h, reparametrization_w, normalize, exact, clip_to
         return tuple(grads) + (None,) * 5

@@ -188,17 +188,16 @@ class BoxConv2d(torch.nn.Module):
 
     def _forward_half(self, input):
         """float16 / bfloat16 input (not offered by the reference's CPU path, and its CUDA path
-        would integrate in half precision): sums are always formed in float32. Without autograd
-        the kernel writes the half-precision output directly; when a gradient is needed the
-        float32 path runs between two casts."""
+        would integrate in half precision): the integral image and all sums are float32, and the
+        kernels read and write the half type directly, forward and backward (grad_output is
+        widened as it is loaded, grad_input rounded once in the store; parameter gradients are
+        float32, or the parameters' own half type after ``module.half()``)."""
         params = (self.x_min, self.x_max, self.y_min, self.y_max)
         if torch.is_grad_enabled() and (input.requires_grad or any(p.requires_grad for p in params)):
-            if self.training:
-                self._clip_parameters()
-            output = BoxConvolutionFunction.apply(
-                input.float(), *(p.float() for p in params),
-                self.reparametrization_h, self.reparametrization_w, self.normalize, self.exact)
-            return output.to(input.dtype)
+            clip_to = (self.max_input_h, self.max_input_w) if self.training else None
+            return BoxConvolutionFunction.apply(
+                input, *params, self.reparametrization_h, self.reparametrization_w,
+                self.normalize, self.exact, clip_to)
         if self.training:
             self._clip_parameters()
         return self.forward_fused(input)

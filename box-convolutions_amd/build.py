@@ -19,8 +19,24 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "build")
 LIB_PATH = os.path.join(HERE, "box_convolution", "libboxconv_hip.so")
 
-SOURCES = ["box_sampling.hip", "box_forward.hip", "integral_image.hip", "box_misc.hip", "boxconv_c_abi.hip"]
-HEADERS = ["boxconv_device.hpp", "boxconv_host.hpp", "box_sampling_common.hpp", os.path.join("..", "..", "include", "boxconv.h")]
+# (source, object name, extra defines). box_sampling_inst.hip holds the explicit instantiations of
+# the backward kernels and is compiled once per element-type pair and part, so that they build in
+# parallel (one translation unit with all of them takes six minutes).
+def _inst(tag, t, tg, part, same):
+    defs = ["-DBOXCONV_INST_T=" + t, "-DBOXCONV_INST_TG=" + tg, "-DBOXCONV_INST_PART=%d" % part]
+    if same:
+        defs.append("-DBOXCONV_INST_SAME_TYPE=1")
+    return ("box_sampling_inst.hip", "box_sampling_inst_%s_%d.o" % (tag, part), defs)
+
+
+SOURCES = [(s, s.replace(".hip", ".o"), []) for s in
+           ("box_sampling.hip", "box_forward.hip", "integral_image.hip", "box_misc.hip", "boxconv_c_abi.hip")]
+for _tag, _t, _tg in (("f32", "float", "float"), ("f64", "double", "double"),
+                      ("f16", "float", "f16_t"), ("bf16", "float", "bf16_t")):
+    for _part in (1, 2):
+        SOURCES.append(_inst(_tag, _t, _tg, _part, _t == _tg))
+HEADERS = ["boxconv_device.hpp", "boxconv_host.hpp", "box_sampling_common.hpp", "box_sampling_impl.hpp",
+           os.path.join("..", "..", "include", "boxconv.h")]
 
 ARCH = os.environ.get("BOXCONV_OFFLOAD_ARCH", "gfx950")
 # packed-fp32 instructions stay disabled: scalar float code only.
@@ -51,19 +67,20 @@ def build(force=False, verbose=True):
     header_paths = [os.path.normpath(os.path.join(CSRC, h)) for h in HEADERS] + [os.path.abspath(__file__)]
     jobs = []
     objs = []
-    for src in SOURCES:
+    for src, obj_name, defines in SOURCES:
         src_path = os.path.join(CSRC, src)
-        obj = os.path.join(OBJ_DIR, src.replace(".hip", ".o"))
+        obj = os.path.join(OBJ_DIR, obj_name)
         objs.append(obj)
         if force or _stale(obj, [src_path] + header_paths):
-            jobs.append([hipcc] + HIPCC_FLAGS + ["-c", src_path, "-o", obj])
+            jobs.append([hipcc] + HIPCC_FLAGS + defines + ["-c", src_path, "-o", obj])
 
     def run(cmd):
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.check_call(cmd)
 
-    with ThreadPoolExecutor(max_workers=min(5, max(1, len(jobs)))) as pool:
+    workers = min(os.cpu_count() or 4, 8, max(1, len(jobs)))
+    with ThreadPoolExecutor(max_workers=workers) as pool:
         list(pool.map(run, jobs))
 
     if force or jobs or _stale(LIB_PATH, objs):

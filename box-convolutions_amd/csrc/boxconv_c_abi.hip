@@ -8,6 +8,7 @@
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <type_traits>
 #include <utility>
 #include <vector>
 
@@ -289,10 +290,11 @@ int forward_impl(const T* integ, const T* x_min, const T* x_max, const T* y_min,
                       "forward launch");
 }
 
-template <class T>
+// TG: element type of grad_output and grad_input (T, or f16_t / bf16_t with T = float).
+template <class T, class TG>
 int backward_impl(const T* integ, const T* x_min, const T* x_max, const T* y_min, const T* y_max,
-                  const T* grad_output, const T* /*output*/, float reparam_h, float reparam_w,
-                  int normalize, int exact, T* grad_input, T* gx_min, T* gx_max, T* gy_min,
+                  const TG* grad_output, const T* /*output*/, float reparam_h, float reparam_w,
+                  int normalize, int exact, TG* grad_input, T* gx_min, T* gx_max, T* gy_min,
                   T* gy_max, int batch, int in_planes, int num_filters, int h, int w,
                   void* workspace, size_t workspace_bytes, void* stream) {
     if (int rc = check_dims(batch, in_planes, num_filters, h, w)) return rc;
@@ -310,6 +312,10 @@ int backward_impl(const T* integ, const T* x_min, const T* x_max, const T* y_min
                         reinterpret_cast<uintptr_t>(workspace) % 256 != 0))
         return fail(BOXCONV_E_WORKSPACE, "backward: workspace of %zu bytes (256-byte aligned) required, got %zu",
                     L.total, workspace_bytes);
+    constexpr bool kSameType = std::is_same<T, TG>::value;
+    if (!kSameType && !L.streaming)
+        return fail(BOXCONV_E_TOO_LARGE, "backward: half-precision grad_output is read directly for rows of at "
+                    "most %d columns; convert wider ones to float first", boxconv::kMaxRowStreamWidth);
 
     hipStream_t s = static_cast<hipStream_t>(stream);
     unsigned char* ws = static_cast<unsigned char*>(workspace);
@@ -334,17 +340,17 @@ int backward_impl(const T* integ, const T* x_min, const T* x_max, const T* y_min
         // one pass over grad_output: parameter sums + column workspace, then grad_input, whose
         // launch finishes the parameter gradients on the side
         const boxconv::StreamPlan sp = boxconv::plan_grad_output_stream(planes * num_filters, h, w, sizeof(T));
-        if (int rc = hip_result(boxconv::grad_output_stream_launch<T>(
+        if (int rc = hip_result(boxconv::grad_output_stream_launch<T, TG>(
                 integ, grad_output, prm, acc, L.acc_slots, gint, sp, d, exact != 0, s),
                 "grad_output streaming launch"))
             return rc;
         if (need_input)
-            if (int rc = hip_result(boxconv::grad_input_launch<T>(
+            if (int rc = hip_result(boxconv::grad_input_launch<T, TG>(
                     gint, sp.R, prm, grad_input, d, normalize != 0, exact != 0, s,
                     need_params ? &finish : nullptr, &finished),
                     "input-gradient launch"))
                 return rc;
-    } else {
+    } else if constexpr (kSameType) {
         // any width: gather kernels on true integral images
         if (need_params)
             if (int rc = hip_result(boxconv::grad_params_gather_launch<T>(
@@ -358,7 +364,7 @@ int backward_impl(const T* integ, const T* x_min, const T* x_max, const T* y_min
                     need_params && reverse_second_pass(), s),
                     "grad_output integral image launch"))
                 return rc;
-            if (int rc = hip_result(boxconv::grad_input_launch<T>(
+            if (int rc = hip_result(boxconv::grad_input_launch<T, T>(
                     gint, 0, prm, grad_input, d, normalize != 0, exact != 0, s),
                     "input-gradient launch"))
                 return rc;
@@ -566,7 +572,7 @@ int boxconv_backward_f32(const float* input_integrated, const float* x_min, cons
                          float* grad_x_min, float* grad_x_max, float* grad_y_min,
                          float* grad_y_max, int batch, int in_planes, int num_filters, int h,
                          int w, void* workspace, size_t workspace_bytes, void* stream) {
-    return backward_impl<float>(input_integrated, x_min, x_max, y_min, y_max, grad_output, output,
+    return backward_impl<float, float>(input_integrated, x_min, x_max, y_min, y_max, grad_output, output,
                                 reparametrization_h, reparametrization_w, normalize, exact,
                                 grad_input, grad_x_min, grad_x_max, grad_y_min, grad_y_max, batch,
                                 in_planes, num_filters, h, w, workspace, workspace_bytes, stream);
@@ -578,10 +584,33 @@ int boxconv_backward_f64(const double* input_integrated, const double* x_min, co
                          double* grad_x_min, double* grad_x_max, double* grad_y_min,
                          double* grad_y_max, int batch, int in_planes, int num_filters, int h,
                          int w, void* workspace, size_t workspace_bytes, void* stream) {
-    return backward_impl<double>(input_integrated, x_min, x_max, y_min, y_max, grad_output, output,
+    return backward_impl<double, double>(input_integrated, x_min, x_max, y_min, y_max, grad_output, output,
                                  reparametrization_h, reparametrization_w, normalize, exact,
                                  grad_input, grad_x_min, grad_x_max, grad_y_min, grad_y_max, batch,
                                  in_planes, num_filters, h, w, workspace, workspace_bytes, stream);
+}
+
+int boxconv_backward_half_f32(const float* input_integrated, const float* x_min, const float* x_max,
+                              const float* y_min, const float* y_max, const void* grad_output,
+                              int io_dtype, float reparametrization_h, float reparametrization_w,
+                              int normalize, int exact, void* grad_input, float* grad_x_min,
+                              float* grad_x_max, float* grad_y_min, float* grad_y_max, int batch,
+                              int in_planes, int num_filters, int h, int w, void* workspace,
+                              size_t workspace_bytes, void* stream) {
+    if (io_dtype == BOXCONV_F16)
+        return backward_impl<float, boxconv::f16_t>(
+            input_integrated, x_min, x_max, y_min, y_max, static_cast<const boxconv::f16_t*>(grad_output),
+            nullptr, reparametrization_h, reparametrization_w, normalize, exact,
+            static_cast<boxconv::f16_t*>(grad_input), grad_x_min, grad_x_max, grad_y_min, grad_y_max,
+            batch, in_planes, num_filters, h, w, workspace, workspace_bytes, stream);
+    if (io_dtype == BOXCONV_BF16)
+        return backward_impl<float, boxconv::bf16_t>(
+            input_integrated, x_min, x_max, y_min, y_max, static_cast<const boxconv::bf16_t*>(grad_output),
+            nullptr, reparametrization_h, reparametrization_w, normalize, exact,
+            static_cast<boxconv::bf16_t*>(grad_input), grad_x_min, grad_x_max, grad_y_min, grad_y_max,
+            batch, in_planes, num_filters, h, w, workspace, workspace_bytes, stream);
+    return fail(BOXCONV_E_INVALID_ARGUMENT, "backward: io_dtype %d is neither BOXCONV_F16 nor BOXCONV_BF16",
+                io_dtype);
 }
 
 int boxconv_clip_parameters_f32(float* x_min, float* x_max, float* y_min, float* y_max, int n,

@@ -91,8 +91,9 @@ inline int64_t column_workspace_plane(int h, int w) {
 // otherwise `gint` is the column workspace M in bands of band_rows rows, each restarting at zero.
 // finish (may be null): parameter-gradient sums that are complete when this launch starts; the
 // row kernel then finishes them on the side (no launch of its own) and *finish_done is set.
-template <class T>
-hipError_t grad_input_launch(const T* gint, int band_rows, BoxParams<T> prm, T* grad_in, Dims d,
+// TO: element type of grad_in: T, or with T = float and the column workspace also f16_t / bf16_t.
+template <class T, class TO>
+hipError_t grad_input_launch(const T* gint, int band_rows, BoxParams<T> prm, TO* grad_in, Dims d,
                              bool normalize, bool exact, hipStream_t stream,
                              const ParamFinish<T>* finish = nullptr, bool* finish_done = nullptr);
 
@@ -109,8 +110,9 @@ StreamPlan plan_grad_output_stream(int64_t planes_f, int h, int w, size_t elem_s
 // grad_params_begin, and workgroups add atomically. grad_params_finish takes the same two values.
 // column_workspace ([planes*F] planes of column_workspace_plane(h, w) elements) may be null: no
 // workspace for the gradient w.r.t. the input. At least one of the two must be given.
-template <class T>
-hipError_t grad_output_stream_launch(const T* integ, const T* grad_out, BoxParams<T> prm,
+// TG: element type of grad_out: T, or with T = float also f16_t / bf16_t (widened on load).
+template <class T, class TG>
+hipError_t grad_output_stream_launch(const T* integ, const TG* grad_out, BoxParams<T> prm,
                                      double* acc, int acc_slots, T* column_workspace,
                                      const StreamPlan& sp, Dims d, bool exact, hipStream_t stream);
 

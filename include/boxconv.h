@@ -192,6 +192,23 @@ int boxconv_backward_f64(const double* input_integrated, const double* x_min, co
                          double* grad_y_max, int batch, int in_planes, int num_filters, int h,
                          int w, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same backward pass with grad_output and grad_input in half precision (io_dtype: BOXCONV_F16
+ * or BOXCONV_BF16; both tensors of that type), everything else float: the float32 integral image
+ * of the input as saved by the forward, float32 box bounds, float32 parameter gradients, float32
+ * (and double) sums. The reference dispatches its CUDA kernels on half tensors
+ * (src/box_convolution_cuda_backward.cu:176,431, AT_DISPATCH_FLOATING_TYPES_AND_HALF) and then
+ * integrates grad_output in half precision; here its rows are widened to float as they are read
+ * and grad_input is rounded once, in the store. Same workspace as boxconv_backward_f32
+ * (boxconv_backward_workspace_bytes with elem_size 4). Rows of at most 2048 columns
+ * (BOXCONV_E_TOO_LARGE otherwise: convert to float first). */
+int boxconv_backward_half_f32(const float* input_integrated, const float* x_min, const float* x_max,
+                              const float* y_min, const float* y_max, const void* grad_output,
+                              int io_dtype, float reparametrization_h, float reparametrization_w,
+                              int normalize, int exact, void* grad_input, float* grad_x_min,
+                              float* grad_x_max, float* grad_y_min, float* grad_y_max, int batch,
+                              int in_planes, int num_filters, int h, int w, void* workspace,
+                              size_t workspace_bytes, void* stream);
+
 /* ---- clip parameters --------------------------------------------------------------------------
  * Replaces `clip_parameters(x_min, x_max, y_min, y_max, reparametrization_h, reparametrization_w,
  * max_input_h, max_input_w, exact) -> None`, reference src/box_convolution_interface.cpp:397-415

@@ -160,9 +160,19 @@ template <class T>
 struct BoxOfWorkgroup {
     T xmin, xmax, ymin, ymax;
 };
+// The box bounds are read through the constant address space: no kernel that samples boxes
+// writes them, and a load the compiler may treat as invariant becomes a scalar load when its
+// index is the same for the whole wave. Scalar loads are counted apart from the vector memory
+// loads, so fetching a box does not wait for (or hold up) the row loads in flight around it.
+template <class T>
+__device__ __forceinline__ T load_invariant(const T* p) {
+    typedef const T __attribute__((address_space(4))) * ConstPtr;
+    return *(ConstPtr)(p);
+}
 template <class T>
 __device__ __forceinline__ BoxOfWorkgroup<T> load_box(const BoxParams<T>& prm, int k_par) {
-    return {prm.xmin[k_par], prm.xmax[k_par], prm.ymin[k_par], prm.ymax[k_par]};
+    return {load_invariant(prm.xmin + k_par), load_invariant(prm.xmax + k_par),
+            load_invariant(prm.ymin + k_par), load_invariant(prm.ymax + k_par)};
 }
 
 using Flip0 = std::integral_constant<int, 0>;

@@ -18,6 +18,10 @@ After the --warmup steps the script keeps stepping, untimed, until the step time
 reference's CPU path timed on this host on a bounded sample of the same workload.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 1..5] [--no-cpu]
+
+Other modes (never the default): --graph replays a captured HIP graph of the step's native calls;
+--forward-only [--rounded] times the inference forward (eval mode, no autograd) on the forward's
+own algorithmic bytes; `config.mode` and `metric` say which one a line came from.
 """
 import argparse
 import json
@@ -118,6 +122,13 @@ def main():
                          "forward + backward through the C ABI) instead of the eager module step: "
                          "the same kernels without Python, autograd and launch latency, which bound "
                          "the small workloads")
+    ap.add_argument("--forward-only", action="store_true",
+                    help="time the inference forward instead of the training step: module.eval(), no "
+                         "autograd, out = module(x) (integral image + box sampling); `value` is then "
+                         "the forward's algorithmic bytes 4*(N_in + 2*N_int + N_out) per second")
+    ap.add_argument("--rounded", action="store_true",
+                    help="with --forward-only: module.exact = False, the reference's fast inference "
+                         "mode (box bounds rounded to whole pixels)")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
                     help="after the timed steps, run torch.neg on a float tensor of this many MiB "
                          "(reads MIB, writes MIB): the plain streaming kernel of known size that "
@@ -155,6 +166,19 @@ def main():
             p.grad = None
         out = module(x)
         out.backward(g)
+
+    if args.forward_only:
+        if args.graph:
+            sys.exit("bench.py: --forward-only and --graph are separate modes")
+        module.eval()
+        module.exact = not args.rounded
+        x.requires_grad_(False)
+        # the forward's own data flow: input -> integral image -> output
+        ab = dict(ab, alg=4 * (ab["n_in"] + 2 * ab["n_int"] + ab["n_out"]), io=4 * (ab["n_in"] + ab["n_out"]))
+
+        def eager_step():
+            with torch.no_grad():
+                module(x)
 
     step = eager_step
 
@@ -253,7 +277,8 @@ def main():
     achieved = bytes_per_launch / avg_launch_s / 1e9
 
     result = {
-        "metric": METRIC,
+        "metric": METRIC if not args.forward_only else
+                  "BoxConv2d inference forward ms/iter + effective HBM GB/s (% peak) at 2x16ch 512x1024 fp32",
         "value": round(value, 2),
         "unit": "GB/s",
         "n_gpus": 1,
@@ -273,7 +298,9 @@ def main():
             "workload": "%s: BoxConv2d(%d,%d,%d,%d) fwd+bwd, input [%d,%d,%d,%d], normalize, exact, "
                         "grads to input and 4 box parameters" % (
                             wl.name, wl.C, wl.F, wl.h, wl.w, wl.B, wl.C, wl.h, wl.w),
-            "mode": "captured HIP graph of the step's native calls" if args.graph else "eager module step",
+            "mode": ("inference forward, eval mode, %s box bounds" % ("rounded" if args.rounded else "exact")
+                     if args.forward_only else
+                     "captured HIP graph of the step's native calls" if args.graph else "eager module step"),
             "algorithmic_bytes_per_step": ab["alg"],
             "io_bytes_per_step": ab["io"],
             "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),

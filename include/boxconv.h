@@ -173,7 +173,9 @@ int boxconv_forward_fused_f32(const float* input_integrated, const float* x_min,
  * normalisation term sum(grad_output*output) is recomputed from input_integrated instead of
  * re-reading it.
  * workspace: boxconv_backward_workspace_bytes(...) bytes, 256-byte aligned. It receives the
- * integral image of grad_output (the bulk), per-band row vectors and the per-box accumulators. */
+ * backward's one intermediate per (plane, filter) - h+1 rows of grad_output filtered along the
+ * row and summed down the rows of a band (the bulk; for rows wider than 2048 columns a true
+ * integral image of grad_output instead) - and the per-box accumulators. */
 size_t boxconv_backward_workspace_bytes(int batch, int in_planes, int num_filters, int h, int w,
                                         int elem_size, int input_needs_grad,
                                         int params_need_grad);

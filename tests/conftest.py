@@ -15,6 +15,19 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs an AMD GPU (run with -m gpu on the MI355X box)")
 
 
+def pytest_terminal_summary(terminalreporter):
+    stats = getattr(sys.modules.get("test_gpu_parity"), "NOISE_STATS", None)
+    if stats and stats["comparisons"]:
+        line = ("assert_parity: %(comparisons)d tensor comparisons, %(needed_noise_term)d passed only with the "
+                "rounding-noise term or the sibling scale (%(of_those_reference_all_zero)d of those have an "
+                "all-zero reference tensor)" % stats)
+        terminalreporter.write_line(line)
+        path = os.environ.get("BOXCONV_PARITY_REPORT")
+        if path:
+            with open(path, "a") as fh:
+                fh.write(line + "\n")
+
+
 @pytest.fixture(scope="session")
 def oracle():
     from oracle import cpu_checker

@@ -210,10 +210,18 @@ __device__ __forceinline__ T gather_box(const T* __restrict__ plane, const BoxSp
 
 // ---------------------------------------------------------------------------------------------
 // Workgroup shapes the row kernels are compiled for: (threads, columns per lane).
-//   (64,1) widths up to 64; (128,1) up to 128; (256,1..4) up to 256..1024; (512,1..4) up to 512..2048.
-// Each kernel has a preferred size (measured at width 1024: 512 threads for forward and grad
-// input, 256 for the grad_output pass); rows too wide for 4 columns per lane at that size take
-// 512 threads, which bounds the register footprint and the length of the per-lane float
+//   (64,1) widths up to 64; (128,1) up to 128; (64,3..4) up to 256; (128,3..4) up to 512;
+//   (256,3..4) and (512,2..4) up to 2048.
+// Rows of up to 512 columns go to one or two waves with three or four columns per lane rather
+// than to four or eight waves with one or two: the per-wave part of a row pair (scan steps,
+// address and loop overhead, the waits of a workgroup-wide barrier) does not shrink with the
+// columns a lane holds, and small images are bound by exactly that (measured, grad_output pass at
+// 128 rows: 256 columns 55 -> 36 us, 384 columns 48 -> 30 us, 512 columns 48 -> 36 us; forward
+// 23 -> 20, 25 -> 15, 24 -> 22 us). Up to 128 columns one column per lane stays (two per lane on
+// one wave measured the same or slower).
+// Wider rows: each kernel has a preferred size (measured at width 1024: 512 threads for forward,
+// 256 for the grad_output pass); rows too wide for 4 columns per lane at that size take 512
+// threads, which bounds the register footprint and the length of the per-lane float
 // accumulation chains.
 struct RowConfig { int nt; int K; bool full; };
 inline int preferred_row_threads(const char* env_name, int fallback) {
@@ -225,6 +233,9 @@ inline RowConfig row_config(int w, int prefer) {
     RowConfig c;
     if (w <= 128) {
         c.nt = w <= 64 ? 64 : 128; c.K = 1;
+    } else if (w <= 512) {
+        c.nt = w <= 256 ? 64 : 128;
+        c.K = (w + c.nt - 1) / c.nt;                   // 3 or 4
     } else {
         // fewest column slots (K * threads) that cover the row; the preferred size wins ties
         const int other = prefer == 256 ? 512 : 256;
@@ -277,18 +288,22 @@ void finish_args(SampleArgs<T>& a, int64_t total) {
     a.per_xcd = (total + kXcds - 1) / kXcds;
 }
 
-#define BOXCONV_DISPATCH_K(KERNEL, NT, K, ...)                                       \
-    switch (K) {                                                                     \
-        case 1: KERNEL(NT, 1, __VA_ARGS__); break;                                   \
-        case 2: KERNEL(NT, 2, __VA_ARGS__); break;                                   \
-        case 3: KERNEL(NT, 3, __VA_ARGS__); break;                                   \
-        default: KERNEL(NT, 4, __VA_ARGS__); break;                                  \
-    }
+// (row_config never asks for a shape that is not listed here)
+#define BOXCONV_DISPATCH_K34(KERNEL, NT, K, ...)                                     \
+    if ((K) == 3) { KERNEL(NT, 3, __VA_ARGS__); } else { KERNEL(NT, 4, __VA_ARGS__); }
 #define BOXCONV_DISPATCH_SHAPE(KERNEL, RC, ...)                                      \
-    if ((RC).nt == 64)       { KERNEL(64, 1, __VA_ARGS__); }                         \
-    else if ((RC).nt == 128) { KERNEL(128, 1, __VA_ARGS__); }                        \
-    else if ((RC).nt == 256) { BOXCONV_DISPATCH_K(KERNEL, 256, (RC).K, __VA_ARGS__) } \
-    else                     { BOXCONV_DISPATCH_K(KERNEL, 512, (RC).K, __VA_ARGS__) }
+    if ((RC).nt == 64) {                                                             \
+        if ((RC).K == 1) { KERNEL(64, 1, __VA_ARGS__); }                             \
+        else { BOXCONV_DISPATCH_K34(KERNEL, 64, (RC).K, __VA_ARGS__) }               \
+    } else if ((RC).nt == 128) {                                                     \
+        if ((RC).K == 1) { KERNEL(128, 1, __VA_ARGS__); }                            \
+        else { BOXCONV_DISPATCH_K34(KERNEL, 128, (RC).K, __VA_ARGS__) }              \
+    } else if ((RC).nt == 256) {                                                     \
+        BOXCONV_DISPATCH_K34(KERNEL, 256, (RC).K, __VA_ARGS__)                       \
+    } else {                                                                         \
+        if ((RC).K == 2) { KERNEL(512, 2, __VA_ARGS__); }                            \
+        else { BOXCONV_DISPATCH_K34(KERNEL, 512, (RC).K, __VA_ARGS__) }              \
+    }
 #define BOXCONV_DISPATCH_SHAPE_EXACT_FULL(KERNEL, RC, EXACT)                         \
     if (EXACT) {                                                                     \
         if ((RC).full) { BOXCONV_DISPATCH_SHAPE(KERNEL, RC, true, true) }            \

@@ -170,6 +170,10 @@ SMALL_CASES = [
     (1, 2, 2, 12, 128), (1, 1, 3, 35, 100),          # two waves per row, full and partial
     # the same sharing of filters for rows of two and four waves
     (1, 2, 5, 20, 100), (1, 1, 6, 12, 128), (1, 1, 4, 20, 200), (1, 2, 7, 9, 256),
+    # one and two waves with three or four columns per lane (rows of 129 to 512 columns), rows that
+    # fill the workgroup's column slots exactly and rows that do not
+    (1, 2, 2, 14, 192), (1, 1, 2, 13, 150), (2, 1, 2, 10, 384), (1, 1, 3, 9, 512), (1, 1, 2, 11, 500),
+    (1, 2, 1, 16, 257),
 ]
 
 
@@ -197,7 +201,7 @@ def test_forward_backward_small(hip, oracle, B, C, F, h, w, kind, dtype):
 
 
 @pytest.mark.parametrize("kind", ["inside", "hanging", "inverted"])
-@pytest.mark.parametrize("h,w", [(150, 90), (257, 256), (97, 520)])
+@pytest.mark.parametrize("h,w", [(150, 90), (257, 256), (97, 520), (140, 400), (131, 170)])
 def test_backward_across_row_bands(hip, oracle, h, w, kind):
     """Images tall enough that the backward pass cuts grad_output into several row bands, with
     boxes whose top and bottom rows fall into different bands; 'inverted' boxes have min > max

@@ -346,7 +346,7 @@ __device__ __forceinline__ void block_accumulate5(const double (&v)[5], double* 
 //
 // LDS: [2 buffers][K*nt + 8] RowPair grad_output rows (4 zero pairs in front, >= 4 behind),
 //      [2][2][4] X[w] triples, [K*nt] tail weights, [K*nt] RowPair W rows, [8*5] doubles,
-//      [2][8] wave totals, [2][8] wave tails.
+//      [2][2][8] wave totals, [2][2][8] wave tails (one set per LDS buffer).
 constexpr int kGPad = 4;
 
 template <class T>
@@ -356,8 +356,8 @@ struct StreamLds {
     T* xw;              // [2][2][4]
     T* delta;           // [K*nt] tail weight of pixel column j
     double* red;        // [5 * kMaxRowWaves]
-    T* wave_tot;        // [2][kMaxRowWaves]
-    T* wave_tail;       // [2][kMaxRowWaves]
+    T* wave_tot;        // [2 buffers][2 rows][kMaxRowWaves]
+    T* wave_tail;       // [2 buffers][2 rows][kMaxRowWaves]
     int glen;
 };
 
@@ -367,7 +367,7 @@ __host__ __device__ constexpr size_t stream_lds_elems(int K, int nt) {
 }
 __host__ __device__ constexpr size_t stream_lds_bytes(int K, int nt, size_t elem) {
     const size_t b = (stream_lds_elems(K, nt) * elem + 15) / 16 * 16;
-    return b + (4 * kMaxRowWaves + 5 * kMaxRowWaves) * sizeof(double);
+    return b + (8 * kMaxRowWaves + 5 * kMaxRowWaves) * sizeof(double);
 }
 
 // `lds_base`: the kernel's own statically sized array, so that every LDS address is a lane
@@ -384,7 +384,7 @@ __device__ __forceinline__ StreamLds<T> carve_stream_lds(unsigned char* lds_base
     const size_t b = (stream_lds_elems(K, nt) * sizeof(T) + 15) / 16 * 16;
     l.red = reinterpret_cast<double*>(lds_base + b);
     l.wave_tot = reinterpret_cast<T*>(l.red + 5 * kMaxRowWaves);
-    l.wave_tail = reinterpret_cast<T*>(l.red + 7 * kMaxRowWaves);
+    l.wave_tail = reinterpret_cast<T*>(l.red + 9 * kMaxRowWaves);
     return l;
 }
 
@@ -529,6 +529,53 @@ grad_output_stream_kernel(SampleArgs<T> a) {
     // sliding rows rotate by renaming instead of moves.
     // OWN_W: the rare box whose mirrored split differs (see above); a tag as well, so that the
     // common case carries none of its code.
+    // Rows i, i+1 of grad_output (registers GA, GB) into LDS buffer FL, with the wave's share of
+    // the tails and, from the owner of column w, the X[w] triples of the same pair. A macro, not
+    // a lambda: arrays handed through a second closure end up in scratch memory.
+#define BOXCONV_PUBLISH_PAIR(FL, GA, GB, TA, T0, T1, BC, B1, B2, TL0, TL1)                          \
+    {                                                                                               \
+        RowPair<T>* Gp = lds.grow + ((FL) ? glen : 0);                                              \
+        T* Xp0 = lds.xw + (FL) * 8;                                                                 \
+        T* Xp1 = Xp0 + 4;                                                                           \
+        TL0 = T(0); TL1 = T(0);                                                                     \
+        _Pragma("unroll")                                                                           \
+        for (int k = 0; k < K; ++k) {                                                               \
+            if (slot_valid<T, 64, FULL>(q1, k, row_bytes))                                          \
+                *at_bytes(Gp + kGPad - 1 + 64 * k, 2 * q1) = RowPair<T>{GA[k], GB[k]};              \
+            {                                                                                       \
+                const T dlt = *at_bytes(lds.delta - 1 + 64 * k, q1);                                \
+                TL0 += dlt * GA[k];                                                                 \
+                TL1 += dlt * GB[k];                                                                 \
+            }                                                                                       \
+            if (PARAMS && (FULL ? (k == K - 1 && tid == nt - 1) : (q1 + slot_bytes<T, 64>(k) == row_bytes))) { \
+                const T dt0 = T0[k] - TA[k], db0 = B1[k] - BC[k];                                   \
+                const T dt1 = T1[k] - T0[k], db1 = B2[k] - B1[k];                                   \
+                T v0 = BC[k] - T0[k], v1 = B1[k] - T1[k];                                           \
+                if (EXACT) {                                                                        \
+                    v0 += s.fxhi * db0; v0 += s.fxlo * dt0;                                         \
+                    v1 += s.fxhi * db1; v1 += s.fxlo * dt1;                                         \
+                }                                                                                   \
+                Xp0[0] = v0; Xp0[1] = dt0; Xp0[2] = db0;                                            \
+                Xp1[0] = v1; Xp1[1] = dt1; Xp1[2] = db1;                                            \
+            }                                                                                       \
+        }                                                                                           \
+    }
+
+    // MERGED (workgroups of up to four waves): one workgroup barrier per row pair. The rows of the
+    // NEXT pair go into the other LDS buffer before the barrier that publishes this pair's wave
+    // totals, so the same barrier makes both visible. (The other buffer was last read for the
+    // pair before this one, i.e. before the previous barrier.) The price: the next pair's loads
+    // must have arrived by that barrier instead of by the end of the iteration; with eight waves
+    // and one workgroup per CU that costs more than the barrier (1024 x 2048, 512 threads: 1.39
+    // against 1.07 ms), so those keep a barrier of their own for the rows.
+    // tl0, tl1: this wave's tails of the pair whose rows are in LDS.
+    constexpr bool MERGED = NT <= 256;
+    T tl0 = T(0), tl1 = T(0);
+    if (MERGED) {
+        BOXCONV_PUBLISH_PAIR(0, g0, g1, ta, t0, t1, bc, b1, b2, tl0, tl1)
+        __syncthreads();
+    }
+
     auto row_pair = [&](int i, auto prefetch_tag, auto flip_tag, auto own_w_tag) {
         constexpr bool PREFETCH = decltype(prefetch_tag)::value;
         constexpr int FLIP = decltype(flip_tag)::value;
@@ -544,30 +591,14 @@ grad_output_stream_kernel(SampleArgs<T> a) {
         RowPair<T>* G = lds.grow + (FLIP ? glen : 0);
         T* X0 = lds.xw + FLIP * 8;
         T* X1 = X0 + 4;
-
-        T tail0 = T(0), tail1 = T(0);
-#pragma unroll
-        for (int k = 0; k < K; ++k) {
-            if (slot_valid<T, 64, FULL>(q1, k, row_bytes))
-                *at_bytes(G + kGPad - 1 + 64 * k, 2 * q1) = RowPair<T>{g0[k], g1[k]};
-            {
-                const T dlt = *at_bytes(lds.delta - 1 + 64 * k, q1);
-                tail0 += dlt * g0[k];
-                tail1 += dlt * g1[k];
-            }
-            if (PARAMS && (FULL ? (k == K - 1 && tid == nt - 1) : (q1 + slot_bytes<T, 64>(k) == row_bytes))) {   // owner of column q = w
-                const T dt0 = t0[k] - ta[k], db0 = b1[k] - bc[k];
-                const T dt1 = t1[k] - t0[k], db1 = b2[k] - b1[k];
-                T v0 = bc[k] - t0[k], v1 = b1[k] - t1[k];
-                if (EXACT) {
-                    v0 += s.fxhi * db0; v0 += s.fxlo * dt0;
-                    v1 += s.fxhi * db1; v1 += s.fxlo * dt1;
-                }
-                X0[0] = v0; X0[1] = dt0; X0[2] = db0;
-                X1[0] = v1; X1[1] = dt1; X1[2] = db1;
-            }
+        T* wtot = lds.wave_tot + FLIP * 2 * kMaxRowWaves;
+        T* wtail = lds.wave_tail + FLIP * 2 * kMaxRowWaves;
+        if (!MERGED) {
+            BOXCONV_PUBLISH_PAIR(FLIP, g0, g1, ta, t0, t1, bc, b1, b2, tl0, tl1)
+            __syncthreads();                                                 // rows are in LDS
         }
-        __syncthreads();                                                     // rows are in LDS
+        T tail0 = tl0, tail1 = tl1;
+        T tn0 = T(0), tn1 = T(0);                       // MERGED: tails of the next pair
 
         // W(i)[q], W(i+1)[q] of the lane's column slots
         T wq0[K], wq1[K];
@@ -679,11 +710,12 @@ grad_output_stream_kernel(SampleArgs<T> a) {
                 base0 = run0 - inc0;                                         // -(lanes to the left)
                 base1 = run1 - inc1;
                 if (lane == 63) {
-                    lds.wave_tot[wave] = inc0; lds.wave_tot[kMaxRowWaves + wave] = inc1;
-                    lds.wave_tail[wave] = wt0; lds.wave_tail[kMaxRowWaves + wave] = wt1;
+                    wtot[wave] = inc0; wtot[kMaxRowWaves + wave] = inc1;
+                    wtail[wave] = wt0; wtail[kMaxRowWaves + wave] = wt1;
                 }
             }
-            __syncthreads();                                                 // wave totals visible
+            if (MERGED && PREFETCH) BOXCONV_PUBLISH_PAIR(FLIP ^ 1, m0, m1, t1, n0, n1, b2, n2, n3, tn0, tn1)
+            __syncthreads();                         // wave totals (and the next pair's rows) visible
             {
                 // A[c] = (sum of all W + tail) - (W of the columns before c)
                 //      = totals of this wave and the waves to the right + all tails - lanes to
@@ -691,11 +723,11 @@ grad_output_stream_kernel(SampleArgs<T> a) {
                 // `wave` is scalar, so the conditions below are scalar.
 #pragma unroll
                 for (int wv = 0; wv < NT / 64; ++wv) {
-                    base0 += lds.wave_tail[wv];
-                    base1 += lds.wave_tail[kMaxRowWaves + wv];
+                    base0 += wtail[wv];
+                    base1 += wtail[kMaxRowWaves + wv];
                     if (wv >= wave) {
-                        base0 += lds.wave_tot[wv];
-                        base1 += lds.wave_tot[kMaxRowWaves + wv];
+                        base0 += wtot[wv];
+                        base1 += wtot[kMaxRowWaves + wv];
                     }
                 }
                 // M rows i+1, i+2: a wave stores one contiguous run of 64*K elements per row. The
@@ -724,7 +756,13 @@ grad_output_stream_kernel(SampleArgs<T> a) {
             }
         }
 
+        if (!SCAN && MERGED) {
+            if (PREFETCH) BOXCONV_PUBLISH_PAIR(FLIP ^ 1, m0, m1, t1, n0, n1, b2, n2, n3, tn0, tn1)
+            __syncthreads();                                                 // the next pair's rows visible
+        }
+
         if (PREFETCH) {
+            if (MERGED) { tl0 = tn0; tl1 = tn1; }
 #pragma unroll
             for (int k = 0; k < K; ++k) {
                 if (PARAMS) {
@@ -757,6 +795,7 @@ grad_output_stream_kernel(SampleArgs<T> a) {
     if (own_w) BOXCONV_ALL_PAIRS(std::true_type)
     else BOXCONV_ALL_PAIRS(std::false_type)
 #undef BOXCONV_ALL_PAIRS
+#undef BOXCONV_PUBLISH_PAIR
 
     if (PARAMS) {
         __syncthreads();

@@ -67,3 +67,40 @@ def test_single_plane_above_two_gib(hip):
     for got_t, want_v, name in zip(grads[1:], (want_xmin, want_xmax, want_ymin, want_ymax),
                                    ("x_min", "x_max", "y_min", "y_max")):
         assert abs(got_t.item() - want_v) <= 1e-3 * abs(want_v) + noise, (name, got_t.item(), want_v)
+
+
+def _shifted(t, elems=1):
+    """A contiguous copy of t whose first element sits `elems` elements past an aligned address."""
+    flat = torch.empty(t.numel() + elems, device=t.device, dtype=t.dtype)
+    out = flat[elems:].view_as(t)
+    out.copy_(t)
+    assert out.data_ptr() % 16 != 0 and out.is_contiguous()
+    return out
+
+
+@pytest.mark.parametrize("shape", [(2, 2, 3, 40, 256), (1, 2, 2, 33, 1024), (1, 1, 2, 70, 384), (2, 1, 4, 24, 64)])
+def test_tensors_that_are_not_16_byte_aligned(hip, shape):
+    """Inputs whose data pointers are only 4-byte aligned (views into a larger buffer): the vector
+    loads must not be used on them. Same bits as with aligned tensors for the integral image and
+    the forward pass; the backward is compared to a tight tolerance (its column workspace is
+    private and aligned either way, only the loads of grad_output and of the integral differ)."""
+    B, C, F, h, w = shape
+    gen = torch.Generator(device="cuda").manual_seed(11)
+    x = torch.randn(B, C, h, w, device="cuda", generator=gen)
+    g = torch.randn(B, C * F, h, w, device="cuda", generator=gen)
+    lo = -torch.rand(C, F, device="cuda", generator=gen) * 9 - 0.3
+    hi = torch.rand(C, F, device="cuda", generator=gen) * 9 + 0.3
+    boxes = (lo, hi, lo * 1.5, hi * 0.7)
+
+    integ = hip.integral_image(x)
+    integ_s = hip.integral_image(_shifted(x))
+    assert torch.equal(integ, integ_s)
+    out = hip.box_convolution_forward(integ, *boxes, True, True)
+    out_s = hip.box_convolution_forward(_shifted(integ), *boxes, True, True)
+    assert torch.equal(out, out_s)
+    ref = hip.box_convolution_backward(integ, *boxes, g, None, 2.0, 3.0, True, True, True, True, True, True, True)
+    got = hip.box_convolution_backward(_shifted(integ), *boxes, _shifted(g), None, 2.0, 3.0, True, True,
+                                       True, True, True, True, True)
+    torch.cuda.synchronize()
+    for a, b in zip(ref, got):
+        assert torch.allclose(a, b, rtol=1e-6, atol=1e-6 * float(a.abs().max()))

@@ -139,6 +139,7 @@ def _workspace(nbytes, device):
 
 
 _MAX_WIDENING_WIDTH = 2048     # widest row boxconv_integral_image_half_f32 reads directly
+_MAX_STREAM_WIDTH = 4096       # widest row boxconv_backward_half_f32 reads directly
 
 
 def integral_image(input):
@@ -312,7 +313,7 @@ def box_convolution_backward(input_integrated, x_min, x_max, y_min, y_max, grad_
         if input_integrated.dtype != torch.float32:
             raise RuntimeError("box_convolution: half-precision grad_output needs a float32 "
                                "input_integrated, got %s" % input_integrated.dtype)
-        if w > _MAX_WIDENING_WIDTH or (h + 1) * (w + 1) * 4 >= 2 ** 31:
+        if w > _MAX_STREAM_WIDTH or (h + 1) * (w + 1) * 4 >= 2 ** 31:
             grads = box_convolution_backward(
                 input_integrated, x_min, x_max, y_min, y_max, grad_output.float(), output,
                 reparametrization_h, reparametrization_w, normalize, exact, input_needs_grad,

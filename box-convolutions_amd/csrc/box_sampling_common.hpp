@@ -16,11 +16,11 @@ namespace {
 
 extern __shared__ __align__(16) unsigned char smem_raw[];
 
-// Largest workgroup of the row-streaming kernels (8 waves). A wide row is spread over more lanes
-// rather than over more than 4 columns per lane: per-lane state (sliding rows, prefetched rows,
-// accumulators) scales with the columns per lane, and these kernels hide HBM latency with
-// occupancy.
-constexpr int kMaxRowThreads = 512;
+// Largest workgroup of the row-streaming kernels (16 waves, for rows of 2049 to 4096 columns;
+// up to 2048 columns at most 8). A wide row is spread over more lanes rather than over more than
+// 4 columns per lane: per-lane state (sliding rows, prefetched rows, accumulators) scales with the
+// columns per lane, and these kernels hide HBM latency with occupancy.
+constexpr int kMaxRowThreads = 1024;
 constexpr int kMaxRowWaves = kMaxRowThreads / 64;
 
 template <class T>
@@ -211,7 +211,9 @@ __device__ __forceinline__ T gather_box(const T* __restrict__ plane, const BoxSp
 // ---------------------------------------------------------------------------------------------
 // Workgroup shapes the row kernels are compiled for: (threads, columns per lane).
 //   (64,1) widths up to 64; (128,1) up to 128; (64,3..4) up to 256; (128,3..4) up to 512;
-//   (256,3..4) and (512,2..4) up to 2048.
+//   (256,3..4) and (512,2..4) up to 2048; (1024,3..4) up to 4096 (float32 only; the fused
+//   grad_output pass does not fit the 128 registers a lane gets at 16 waves, so there its two
+//   halves run as two launches).
 // Rows of up to 512 columns go to one or two waves with three or four columns per lane rather
 // than to four or eight waves with one or two: the per-wave part of a row pair (scan steps,
 // address and loop overhead, the waits of a workgroup-wide barrier) does not shrink with the
@@ -236,6 +238,9 @@ inline RowConfig row_config(int w, int prefer) {
     } else if (w <= 512) {
         c.nt = w <= 256 ? 64 : 128;
         c.K = (w + c.nt - 1) / c.nt;                   // 3 or 4
+    } else if (w > 2048) {
+        c.nt = 1024;
+        c.K = std::min(std::max((w + 1023) / 1024, 3), 4);
     } else {
         // fewest column slots (K * threads) that cover the row; the preferred size wins ties
         const int other = prefer == 256 ? 512 : 256;
@@ -251,7 +256,9 @@ inline RowConfig row_config(int w, int prefer) {
 // The row kernels address a plane with 32-bit byte offsets and hold a full row per workgroup.
 inline bool row_kernels_apply(int h, int w, size_t elem_size) {
     const uint64_t plane_bytes = (static_cast<uint64_t>(h) + 1) * (static_cast<uint64_t>(w) + 1) * elem_size;
-    return w <= kMaxRowStreamWidth && plane_bytes < (1ull << 31) && !force_gather_kernels();
+    // rows of more than 2048 columns: float32 (and 16-bit) elements only
+    const int max_w = elem_size <= 4 ? kMaxRowStreamWidth : kMaxRowStreamWidth / 2;
+    return w <= max_w && plane_bytes < (1ull << 31) && !force_gather_kernels();
 }
 
 // The grad-input kernel runs right after the pass that wrote the integral of grad_output; the
@@ -300,10 +307,16 @@ void finish_args(SampleArgs<T>& a, int64_t total) {
         else { BOXCONV_DISPATCH_K34(KERNEL, 128, (RC).K, __VA_ARGS__) }              \
     } else if ((RC).nt == 256) {                                                     \
         BOXCONV_DISPATCH_K34(KERNEL, 256, (RC).K, __VA_ARGS__)                       \
-    } else {                                                                         \
+    } else if ((RC).nt == 512) {                                                     \
         if ((RC).K == 2) { KERNEL(512, 2, __VA_ARGS__); }                            \
         else { BOXCONV_DISPATCH_K34(KERNEL, 512, (RC).K, __VA_ARGS__) }              \
+    } else {                                                                         \
+        BOXCONV_DISPATCH_WIDE(KERNEL, (RC).K, __VA_ARGS__)                           \
     }
+// 1024 threads: instantiated for 4-byte arithmetic only (`T` is the launch function's type)
+#define BOXCONV_DISPATCH_WIDE(KERNEL, K, ...)                                        \
+    if constexpr (sizeof(T) <= 4) { BOXCONV_DISPATCH_K34(KERNEL, 1024, K, __VA_ARGS__) } \
+    else { return hipErrorInvalidValue; }
 #define BOXCONV_DISPATCH_SHAPE_EXACT_FULL(KERNEL, RC, EXACT)                         \
     if (EXACT) {                                                                     \
         if ((RC).full) { BOXCONV_DISPATCH_SHAPE(KERNEL, RC, true, true) }            \

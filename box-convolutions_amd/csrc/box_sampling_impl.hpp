@@ -394,14 +394,22 @@ __device__ __forceinline__ StreamLds<T> carve_stream_lds(unsigned char* lds_base
 // instead of spilling.
 // TG: element type of grad_output (T, or a 16-bit type when T is float: a.grad_out then points at
 // elements of TG, widened to float as they are loaded).
-template <class T, class TG, int NT, int K, bool EXACT, bool FULL, bool PARAMS, bool SCAN>
+// S > 1 (parameter sums only, rows wider than one workgroup's column slots): S workgroups share a
+// band. Each owns NT*K of the row's columns q (its integral rows, its share of the five sums, a
+// slot of its own for them) but places the WHOLE row pair of grad_output in LDS, since the taps
+// of a column can fall anywhere in the row. The terms that belong to column w (the tails, the
+// two single taps) are added by the workgroup that owns that column, over all pixel columns.
+template <class T, class TG, int NT, int K, bool EXACT, bool FULL, bool PARAMS, bool SCAN, int S = 1>
 __global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu((K >= 3 && PARAMS && SCAN) ? 2 : 1, (K >= 3 && PARAMS && SCAN) ? 2 : 8)))
 grad_output_stream_kernel(SampleArgs<T> a) {
+    static_assert(S == 1 || (S == 2 && PARAMS && !SCAN && !FULL), "column parts: parameter sums only, two parts");
     const unsigned vid = xcd_contiguous_id(a.per_xcd);
     if (vid >= a.total) return;                      // whole workgroup leaves together
     const unsigned nbands = a.nb, nfilt = a.F;
-    const int band = static_cast<int>(vid % nbands);
-    const unsigned pf32 = vid / nbands;
+    const int part = S > 1 ? static_cast<int>(vid % S) : 0;
+    const unsigned vband = S > 1 ? vid / S : vid;
+    const int band = static_cast<int>(vband % nbands);
+    const unsigned pf32 = vband / nbands;
     const int f = static_cast<int>(pf32 % nfilt);
     const int64_t pf = pf32, p = pf32 / nfilt;
     const int k_par = static_cast<int>(static_cast<unsigned>(a.plane0 + p) % static_cast<unsigned>(a.C)) * a.F + f;
@@ -428,8 +436,8 @@ grad_output_stream_kernel(SampleArgs<T> a) {
     const bool keep_in_cache =
         static_cast<uint64_t>(from_end) * a.R * mpitch * sizeof(T) < static_cast<uint64_t>(a.keep_tail);
     const Rows<T, FULL> mout(mrows, mpitch, static_cast<int>(mpitch), h + 1);
-    __shared__ __align__(16) unsigned char lds_bytes[stream_lds_bytes(K, NT, sizeof(T))];
-    const StreamLds<T> lds = carve_stream_lds<T>(lds_bytes, K, nt);
+    __shared__ __align__(16) unsigned char lds_bytes[stream_lds_bytes(K, NT * S, sizeof(T))];
+    const StreamLds<T> lds = carve_stream_lds<T>(lds_bytes, K, nt * S);
     const int glen = lds.glen;
 
     const int i0 = band * a.R;
@@ -444,21 +452,33 @@ grad_output_stream_kernel(SampleArgs<T> a) {
     // pair (K consecutive ones, K*tid ..) belong to the same wave, so that the change of ownership
     // goes through LDS without a workgroup barrier.
     constexpr int CH = 64 * K;
-    const int jbase = wave * CH + lane;
+    const int jbase = part * (NT * K) + wave * CH + lane;
     const int q1 = (1 + jbase) * static_cast<int>(sizeof(T));
     const int q1g = (1 + jbase) * static_cast<int>(sizeof(TG));     // the same slots in a row of TG
+    // S > 1: the columns of the other part, which this workgroup only copies into LDS
+    const int jother = (1 - part) * (NT * K) + wave * CH + lane;
+    const int q1o = (1 + jother) * static_cast<int>(sizeof(T));
+    const int q1og = (1 + jother) * static_cast<int>(sizeof(TG));
+    const bool owns_w = part == S - 1;               // the part with the row's last column
     T g0[K], g1[K];
-    auto load_g = [&](int i, T (&dst)[K]) {
+    T go0[K] = {}, go1[K] = {};
+    auto load_g_at = [&](int i, int qg, T (&dst)[K]) {
         const RowRef r = grows.row(min(i, h - 1), i < i1);     // rows past the band read as zeros
 #pragma unroll
-        for (int k = 0; k < K; ++k) dst[k] = static_cast<T>(widen(load_slot<TG, 64, kCacheStream>(r, q1g, k)));
+        for (int k = 0; k < K; ++k) dst[k] = static_cast<T>(widen(load_slot<TG, 64, kCacheStream>(r, qg, k)));
     };
+    auto load_g = [&](int i, T (&dst)[K]) { load_g_at(i, q1g, dst); };
     load_g(i0, g0);
     load_g(i0 + 1, g1);
+    if (S > 1) {
+        load_g_at(i0, q1og, go0);
+        load_g_at(i0 + 1, q1og, go1);
+    }
 
     // clear the grad_output rows once: pads and the columns beyond w stay zero for good; the
     // same for the W rows
     for (int e = tid; e < 2 * glen; e += nt) lds.grow[e] = RowPair<T>{T(0), T(0)};
+    if (S > 1 && tid < 16) lds.xw[tid] = T(0);
     if (SCAN) {
         for (int e = tid; e < K * nt; e += nt) lds.wrow[e] = RowPair<T>{T(0), T(0)};
         if (band == 0)
@@ -495,6 +515,10 @@ grad_output_stream_kernel(SampleArgs<T> a) {
         const T d = (FULL || j < w) ? tail_weight(j, s.ylo, s.yhi, s.fylo, s.fyhi) : T(0);
         lds.delta[j] = d;
         wave_has_tail = wave_has_tail || d != T(0);
+        if (S > 1) {
+            const int jo = jother + 64 * k;
+            lds.delta[jo] = jo < w ? tail_weight(jo, s.ylo, s.yhi, s.fylo, s.fyhi) : T(0);
+        }
     }
     if (PARAMS) {
         const int j_ymax = w - s.yhi, j_ymin = w - s.ylo + 1;
@@ -532,7 +556,7 @@ grad_output_stream_kernel(SampleArgs<T> a) {
     // Rows i, i+1 of grad_output (registers GA, GB) into LDS buffer FL, with the wave's share of
     // the tails and, from the owner of column w, the X[w] triples of the same pair. A macro, not
     // a lambda: arrays handed through a second closure end up in scratch memory.
-#define BOXCONV_PUBLISH_PAIR(FL, GA, GB, TA, T0, T1, BC, B1, B2, TL0, TL1)                          \
+#define BOXCONV_PUBLISH_PAIR(FL, GA, GB, GOA, GOB, TA, T0, T1, BC, B1, B2, TL0, TL1)                \
     {                                                                                               \
         RowPair<T>* Gp = lds.grow + ((FL) ? glen : 0);                                              \
         T* Xp0 = lds.xw + (FL) * 8;                                                                 \
@@ -542,10 +566,17 @@ grad_output_stream_kernel(SampleArgs<T> a) {
         for (int k = 0; k < K; ++k) {                                                               \
             if (slot_valid<T, 64, FULL>(q1, k, row_bytes))                                          \
                 *at_bytes(Gp + kGPad - 1 + 64 * k, 2 * q1) = RowPair<T>{GA[k], GB[k]};              \
-            {                                                                                       \
+            if (S > 1 && slot_valid<T, 64, false>(q1o, k, row_bytes))                               \
+                *at_bytes(Gp + kGPad - 1 + 64 * k, 2 * q1o) = RowPair<T>{GOA[k], GOB[k]};           \
+            if (S == 1 || owns_w) {                                                                 \
                 const T dlt = *at_bytes(lds.delta - 1 + 64 * k, q1);                                \
                 TL0 += dlt * GA[k];                                                                 \
                 TL1 += dlt * GB[k];                                                                 \
+                if (S > 1) {                                                                        \
+                    const T dlo = *at_bytes(lds.delta - 1 + 64 * k, q1o);                           \
+                    TL0 += dlo * GOA[k];                                                            \
+                    TL1 += dlo * GOB[k];                                                            \
+                }                                                                                   \
             }                                                                                       \
             if (PARAMS && (FULL ? (k == K - 1 && tid == nt - 1) : (q1 + slot_bytes<T, 64>(k) == row_bytes))) { \
                 const T dt0 = T0[k] - TA[k], db0 = B1[k] - BC[k];                                   \
@@ -572,7 +603,7 @@ grad_output_stream_kernel(SampleArgs<T> a) {
     constexpr bool MERGED = NT <= 256;
     T tl0 = T(0), tl1 = T(0);
     if (MERGED) {
-        BOXCONV_PUBLISH_PAIR(0, g0, g1, ta, t0, t1, bc, b1, b2, tl0, tl1)
+        BOXCONV_PUBLISH_PAIR(0, g0, g1, go0, go1, ta, t0, t1, bc, b1, b2, tl0, tl1)
         __syncthreads();
     }
 
@@ -581,11 +612,16 @@ grad_output_stream_kernel(SampleArgs<T> a) {
         constexpr int FLIP = decltype(flip_tag)::value;
         constexpr bool OWN_W = decltype(own_w_tag)::value;
         T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {}, m0[K] = {}, m1[K] = {};
+        T mo0[K] = {}, mo1[K] = {};
         if (PREFETCH) {
             if (PARAMS)
                 load_pair<T, 64, K, FULL>(irows, i + 2, s.xlo, s.xhi, h, q1, n0, n1, n2, n3);
             load_g(i + 2, m0);
             load_g(i + 3, m1);
+            if (S > 1) {
+                load_g_at(i + 2, q1og, mo0);
+                load_g_at(i + 3, q1og, mo1);
+            }
         }
 
         RowPair<T>* G = lds.grow + (FLIP ? glen : 0);
@@ -594,7 +630,7 @@ grad_output_stream_kernel(SampleArgs<T> a) {
         T* wtot = lds.wave_tot + FLIP * 2 * kMaxRowWaves;
         T* wtail = lds.wave_tail + FLIP * 2 * kMaxRowWaves;
         if (!MERGED) {
-            BOXCONV_PUBLISH_PAIR(FLIP, g0, g1, ta, t0, t1, bc, b1, b2, tl0, tl1)
+            BOXCONV_PUBLISH_PAIR(FLIP, g0, g1, go0, go1, ta, t0, t1, bc, b1, b2, tl0, tl1)
             __syncthreads();                                                 // rows are in LDS
         }
         T tail0 = tl0, tail1 = tl1;
@@ -643,7 +679,7 @@ grad_output_stream_kernel(SampleArgs<T> a) {
                 sum[4] += vw0 * tail0 + vw1 * tail1;
                 sum[1] += dbw0 * tail0 + dbw1 * tail1;
                 sum[0] -= dtw0 * tail0 + dtw1 * tail1;
-                if (tid == 0) {
+                if (tid == 0 && (S == 1 || owns_w)) {
                     const RowPair<T> gmax = G[idx_ymax], gmin = G[idx_ymin];
                     sum[3] += vw0 * gmax.r0 + vw1 * gmax.r1;
                     sum[2] -= vw0 * gmin.r0 + vw1 * gmin.r1;
@@ -714,7 +750,7 @@ grad_output_stream_kernel(SampleArgs<T> a) {
                     wtail[wave] = wt0; wtail[kMaxRowWaves + wave] = wt1;
                 }
             }
-            if (MERGED && PREFETCH) BOXCONV_PUBLISH_PAIR(FLIP ^ 1, m0, m1, t1, n0, n1, b2, n2, n3, tn0, tn1)
+            if (MERGED && PREFETCH) BOXCONV_PUBLISH_PAIR(FLIP ^ 1, m0, m1, mo0, mo1, t1, n0, n1, b2, n2, n3, tn0, tn1)
             __syncthreads();                         // wave totals (and the next pair's rows) visible
             {
                 // A[c] = (sum of all W + tail) - (W of the columns before c)
@@ -757,7 +793,7 @@ grad_output_stream_kernel(SampleArgs<T> a) {
         }
 
         if (!SCAN && MERGED) {
-            if (PREFETCH) BOXCONV_PUBLISH_PAIR(FLIP ^ 1, m0, m1, t1, n0, n1, b2, n2, n3, tn0, tn1)
+            if (PREFETCH) BOXCONV_PUBLISH_PAIR(FLIP ^ 1, m0, m1, mo0, mo1, t1, n0, n1, b2, n2, n3, tn0, tn1)
             __syncthreads();                                                 // the next pair's rows visible
         }
 
@@ -770,6 +806,7 @@ grad_output_stream_kernel(SampleArgs<T> a) {
                     t0[k] = n0[k]; t1[k] = n1[k]; b1[k] = n2[k]; b2[k] = n3[k];
                 }
                 g0[k] = m0[k]; g1[k] = m1[k];
+                if (S > 1) { go0[k] = mo0[k]; go1[k] = mo1[k]; }
             }
         }
         // keep the two unrolled pairs apart: loads of the pair after next hoisted up here would
@@ -802,7 +839,7 @@ grad_output_stream_kernel(SampleArgs<T> a) {
         // slots > 0: one slot per workgroup, summed by the finalize kernel in a fixed order
         // (no clearing pass, no atomics, bit-reproducible); else atomics into the box's five sums
         if (a.acc_slots > 0)
-            block_accumulate5(total, a.acc + ((static_cast<int64_t>(a.plane0 + p) * a.F + f) * a.acc_slots + band) * 5,
+            block_accumulate5(total, a.acc + ((static_cast<int64_t>(a.plane0 + p) * a.F + f) * a.acc_slots + band * S + part) * 5,
                               lds.red, false);
         else
             block_accumulate5(total, a.acc + static_cast<int64_t>(k_par) * 5, lds.red);
@@ -1011,19 +1048,47 @@ hipError_t grad_output_stream_launch(const T* integ, const TG* grad_out, BoxPara
     a.src = integ; a.grad_out = reinterpret_cast<const T*>(grad_out); a.acc = acc; a.acc_slots = acc_slots;
     a.dst = column_workspace;
     a.mpitch = column_workspace_pitch(d.w);
-    if (acc_slots != 0 && acc_slots != sp.nb) return hipErrorInvalidValue;
+    if (acc_slots != 0 && acc_slots != sp.nb * sp.parts) return hipErrorInvalidValue;
     a.nb = sp.nb; a.R = sp.R;
     a.keep_tail = scan ? cached_tail_bytes() / kXcds : 0;
     finish_args(a, planes_f * a.nb);
     const RowConfig rc = stream_row_config(d.w);
     const dim3 grid(static_cast<unsigned>(a.per_xcd * kXcds));
     const size_t lds = 0;                              // the kernel's LDS is statically sized
+    if (rc.nt == 1024) {
+        // Rows of 2049 to 4096 columns: 16 waves per workgroup leave a lane 128 registers, which
+        // the kernel that does both jobs at once does not fit; the two jobs run one after the
+        // other (grad_output is then read twice).
+        if constexpr (sizeof(T) <= 4) {
+            // parameter sums: two workgroups of 512 threads per band, each owning half the columns
+            // (a lane of the 1024-thread shape would spill half of that kernel's state)
+            SampleArgs<T> ap = a;
+            if (params && acc_slots == 0) return hipErrorInvalidValue;   // (the atomic mode has no slot per part)
+            finish_args(ap, planes_f * a.nb * 2);
+            const dim3 grid_p(static_cast<unsigned>(ap.per_xcd * kXcds));
+#define LAUNCH_GW(NT, KK, EX, FU) \
+            if (params) BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_kernel<T, TG, 512, KK, EX, false, true, false, 2>), grid_p, dim3(512), lds, stream, ap); \
+            if (scan)   BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_kernel<T, TG, NT, KK, EX, FU, false, true>), grid, dim3(NT), lds, stream, a)
+#define LAUNCH_GW_K(EX, FU) if (rc.K == 3) { LAUNCH_GW(1024, 3, EX, FU); } else { LAUNCH_GW(1024, 4, EX, FU); }
+            if (exact) { if (rc.full) { LAUNCH_GW_K(true, true) } else { LAUNCH_GW_K(true, false) } }
+            else       { if (rc.full) { LAUNCH_GW_K(false, true) } else { LAUNCH_GW_K(false, false) } }
+#undef LAUNCH_GW_K
+#undef LAUNCH_GW
+            return hipGetLastError();
+        } else {
+            return hipErrorInvalidValue;
+        }
+    }
+#pragma push_macro("BOXCONV_DISPATCH_WIDE")
+#undef BOXCONV_DISPATCH_WIDE
+#define BOXCONV_DISPATCH_WIDE(KERNEL, K, ...) { return hipErrorInvalidValue; }
 #define LAUNCH_GS(NT, KK, EX, FU) \
     if (params && scan) BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_kernel<T, TG, NT, KK, EX, FU, true, true>), grid, dim3(NT), lds, stream, a); \
     else if (params)    BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_kernel<T, TG, NT, KK, EX, FU, true, false>), grid, dim3(NT), lds, stream, a); \
     else                BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_kernel<T, TG, NT, KK, EX, FU, false, true>), grid, dim3(NT), lds, stream, a)
     BOXCONV_DISPATCH_SHAPE_EXACT_FULL(LAUNCH_GS, rc, exact)
 #undef LAUNCH_GS
+#pragma pop_macro("BOXCONV_DISPATCH_WIDE")
     return hipGetLastError();
 }
 

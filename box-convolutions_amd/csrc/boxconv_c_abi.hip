@@ -131,7 +131,7 @@ BackwardLayout backward_layout(int batch, int in_planes, int num_filters, int h,
         off += align_up(static_cast<size_t>(aux) * 8, 256);
     }
     L.acc_off = off;
-    L.acc_slots = (need_params && L.streaming) ? sp.nb : 0;
+    L.acc_slots = (need_params && L.streaming) ? sp.nb * sp.parts : 0;
     if (need_params)
         off += align_up(static_cast<size_t>(in_planes) * num_filters * 5 * 8 *
                         (L.acc_slots > 0 ? static_cast<size_t>(batch) * L.acc_slots : 1), 256);
@@ -490,7 +490,7 @@ int boxconv_integral_image_half_f32(const void* in, int input_dtype, float* out,
     if (!boxconv::integral_image_widening_applies(h, w))
         return fail(BOXCONV_E_TOO_LARGE, "integral image: half-precision input is read directly for rows "
                     "of at most %d columns and planes below 2 GiB; convert wider inputs to float first",
-                    boxconv::kMaxRowStreamWidth);
+                    boxconv::kMaxWideningWidth);
     if (input_dtype == BOXCONV_F16)
         return integral_image_widening_impl(static_cast<const boxconv::f16_t*>(in), out, planes, h, w,
                                             workspace, workspace_bytes, stream);

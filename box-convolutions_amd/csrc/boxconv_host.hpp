@@ -101,6 +101,8 @@ hipError_t grad_input_launch(const T* gint, int band_rows, BoxParams<T> prm, TO*
 struct StreamPlan {
     bool usable;             // false: width or LDS need outside what the streaming kernel covers
     int nb, R;               // bands per plane, rows per band (R even)
+    int parts;               // workgroups that share a band for the parameter sums (1, or 2 for rows
+                             // wider than 2048 columns): accumulation slots per (plane, filter) = nb * parts
 };
 StreamPlan plan_grad_output_stream(int64_t planes_f, int h, int w, size_t elem_size);
 
@@ -166,7 +168,9 @@ void profile_after(const char* name, hipStream_t stream);
         ::boxconv::profile_after(NAME, STREAM);                                   \
     } while (0)
 
-constexpr int kMaxRowStreamWidth = 2048;
-constexpr size_t kMaxDynamicLds = 64 * 1024;   // dynamic LDS a launch may request without opting in to more
+constexpr int kMaxRowStreamWidth = 4096;       // float32 rows; float64 rows half of that
+constexpr int kMaxScanRowsWidth = 4096;        // widest row the one-workgroup-per-row integral kernels take
+constexpr int kMaxWideningWidth = 2048;        // widest float16 / bfloat16 row the integral image reads directly
+constexpr size_t kMaxDynamicLds = 160 * 1024;  // LDS of a gfx950 CU, all of which one workgroup may use
 
 }  // namespace boxconv

@@ -11,7 +11,7 @@
 //   2. band_prefix_kernel  : running sum of aux over bands (in place) -> sum of all bands above
 //   3. band_scan_kernel    : per band, rows top to bottom: column accumulators (registers) +=
 //                            input row, then a row-direction prefix of the accumulators.
-// With a single band (tall enough grid without cutting) only launch 3 runs. Rows of at most 2048
+// With a single band (tall enough grid without cutting) only launch 3 runs. Rows of at most 4096
 // columns use band_scan_rows_kernel for launch 3, which adds up the bands above itself (no launch
 // 2). For float rows that fill a workgroup exactly and planes of at most 16 bands of 32 rows, one
 // kernel does everything in a single pass over the input (band_scan_lookback_kernel): workgroups
@@ -664,7 +664,6 @@ bool single_pass_applies(const IntegralPlan& pl) {
 
 // Rows this narrow are scanned by band_scan_rows_kernel, which sums the band column sums itself;
 // the bands above a workgroup are few (nb <= h/32), so re-reading them is cheaper than a pass.
-constexpr int kMaxScanRowsWidth = 2048;
 inline bool scan_by_rows(int h, int w, size_t elem) {
     const uint64_t plane_bytes = (static_cast<uint64_t>(h) + 1) * (static_cast<uint64_t>(w) + 1) * elem;
     return w <= kMaxScanRowsWidth && plane_bytes < (1ull << 31);
@@ -697,7 +696,7 @@ IntegralPlan plan_integral(int64_t planes, int h, int w, int64_t want) {
     const int64_t resident = w > 0 ? 256 * (8 / std::max(1, w / 256)) : 0;   // two waves per SIMD each
     const bool measured_faster = (w == 256 || w == 512 || w == 1024 || w == 2048) &&
                                  ((groups <= resident && bands32 <= 32) || groups >= 4096);
-    const bool single_pass = wanted >= 2 && h > kLookbackRows && scan_by_rows(h, w, sizeof(float)) &&
+    const bool single_pass = wanted >= 2 && h > kLookbackRows && w <= 2048 && scan_by_rows(h, w, sizeof(float)) &&
                              bands32 <= kLookbackBands && (lookback_any_shape() || measured_faster);
     if (single_pass) nb = (h + kLookbackRows - 1) / kLookbackRows;
     nb = std::max(nb, (h + 255) / 256);
@@ -729,7 +728,7 @@ hipError_t clip_and_prepare_integral_launch(const ClipArgs<T>& clip, int64_t pla
     return hipGetLastError();
 }
 
-// The tiled kernels for widths above 2048 read T only.
+// The tiled kernels for widths above 4096 read T only.
 template <class T, class TI>
 struct TiledScan {
     static hipError_t run(const TI*, T*, double*, int64_t, int, int, int, int, bool, hipStream_t) {
@@ -784,7 +783,8 @@ hipError_t integral_image_any(const TI* in, T* out, int64_t planes, int h, int w
         if (w <= 256)       return launch_scan_rows<T, TI, 1, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
         else if (w <= 512)  return launch_scan_rows<T, TI, 2, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
         else if (w <= 1024) return launch_scan_rows<T, TI, 4, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
-        else                return launch_scan_rows<T, TI, 8, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
+        else if (w <= 2048) return launch_scan_rows<T, TI, 8, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
+        else                return launch_scan_rows<T, TI, 16, 4>(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
     }
     return TiledScan<T, TI>::run(in, out, aux, planes, h, w, nb, R, reverse_order, stream);
 }
@@ -803,7 +803,9 @@ hipError_t integral_image_widening_launch(const TI* in, float* out, int64_t plan
     return integral_image_any<float, TI>(in, out, planes, h, w, aux, pl, false, false, stream);
 }
 
-bool integral_image_widening_applies(int h, int w) { return scan_by_rows(h, w, sizeof(float)); }
+bool integral_image_widening_applies(int h, int w) {
+    return w <= kMaxWideningWidth && scan_by_rows(h, w, sizeof(float));
+}
 
 template hipError_t integral_image_widening_launch<f16_t>(const f16_t*, float*, int64_t, int, int,
                                                           double*, const IntegralPlan&, hipStream_t);

@@ -174,8 +174,8 @@ int boxconv_forward_fused_f32(const float* input_integrated, const float* x_min,
  * re-reading it.
  * workspace: boxconv_backward_workspace_bytes(...) bytes, 256-byte aligned. It receives the
  * backward's one intermediate per (plane, filter) - h+1 rows of grad_output filtered along the
- * row and summed down the rows of a band (the bulk; for rows wider than 2048 columns a true
- * integral image of grad_output instead) - and the per-box accumulators. */
+ * row and summed down the rows of a band (the bulk; for rows wider than 4096 columns, 2048 in
+ * float64, a true integral image of grad_output instead) - and the per-box accumulators. */
 size_t boxconv_backward_workspace_bytes(int batch, int in_planes, int num_filters, int h, int w,
                                         int elem_size, int input_needs_grad,
                                         int params_need_grad);
@@ -201,7 +201,7 @@ int boxconv_backward_f64(const double* input_integrated, const double* x_min, co
  * (src/box_convolution_cuda_backward.cu:176,431, AT_DISPATCH_FLOATING_TYPES_AND_HALF) and then
  * integrates grad_output in half precision; here its rows are widened to float as they are read
  * and grad_input is rounded once, in the store. Same workspace as boxconv_backward_f32
- * (boxconv_backward_workspace_bytes with elem_size 4). Rows of at most 2048 columns
+ * (boxconv_backward_workspace_bytes with elem_size 4). Rows of at most 4096 columns
  * (BOXCONV_E_TOO_LARGE otherwise: convert to float first). */
 int boxconv_backward_half_f32(const float* input_integrated, const float* x_min, const float* x_max,
                               const float* y_min, const float* y_max, const void* grad_output,

@@ -109,12 +109,14 @@ def test_workspace_sizes(lib):
     assert only_params % (2 * 16 * 8 * 5 * 8) == 0
     assert only_input >= gint and full == only_input + only_params
     assert lib.boxconv_backward_workspace_bytes(2, 16, 8, 512, 1024, 2, 1, 1) == 0   # bad elem size
-    # the shape chooser at the width limit: float32 rows of 2048 columns stream (column workspace
-    # of h+1 rows of w), float64 rows of 2048 columns do not fit the streaming kernel's LDS and
-    # take the gather kernels (a true integral image of (h+1)(w+1) doubles), as do wider rows
-    f32_2048 = lib.boxconv_backward_workspace_bytes(1, 1, 1, 64, 2048, 4, 1, 0)
+    # the shape chooser at the width limits: float32 rows stream up to 4096 columns (column workspace
+    # of h+1 rows of w rounded up to 4), float64 rows up to 2048; wider rows take the gather
+    # kernels (a true integral image of (h+1)(w+1) elements)
+    f32_4096 = lib.boxconv_backward_workspace_bytes(1, 1, 1, 64, 4096, 4, 1, 0)
+    f32_4097 = lib.boxconv_backward_workspace_bytes(1, 1, 1, 64, 4097, 4, 1, 0)
     f64_2048 = lib.boxconv_backward_workspace_bytes(1, 1, 1, 64, 2048, 8, 1, 0)
-    f32_2049 = lib.boxconv_backward_workspace_bytes(1, 1, 1, 64, 2049, 4, 1, 0)
-    assert 65 * 2048 * 4 <= f32_2048 < 65 * 2049 * 4
-    assert f64_2048 >= 65 * 2049 * 8
-    assert f32_2049 >= 65 * 2050 * 4
+    f64_2049 = lib.boxconv_backward_workspace_bytes(1, 1, 1, 64, 2049, 8, 1, 0)
+    assert 65 * 4096 * 4 <= f32_4096 < 65 * 4097 * 4
+    assert f32_4097 >= 65 * 4098 * 4
+    assert 65 * 2048 * 8 <= f64_2048 < 65 * 2049 * 8
+    assert f64_2049 >= 65 * 2050 * 8

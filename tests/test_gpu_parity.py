@@ -27,6 +27,7 @@ def host(t):
 INTEGRAL_SHAPES = [
     (1, 2, 2), (3, 5, 7), (2, 10, 10), (6, 28, 28), (1, 33, 257), (2, 64, 128), (1, 200, 36),
     (1, 300, 1023), (2, 130, 1024), (1, 70, 2048), (1, 40, 2500), (1, 36, 4100), (1, 9, 9000),
+    (2, 100, 4096), (1, 170, 3000),                     # sixteen waves per row, several bands
     (5, 1, 1), (2, 1, 300), (2, 300, 1),
     # single-pass kernel: many bands, partial last band, 64 bands, one band too many for it
     (3, 512, 1000), (1, 2048, 64), (1, 2100, 40), (40, 100, 520), (9, 97, 1536),
@@ -174,6 +175,9 @@ SMALL_CASES = [
     # fill the workgroup's column slots exactly and rows that do not
     (1, 2, 2, 14, 192), (1, 1, 2, 13, 150), (2, 1, 2, 10, 384), (1, 1, 3, 9, 512), (1, 1, 2, 11, 500),
     (1, 2, 1, 16, 257),
+    # rows of 2049 to 4096 columns: 1024 threads, three or four columns per lane (float32; float64
+    # rows this wide and anything wider take the gather kernels)
+    (1, 1, 1, 8, 3072), (1, 2, 1, 7, 4096), (1, 1, 2, 6, 3500), (1, 1, 1, 5, 2049), (1, 1, 1, 5, 4100),
 ]
 
 
@@ -201,7 +205,7 @@ def test_forward_backward_small(hip, oracle, B, C, F, h, w, kind, dtype):
 
 
 @pytest.mark.parametrize("kind", ["inside", "hanging", "inverted"])
-@pytest.mark.parametrize("h,w", [(150, 90), (257, 256), (97, 520), (140, 400), (131, 170)])
+@pytest.mark.parametrize("h,w", [(150, 90), (257, 256), (97, 520), (140, 400), (131, 170), (100, 2600)])
 def test_backward_across_row_bands(hip, oracle, h, w, kind):
     """Images tall enough that the backward pass cuts grad_output into several row bands, with
     boxes whose top and bottom rows fall into different bands; 'inverted' boxes have min > max

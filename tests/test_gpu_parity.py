@@ -205,7 +205,7 @@ def test_forward_backward_small(hip, oracle, B, C, F, h, w, kind, dtype):
 
 
 @pytest.mark.parametrize("kind", ["inside", "hanging", "inverted"])
-@pytest.mark.parametrize("h,w", [(150, 90), (257, 256), (97, 520), (140, 400), (131, 170), (100, 2600)])
+@pytest.mark.parametrize("h,w", [(150, 90), (257, 256), (97, 520), (140, 400), (131, 170), (100, 2600), (3000, 40)])
 def test_backward_across_row_bands(hip, oracle, h, w, kind):
     """Images tall enough that the backward pass cuts grad_output into several row bands, with
     boxes whose top and bottom rows fall into different bands; 'inverted' boxes have min > max

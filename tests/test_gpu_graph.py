@@ -86,3 +86,41 @@ def test_captured_training_step_replays_identically(hip):
         torch.cuda.synchronize()
         for got, ref in zip(static_out, want):
             assert torch.equal(got, ref)
+
+
+def test_module_under_make_graphed_callables():
+    """torch.cuda.make_graphed_callables captures the module's forward and backward (autograd
+    included) into HIP graphs; replays must give the bits of the eager step. Nothing in the path
+    allocates outside torch's capture-safe allocator, synchronises or records a memset node."""
+    import warnings
+    from box_convolution import BoxConv2d
+    import random
+    dev = torch.device("cuda:0")
+
+    def make():
+        random.seed(5)
+        return BoxConv2d(3, 4, 40, 96).to(dev).train()
+
+    gen = torch.Generator(device=dev).manual_seed(3)
+    x = torch.randn(2, 3, 40, 96, device=dev, generator=gen).requires_grad_(True)
+    g = torch.randn(2, 12, 40, 96, device=dev, generator=gen)
+    eager = make()
+    out = eager(x)
+    out.backward(g)
+    want = [out.detach().clone(), x.grad.clone()] + [p.grad.clone() for p in eager.parameters()]
+
+    module = make()
+    sample = torch.randn_like(x).requires_grad_(True)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        graphed = torch.cuda.make_graphed_callables(module, (sample,))
+        for _ in range(3):
+            x.grad = None
+            for p in module.parameters():
+                p.grad = None
+            out = graphed(x)
+            out.backward(g)
+            torch.cuda.synchronize()
+            got = [out.detach(), x.grad] + [p.grad for p in module.parameters()]
+            for a, b in zip(want, got):
+                assert torch.equal(a, b)

@@ -33,10 +33,20 @@ __global__ void __launch_bounds__(NT) forward_rows_kernel(SampleArgs<T> a, Forwa
     const unsigned vid = xcd_contiguous_id(a.per_xcd);
     if (vid >= a.total) return;
     const unsigned nbands = a.nb, nfilt = a.F;
-    const int band = static_cast<int>(vid % nbands);
-    const unsigned pf32 = vid / nbands;
-    const int f = static_cast<int>(pf32 % nfilt);
-    const int64_t pf = pf32, p = pf32 / nfilt;
+    int band, f;
+    unsigned p32;
+    if (a.band_major) {                 // the filters of a band side by side (see forward_launch_any)
+        f = static_cast<int>(vid % nfilt);
+        const unsigned pb = vid / nfilt;
+        band = static_cast<int>(pb % nbands);
+        p32 = pb / nbands;
+    } else {
+        band = static_cast<int>(vid % nbands);
+        const unsigned pf_ = vid / nbands;
+        f = static_cast<int>(pf_ % nfilt);
+        p32 = pf_ / nfilt;
+    }
+    const int64_t p = p32, pf = p * nfilt + f;
     const int k_par = static_cast<int>(static_cast<unsigned>(a.plane0 + p) % static_cast<unsigned>(a.C)) * a.F + f;
     const int h = a.h, w = a.w;
     const unsigned row_bytes = static_cast<unsigned>(w) * sizeof(T);
@@ -210,6 +220,11 @@ hipError_t forward_launch_any(const T* integ, BoxParams<T> prm, ForwardTail<TO> 
     a.R += a.R & 1;                                   // rows are handled in pairs
     a.nb = (d.h + a.R - 1) / a.R;
     finish_args(a, planes_f * a.nb);
+    // An integral plane that does not fit an XCD's 4 MB L2 is streamed from memory once per filter
+    // when the bands of one filter run one after the other; with the filters of a band side by
+    // side their rows (a box height apart at most) are fetched together (1024 x 2048 with two
+    // filters: 737 -> 703 us). Planes that fit are faster in filter order (512 x 1024: 97 vs 100 us).
+    a.band_major = (static_cast<uint64_t>(d.h + 1) * (d.w + 1) * sizeof(T) > (4u << 20)) ? 1 : 0;
     const dim3 grid(static_cast<unsigned>(a.per_xcd * kXcds));
     const size_t lds = 4 * static_cast<size_t>(d.w + 3) * sizeof(T);
 #define LAUNCH_FWD(NT, KK, EX, FU) \

@@ -33,19 +33,12 @@ __global__ void __launch_bounds__(NT) forward_rows_kernel(SampleArgs<T> a, Forwa
     const unsigned vid = xcd_contiguous_id(a.per_xcd);
     if (vid >= a.total) return;
     const unsigned nbands = a.nb, nfilt = a.F;
-    int band, f;
-    unsigned p32;
-    if (a.band_major) {                 // the filters of a band side by side (see forward_launch_any)
-        f = static_cast<int>(vid % nfilt);
-        const unsigned pb = vid / nfilt;
-        band = static_cast<int>(pb % nbands);
-        p32 = pb / nbands;
-    } else {
-        band = static_cast<int>(vid % nbands);
-        const unsigned pf_ = vid / nbands;
-        f = static_cast<int>(pf_ % nfilt);
-        p32 = pf_ / nfilt;
-    }
+    // (plane, filter, band) order, or (plane, band, filter): see forward_launch_any
+    const unsigned inner = a.band_major ? nfilt : nbands, outer = a.band_major ? nbands : nfilt;
+    const unsigned v_in = vid % inner, v_rest = vid / inner;
+    const unsigned v_out = v_rest % outer, p32 = v_rest / outer;
+    const int band = static_cast<int>(a.band_major ? v_out : v_in);
+    const int f = static_cast<int>(a.band_major ? v_in : v_out);
     const int64_t p = p32, pf = p * nfilt + f;
     const int k_par = static_cast<int>(static_cast<unsigned>(a.plane0 + p) % static_cast<unsigned>(a.C)) * a.F + f;
     const int h = a.h, w = a.w;

@@ -3,6 +3,8 @@
 Tolerances: forward and grad_input max|gpu-cpu|/max|cpu| <= 1e-4, box-parameter gradients <= 1e-3
 for float32 (the targets the build is held to); 1e-9 for float64.
 """
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -282,10 +284,12 @@ def test_grad_input_filter_sharing_matches_one_set_per_workgroup(hip, monkeypatc
     def grad_input():
         return hip.box_convolution_backward(integ, *boxes, g, None, 5.0, 3.0, True, True,
                                             True, False, False, False, False)[0].clone()
+    preset = os.environ.get("BOXCONV_GI_SPLIT_FILTERS")     # (a run of the suite with the switch set)
     shared = grad_input()
     monkeypatch.setenv("BOXCONV_GI_SPLIT_FILTERS", "0")
     single = grad_input()
-    assert not torch.equal(shared, single) or F < 3       # really two different code paths
+    if os.environ.get("BOXCONV_FORCE_GATHER") != "1" and preset is None:
+        assert not torch.equal(shared, single) or F < 3   # really two different code paths
     scale = single.abs().max().item()
     assert (shared - single).abs().max().item() <= 4e-6 * scale
 

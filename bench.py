@@ -37,7 +37,10 @@ HBM_PEAK_GBS = 8000.0   # MI355X HBM3E
 EVENT_EVERY = 5     # launches of the dominant kernel per HIP-event pair in the timed region
 REPEATS = 7         # timed regions of --steps steps each; the median one is reported
 PREWARM_MAX_S = 1.5 # upper bound on the untimed clock-up phase after --warmup
-TIMED_KERNELS = ("grad_output_stream", "band_scan", "band_colsum", "forward_rows", "grad_input_cols")
+RANKING_STEPS = 3   # untimed eager steps per kernel name while the per-kernel times are taken
+# every kernel a training step launches ("clip" is the parameter projection, which shares its
+# launch with the marking of the single-pass integral image's hand-over words)
+TIMED_KERNELS = ("grad_output_stream", "band_scan", "band_colsum", "forward_rows", "grad_input_cols", "clip")
 METRIC = "BoxConv2d fwd+bwd ms/iter + effective HBM GB/s (% peak) at 2x16ch 512x1024 fp32"
 
 
@@ -45,6 +48,7 @@ def kernel_algorithmic_bytes(ab, elem=4):
     """Algorithmic bytes moved by ONE launch of each kernel at a given workload: the share of the
     step's data flow that the kernel is responsible for (each is launched once per step)."""
     return {
+        "clip": 0,                                               # kilobytes of box parameters and marker words
         # read grad_output and the input's integral, write the (band-local) integral of grad_output
         "grad_output_stream": elem * (ab["n_out"] + ab["n_int"] + ab["n_gint"]),
         "band_scan": elem * (ab["n_in"] + ab["n_int"]),          # read input, write its integral
@@ -109,6 +113,106 @@ def cpu_baseline(k, ab_full):
     }
 
 
+def make_step(wl, dev):
+    """(module, x, g, eager_step) for one workload, tensors resident on `dev`."""
+    import torch
+    from box_convolution import BoxConv2d
+    module = BoxConv2d(wl.C, wl.F, wl.h, wl.w, wl.reparametrization_factor).to(dev)
+    with torch.no_grad():
+        for p, v in zip((module.x_min, module.x_max, module.y_min, module.y_max),
+                        (wl.x_min, wl.x_max, wl.y_min, wl.y_max)):
+            p.copy_(v)
+    module.train()
+    x = wl.x.to(dev).requires_grad_(True)
+    g = wl.grad_output.to(dev)
+    params = list(module.parameters())
+
+    def eager_step():
+        x.grad = None
+        for p in params:
+            p.grad = None
+        out = module(x)
+        out.backward(g)
+    return module, x, g, eager_step
+
+
+def capture_native_step(wl, module, x, g):
+    """A HIP graph of the native calls of one training step (clip + integral image + forward,
+    backward through the C ABI); returns (replay, keep_alive)."""
+    import torch
+    from box_convolution import _native
+    stored = [p.detach() for p in (module.x_min, module.x_max, module.y_min, module.y_max)]
+    x_static = x.detach()
+
+    def native_step():
+        integ, out, real = _native.training_forward(
+            x_static, *stored, wl.reparametrization_h, wl.reparametrization_w, wl.h, wl.w, True, True)
+        return out, _native.box_convolution_backward(
+            integ, *real, g, None, wl.reparametrization_h, wl.reparametrization_w, True, True,
+            True, True, True, True, True)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        native_step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        keep_alive = native_step()
+    return graph.replay, (graph, keep_alive)
+
+
+def time_steps(step, steps, repeats):
+    """Median, min, max seconds per region of `steps` steps between two synchronisations."""
+    import torch
+    regions = []
+    for _ in range(repeats):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        regions.append(time.perf_counter() - t0)
+    return sorted(regions)[len(regions) // 2], min(regions), max(regions)
+
+
+def small_workload_extra(k, dev, steps=200):
+    """Eager and captured-graph step time of a small workload (its kernels take tens of
+    microseconds, so the eager figure is what the host can enqueue)."""
+    from baseline_workloads import algorithmic_bytes, make_workload
+    wl = make_workload(k)
+    module, x, g, eager_step = make_step(wl, dev)
+    ab = algorithmic_bytes(wl.B, wl.C, wl.F, wl.h, wl.w)
+    for _ in range(20):
+        eager_step()
+    eager, _, _ = time_steps(eager_step, steps, 3)
+    replay, keep = capture_native_step(wl, module, x, g)
+    for _ in range(20):
+        replay()
+    graph, _, _ = time_steps(replay, steps, 3)
+    del keep
+    return {
+        "workload": wl.name,
+        "eager_ms_per_step": round(1e3 * eager / steps, 4),
+        "graph_ms_per_step": round(1e3 * graph / steps, 4),
+        "eager_GBps": round(ab["alg"] / (eager / steps) / 1e9, 1),
+        "graph_GBps": round(ab["alg"] / (graph / steps) / 1e9, 1),
+        "eager_over_graph": round(eager / graph, 2),
+    }
+
+
+def event_pair_overhead_ms(n=50):
+    """What a pair of HIP events with nothing between them measures on the current stream."""
+    import torch
+    torch.cuda.synchronize()
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+    for a, b in pairs:
+        a.record()
+        b.record()
+    torch.cuda.synchronize()
+    vals = sorted(a.elapsed_time(b) for a, b in pairs)
+    return vals[len(vals) // 2]
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -116,6 +220,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", type=int, default=3, choices=[1, 2, 3, 4, 5])
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--no-extra", action="store_true",
+                    help="skip the eager/graph step time of the BoxENet-block workload (`extra`)")
     ap.add_argument("--phases", action="store_true", help="also print per-kernel times to stderr")
     ap.add_argument("--graph", action="store_true",
                     help="time replays of a captured HIP graph of the step's native calls (training "
@@ -170,22 +276,8 @@ def main():
         wl = make_workload(args.workload)
     ab = algorithmic_bytes(wl.B, wl.C, wl.F, wl.h, wl.w)
 
-    module = BoxConv2d(wl.C, wl.F, wl.h, wl.w, wl.reparametrization_factor).to(dev)
-    with torch.no_grad():
-        for p, v in zip((module.x_min, module.x_max, module.y_min, module.y_max),
-                        (wl.x_min, wl.x_max, wl.y_min, wl.y_max)):
-            p.copy_(v)
-    module.train()
-    x = wl.x.to(dev).requires_grad_(True)
-    g = wl.grad_output.to(dev)
+    module, x, g, eager_step = make_step(wl, dev)
     params = list(module.parameters())
-
-    def eager_step():
-        x.grad = None
-        for p in params:
-            p.grad = None
-        out = module(x)
-        out.backward(g)
 
     if args.forward_only:
         if args.graph:
@@ -229,36 +321,24 @@ def main():
             break
         last = cur
 
-    # which kernel takes the most time per step (three untimed eager steps per candidate)
+    # which kernel takes the most time per step (RANKING_STEPS untimed eager steps per kernel
+    # name). An event pair with nothing between its events already measures a few microseconds;
+    # that is taken off every bracketed launch, so that the figures are the kernels' own time.
+    pair_ms = event_pair_overhead_ms()
     per_kernel = {}
     for name in TIMED_KERNELS:
         _native.profile_arm(name)
-        for _ in range(3):
+        for _ in range(RANKING_STEPS):
             eager_step()
         ms, launches = _native.profile_collect()
-        per_kernel[name] = (ms / 3, launches // 3, ms / max(launches, 1))
+        ms = max(ms - pair_ms * launches, 0.0)
+        per_kernel[name] = (ms / RANKING_STEPS, launches // RANKING_STEPS, ms / max(launches, 1))
     dominant = max(per_kernel, key=lambda n: per_kernel[n][0])
 
     if args.graph:
         # the native calls of one step, captured once: clip + integral image + forward, backward
-        stored = [p.detach() for p in (module.x_min, module.x_max, module.y_min, module.y_max)]
-        x_static = x.detach()
-
-        def native_step():
-            integ, out, real = _native.training_forward(
-                x_static, *stored, wl.reparametrization_h, wl.reparametrization_w, wl.h, wl.w, True, True)
-            return out, _native.box_convolution_backward(
-                integ, *real, g, None, wl.reparametrization_h, wl.reparametrization_w, True, True,
-                True, True, True, True, True)
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            native_step()
-        torch.cuda.current_stream().wait_stream(side)
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            keep_alive = native_step()
-        step = graph.replay
+        replay, keep_alive = capture_native_step(wl, module, x, g)
+        step = replay
         for _ in range(max(args.warmup, 5)):
             step()
         torch.cuda.synchronize()
@@ -280,6 +360,7 @@ def main():
         dom_ms, dom_launches = per_kernel[dominant][2] * 3, 3
     else:
         dom_ms, dom_launches = _native.profile_collect()
+        dom_ms = max(dom_ms - pair_ms * dom_launches, 0.0)
     elapsed = sorted(regions)[len(regions) // 2]
 
     if args.copy_probe > 0:
@@ -312,6 +393,9 @@ def main():
         "ms_per_step_max": round(1e3 * max(regions) / args.steps, 4),
         "timed_regions": REPEATS,
         "prewarm_steps": prewarm_steps,
+        # every untimed step before the timed regions: --warmup, the clock-up phase, and the
+        # RANKING_STEPS steps per kernel name during which the per-kernel times were taken
+        "warmup_total": args.warmup + prewarm_steps + RANKING_STEPS * len(TIMED_KERNELS),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -343,8 +427,15 @@ def main():
             "avg_launch_us": round(1e6 * avg_launch_s, 2),
             "launches_timed": dom_launches,
         },
+        # own time of every kernel of the step (HIP events around each launch, the empty event
+        # pair's own reading taken off); their sum is what the step would take with no gaps
         "kernel_ms_per_step": {k: round(v[0], 4) for k, v in per_kernel.items()},
+        "kernel_sum_ms": round(sum(v[0] for v in per_kernel.values()), 4),
+        "event_pair_overhead_us": round(1e3 * pair_ms, 2),
     }
+    if not (args.no_extra or args.graph or args.forward_only or args.shape):
+        # the realistic layer shape of the reference's model zoo (a BoxENet block)
+        result["extra"] = {"boxenet_block": small_workload_extra(2, dev)}
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(args.workload, ab)
         result["cpu_baseline"]["speedup_vs_cpu"] = round(result["cpu_baseline"]["ms_per_step"] / ms_per_step, 1)

@@ -99,12 +99,22 @@ def make_workload(k, batch=None, in_planes=None, reparametrization_factor=8):
             x = torch.randn(B, C, h, w, generator=gen)
     g = torch.randn(B, C * F, h, w, generator=gen)
 
+    wl = Workload(k, name, B, C, F, h, w, reparametrization_factor, x, g, *stored,
+                  reparam_h, reparam_w)
     if batch is not None or in_planes is not None:
-        b = B if batch is None else batch
-        c = C if in_planes is None else in_planes
-        x = x[:b, :c].contiguous()
-        g = g.view(B, C, F, h, w)[:b, :c].reshape(b, c * F, h, w).contiguous()
-        stored = [p[:c].contiguous() for p in stored]
-        B, C = b, c
-    return Workload(k, name, B, C, F, h, w, reparametrization_factor, x, g, *stored,
-                    reparam_h, reparam_w)
+        wl = restrict(wl, 0, C if in_planes is None else in_planes, batch)
+    return wl
+
+
+def restrict(wl, c0, c1, batch=None):
+    """The input planes [c0, c1) (and the first `batch` batch items) of a workload: same data,
+    same boxes for the planes that remain. Box convolution is independent per input plane and a
+    parameter gradient only sums over the batch, so a checker run on the restricted workload
+    reproduces exactly the matching slices of the full result."""
+    b = wl.B if batch is None else batch
+    F, h, w = wl.F, wl.h, wl.w
+    x = wl.x[:b, c0:c1].contiguous()
+    g = wl.grad_output.view(wl.B, wl.C, F, h, w)[:b, c0:c1].reshape(b, (c1 - c0) * F, h, w).contiguous()
+    stored = [p[c0:c1].contiguous() for p in (wl.x_min, wl.x_max, wl.y_min, wl.y_max)]
+    return wl._replace(B=b, C=c1 - c0, x=x, grad_output=g, x_min=stored[0], x_max=stored[1],
+                       y_min=stored[2], y_max=stored[3])

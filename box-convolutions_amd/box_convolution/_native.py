@@ -16,7 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_NAME = "libboxconv_hip.so"
 LIB_PATH = os.path.join(_HERE, LIB_NAME)
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _lib = None
 
@@ -27,6 +27,7 @@ _vp, _i, _i64, _sz, _f, _d = (ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, cty
 _SIGNATURES = {
     "boxconv_abi_version": (_i, []),
     "boxconv_last_error": (ctypes.c_char_p, []),
+    "boxconv_reload_env": (None, []),
     "boxconv_profile_arm": (_i, [ctypes.c_char_p]),
     "boxconv_profile_arm_every": (_i, [ctypes.c_char_p, _i]),
     "boxconv_profile_collect": (_i, [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int)]),
@@ -485,6 +486,12 @@ def training_forward(input, x_min, x_max, y_min, y_max, reparametrization_h, rep
 KERNEL_NAMES = ("band_colsum", "band_prefix", "band_scan", "forward_rows", "grad_output_stream",
                 "grad_input_cols", "param_grad_finalize", "fill_zero", "fill_marker", "clip",
                 "forward_gather", "grad_input_gather", "grad_params_gather")
+
+
+def reload_switches():
+    """Make the library read its BOXCONV_* environment switches again (it reads them once, at
+    first use). For tests that change a switch inside a running process."""
+    load().boxconv_reload_env()
 
 
 def profile_arm(kernel_name, every=1):

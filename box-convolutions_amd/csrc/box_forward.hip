@@ -192,10 +192,10 @@ hipError_t forward_launch_any(const T* integ, BoxParams<T> prm, ForwardTail<TO> 
     SampleArgs<T> a = base_args(prm, d);
     a.src = integ; a.normalize = normalize ? 1 : 0;
 
-    // (the row kernel keeps two row pairs of w + 3 columns in LDS: float64 rows of 2046 columns
-    // and more would ask for more than a launch gets without opting in)
+    // (the row kernel keeps two row pairs of w + 3 columns in LDS, up to 64 KiB + 48 bytes for the
+    // widest rows it takes; a device that grants a workgroup less goes to the gather kernel)
     if (!row_kernels_apply(d.h, d.w, sizeof(T)) ||
-        4 * static_cast<size_t>(d.w + 3) * sizeof(T) > kMaxDynamicLds) {
+        4 * static_cast<size_t>(d.w + 3) * sizeof(T) > std::min(kMaxDynamicLds, device_lds_limit())) {
         finish_args(a, planes_f * d.hw());
         const dim3 grid(static_cast<unsigned>((a.total + 255) / 256));
         if (exact) BOXCONV_LAUNCH("forward_gather", (forward_gather_kernel<T, TO, true, TAIL>), grid, dim3(256), 0, stream, a, tail);
@@ -203,8 +203,7 @@ hipError_t forward_launch_any(const T* integ, BoxParams<T> prm, ForwardTail<TO> 
         return hipGetLastError();
     }
 
-    static const int fwd_threads = preferred_row_threads("BOXCONV_FWD_THREADS", 512);
-    const RowConfig rc = row_config(d.w, fwd_threads);
+    const RowConfig rc = row_config(d.w, switches().fwd_threads);
     // Many short-lived workgroups (bands of 8 rows at the headline size): the kernel then ends
     // with a short tail. Measured per step: 16 workgroup-waves' worth of bands 0.501 ms, 8 0.508 ms,
     // 4 0.517 ms, 32 (bands of 4 rows, too much halo) 0.523 ms.

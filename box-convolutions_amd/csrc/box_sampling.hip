@@ -1,13 +1,79 @@
 // Host-side pieces of the box-sampling kernels that do not depend on the element type; the
 // kernels themselves are templates in box_sampling_impl.hpp, instantiated by box_sampling_inst.hip.
 
+#include <atomic>
+#include <mutex>
+
 #include "box_sampling_impl.hpp"   // stream_lds_bytes; the templates in it are not instantiated here
 
 namespace boxconv {
 
-bool force_gather_kernels() {
-    const char* e = std::getenv("BOXCONV_FORCE_GATHER");
-    return e != nullptr && e[0] == '1';
+namespace {
+
+Switches read_switches() {
+    auto text = [](const char* name) { return std::getenv(name); };
+    auto flag_unless_zero = [&](const char* name) { const char* e = text(name); return e == nullptr || e[0] != '0'; };
+    auto threads = [&](const char* name, int fallback) {
+        const char* e = text(name);
+        const int n = e ? std::atoi(e) : fallback;
+        return (n == 256 || n == 512) ? n : fallback;
+    };
+    Switches s{};
+    const char* e = text("BOXCONV_FORCE_GATHER");
+    s.force_gather = e != nullptr && e[0] == '1';
+    s.gi_reverse = flag_unless_zero("BOXCONV_GI_REVERSE");
+    s.bwd_reverse = flag_unless_zero("BOXCONV_BWD_REVERSE");
+    e = text("BOXCONV_GI_SPLIT_FILTERS");
+    s.gi_split_filters = e == nullptr || std::atoi(e) != 0;
+    e = text("BOXCONV_INTEGRAL_LOOKBACK");
+    s.lookback = e == nullptr || std::atoi(e) != 0;
+    s.lookback_any_shape = e != nullptr && std::atoi(e) == 2;
+    e = text("BOXCONV_INTEGRAL_SPIN");
+    s.spin_limit = e != nullptr ? std::max(0, std::atoi(e)) : 64;
+    s.fwd_threads = threads("BOXCONV_FWD_THREADS", 512);
+    s.stream_threads = threads("BOXCONV_STREAM_THREADS", 256);
+    e = text("BOXCONV_L_KEEP_MB");
+    s.keep_tail_bytes = static_cast<int64_t>(e != nullptr ? std::max(0, std::atoi(e)) : 192) << 20;
+    return s;
+}
+
+std::mutex g_switch_mutex;
+std::atomic<bool> g_switches_read{false};
+Switches g_switches;
+
+constexpr int kLdsDevices = 64;
+std::atomic<int64_t> g_lds_limit[kLdsDevices];     // 0 = not looked up yet, -1 = query failed
+
+}  // namespace
+
+const Switches& switches() {
+    if (!g_switches_read.load(std::memory_order_acquire)) {
+        std::lock_guard<std::mutex> lock(g_switch_mutex);
+        if (!g_switches_read.load(std::memory_order_relaxed)) {
+            g_switches = read_switches();
+            g_switches_read.store(true, std::memory_order_release);
+        }
+    }
+    return g_switches;
+}
+
+void reload_switches() {
+    std::lock_guard<std::mutex> lock(g_switch_mutex);
+    g_switches = read_switches();
+    g_switches_read.store(true, std::memory_order_release);
+}
+
+size_t device_lds_limit() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kLdsDevices) return 0;
+    int64_t v = g_lds_limit[dev].load(std::memory_order_relaxed);
+    if (v == 0) {
+        int bytes = 0;
+        v = hipDeviceGetAttribute(&bytes, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) == hipSuccess && bytes > 0
+                ? bytes : -1;
+        g_lds_limit[dev].store(v, std::memory_order_relaxed);
+    }
+    return v > 0 ? static_cast<size_t>(v) : 0;
 }
 
 namespace {

@@ -227,11 +227,6 @@ __device__ __forceinline__ T gather_box(const T* __restrict__ plane, const BoxSp
 // threads, which bounds the register footprint and the length of the per-lane float
 // accumulation chains.
 struct RowConfig { int nt; int K; bool full; };
-inline int preferred_row_threads(const char* env_name, int fallback) {
-    const char* e = std::getenv(env_name);
-    const int n = e ? std::atoi(e) : fallback;
-    return (n == 256 || n == 512) ? n : fallback;
-}
 inline RowConfig row_config(int w, int prefer) {
     RowConfig c;
     if (w <= 128) {
@@ -264,17 +259,10 @@ inline bool row_kernels_apply(int h, int w, size_t elem_size) {
 
 // The grad-input kernel runs right after the pass that wrote the integral of grad_output; the
 // planes written last are the ones most likely still held by the memory-side cache.
-inline bool reverse_grad_input() {
-    static const bool v = [] {
-        const char* e = std::getenv("BOXCONV_GI_REVERSE");
-        return e == nullptr || e[0] != '0';
-    }();
-    return v;
-}
+inline bool reverse_grad_input() { return switches().gi_reverse; }
 
 inline RowConfig stream_row_config(int w) {
-    static const int prefer = preferred_row_threads("BOXCONV_STREAM_THREADS", 256);
-    return row_config(w, prefer);
+    return row_config(w, switches().stream_threads);
 }
 
 inline int bands_for(int64_t independent, int h, int min_rows, int64_t want) {

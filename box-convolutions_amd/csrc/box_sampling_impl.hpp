@@ -925,12 +925,8 @@ FinalizeArgs<T> finalize_args(const ParamFinish<T>& f) {
 }
 
 // BOXCONV_GI_SPLIT_FILTERS=0: every workgroup of the grad-input kernel walks through all
-// filters itself (for comparison; read at every call, so that a test can switch it within one
-// process).
-inline bool split_filters_enabled() {
-    const char* e = std::getenv("BOXCONV_GI_SPLIT_FILTERS");
-    return e == nullptr || std::atoi(e) != 0;
-}
+// filters itself (for comparison).
+inline bool split_filters_enabled() { return switches().gi_split_filters; }
 
 // Shape of the grad-input launch for an image of h x w with F filters per plane: 2^lq lanes
 // (4 columns each) side by side, rb output rows per lane, fs sets of threads sharing the filters.
@@ -1028,13 +1024,7 @@ hipError_t grad_input_launch(const T* gint, int band_rows, BoxParams<T> prm, TO*
 
 // How much of the band-local integral, counted from its end, is written with the ordinary cache
 // policy (the memory-side cache holds 256 MB; the grad-input kernel reads that part first).
-inline int64_t cached_tail_bytes() {
-    static const int64_t v = [] {
-        const char* e = std::getenv("BOXCONV_L_KEEP_MB");
-        return static_cast<int64_t>(e != nullptr ? std::max(0, std::atoi(e)) : 192) << 20;
-    }();
-    return v;
-}
+inline int64_t cached_tail_bytes() { return switches().keep_tail_bytes; }
 
 template <class T, class TG>
 hipError_t grad_output_stream_launch(const T* integ, const TG* grad_out, BoxParams<T> prm,
@@ -1053,6 +1043,9 @@ hipError_t grad_output_stream_launch(const T* integ, const TG* grad_out, BoxPara
     a.keep_tail = scan ? cached_tail_bytes() / kXcds : 0;
     finish_args(a, planes_f * a.nb);
     const RowConfig rc = stream_row_config(d.w);
+    // The workspace layout was fixed by plan_grad_output_stream for a gfx950 CU's LDS; a device
+    // that grants a workgroup less cannot run this kernel (and has no fallback at this point).
+    if (stream_lds_bytes(rc.K, rc.nt, sizeof(T)) > device_lds_limit()) return hipErrorInvalidConfiguration;
     const dim3 grid(static_cast<unsigned>(a.per_xcd * kXcds));
     const size_t lds = 0;                              // the kernel's LDS is statically sized
     if (rc.nt == 1024) {

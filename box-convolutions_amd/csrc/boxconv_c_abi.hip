@@ -91,13 +91,7 @@ int check_dims(int batch, int in_planes, int num_filters, int h, int w) {
 }
 
 // Walk the planes last to first in the second pass over a tensor (see integral_image_launch).
-bool reverse_second_pass() {
-    static const bool v = [] {
-        const char* e = std::getenv("BOXCONV_BWD_REVERSE");
-        return e == nullptr || e[0] != '0';
-    }();
-    return v;
-}
+bool reverse_second_pass() { return boxconv::switches().bwd_reverse; }
 
 // Workspace of the backward pass:
 //   [column workspace M of grad_output: planes*F planes of (h+1) rows, or their integral images
@@ -438,6 +432,8 @@ int boxconv_profile_collect(double* total_ms, int* launches) {
 }
 
 const char* boxconv_last_error(void) { return g_error; }
+
+void boxconv_reload_env(void) { boxconv::reload_switches(); }
 
 size_t boxconv_integral_image_workspace_bytes(int64_t planes, int h, int w) {
     if (planes <= 0 || h < 1 || w < 1) return 0;

@@ -274,12 +274,16 @@ __device__ __forceinline__ void buffer_store(bf16_t v, const RowRef& r, int off)
 // inside the row, nothing to test.
 //
 // A buffer store of more than 8 bytes per lane reads its data registers over several cycles
-// after issue. The compiler keeps the next write to those registers one wait state away only
-// when the store has no scalar offset register; with one (the stacked descriptors of `Rows` above) it
-// assumes no hazard, and a conversion to double placed right behind such a store was observed
-// to replace the first two dwords of the data in the lanes the store reads last. Two wait
-// states behind every wide store rule that out at a cost of two cycles.
-__device__ __forceinline__ void settle_wide_store() { asm volatile("s_nop 1"); }
+// after issue. Observed once: with a scalar offset register on the store (the stacked descriptors
+// of `Rows` above), a conversion to double scheduled right behind a 16-byte store replaced the
+// first two dwords of the data in some lanes (row h of the column workspace at width 2048). The
+// working hypothesis is a store-data hazard that the compiler's hazard recogniser does not cover
+// for this form; it has not been confirmed beyond that observation and the fact that wait states
+// behind the store remove it. settle_wide_store therefore takes the data registers as an operand
+// of the wait-state statement: their live range then extends past the wait states, so no
+// instruction that overwrites them can be scheduled in between.
+template <class V>
+__device__ __forceinline__ void settle_wide_store(const V& data) { asm volatile("s_nop 1" : : "v"(data)); }
 
 template <int POLICY, int K>
 __device__ __forceinline__ void buffer_store_wide(const float (&v)[K], const RowRef& r, int off) {
@@ -292,13 +296,13 @@ __device__ __forceinline__ void buffer_store_wide(const float (&v)[K], const Row
             const v4u pack = {__builtin_bit_cast(unsigned, v[k]), __builtin_bit_cast(unsigned, v[k + 1]),
                               __builtin_bit_cast(unsigned, v[k + 2]), __builtin_bit_cast(unsigned, v[k + 3])};
             __builtin_amdgcn_raw_buffer_store_b128(pack, r.rs, off + 4 * k, r.soff, POLICY);
+            settle_wide_store(pack);
         }
-        settle_wide_store();
     } else if constexpr (K == 3) {
         const v3u pack = {__builtin_bit_cast(unsigned, v[0]), __builtin_bit_cast(unsigned, v[1]),
                           __builtin_bit_cast(unsigned, v[2])};
         __builtin_amdgcn_raw_buffer_store_b96(pack, r.rs, off, r.soff, POLICY);
-        settle_wide_store();
+        settle_wide_store(pack);
     } else if constexpr (K == 2) {
         const v2u pack = {__builtin_bit_cast(unsigned, v[0]), __builtin_bit_cast(unsigned, v[1])};
         __builtin_amdgcn_raw_buffer_store_b64(pack, r.rs, off, r.soff, POLICY);

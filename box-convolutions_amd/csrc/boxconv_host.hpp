@@ -151,10 +151,32 @@ hipError_t clip_launch(T* xmin, T* xmax, T* ymin, T* ymax, T* real, int n, doubl
                        double reparam_w, double max_h, double max_w, bool exact,
                        hipStream_t stream);
 
+// Measurement and test switches (environment variables BOXCONV_*). They are read ONCE, at the
+// first call that needs them, and again only by reload_switches() (exported as
+// boxconv_reload_env): no entry point calls getenv on its way to a launch.
+struct Switches {
+    bool force_gather;        // BOXCONV_FORCE_GATHER=1: per-pixel gather kernels for every shape
+    bool gi_reverse;          // BOXCONV_GI_REVERSE=0 clears it: grad-input walks the planes first to last
+    bool bwd_reverse;         // BOXCONV_BWD_REVERSE=0 clears it: the same for the gather path's second pass
+    bool gi_split_filters;    // BOXCONV_GI_SPLIT_FILTERS=0 clears it: no filter sharing in small grad-input launches
+    bool lookback;            // BOXCONV_INTEGRAL_LOOKBACK=0 clears it: no single-pass integral image
+    bool lookback_any_shape;  // BOXCONV_INTEGRAL_LOOKBACK=2: single pass for every shape it covers
+    int spin_limit;           // BOXCONV_INTEGRAL_SPIN: polls of a hand-over word before re-summing (64)
+    int fwd_threads;          // BOXCONV_FWD_THREADS: 256 or 512 (512)
+    int stream_threads;       // BOXCONV_STREAM_THREADS: 256 or 512 (256)
+    int64_t keep_tail_bytes;  // BOXCONV_L_KEEP_MB: end of the column workspace stored with the ordinary cache policy (192 MB)
+};
+const Switches& switches();
+void reload_switches();       // not synchronised with calls in flight on other threads
+
 // True when the environment asks for the gather kernels (one thread per output pixel, no LDS
 // row staging) instead of the row-streaming ones; the gather kernels also serve widths the
 // row-streaming kernels do not cover.
-bool force_gather_kernels();
+inline bool force_gather_kernels() { return switches().force_gather; }
+
+// LDS bytes one workgroup may use on the current device (hipDeviceAttributeMaxSharedMemoryPerBlock,
+// looked up once per device; 0 if the query fails, which sends every shape to the gather kernels).
+size_t device_lds_limit();
 
 // Optional per-kernel timing (see boxconv_profile_arm in include/boxconv.h). When a kernel name is
 // armed, every launch of that kernel is bracketed by a pair of HIP events on its stream.
@@ -172,5 +194,7 @@ constexpr int kMaxRowStreamWidth = 4096;       // float32 rows; float64 rows hal
 constexpr int kMaxScanRowsWidth = 4096;        // widest row the one-workgroup-per-row integral kernels take
 constexpr int kMaxWideningWidth = 2048;        // widest float16 / bfloat16 row the integral image reads directly
 constexpr size_t kMaxDynamicLds = 160 * 1024;  // LDS of a gfx950 CU, all of which one workgroup may use
+                                               // (the library is built for gfx950 only; launches also
+                                               // check device_lds_limit())
 
 }  // namespace boxconv

@@ -599,21 +599,11 @@ hipError_t launch_scan_rows(const TI* in, T* out, const double* aux, int64_t pla
 // load round trip plus a short sleep, 1 to 2 us; the sums of a band above normally arrive within
 // a few polls, and re-summing 32 rows costs a few microseconds, so 64 polls (about 100 us at
 // worst) bound the damage should workgroups ever be started out of order.
-// (both read at every call, so that a test can switch them within one process)
-int lookback_spin_limit() {
-    const char* e = getenv("BOXCONV_INTEGRAL_SPIN");
-    return e != nullptr ? std::max(0, atoi(e)) : 64;
-}
+int lookback_spin_limit() { return switches().spin_limit; }
 // BOXCONV_INTEGRAL_LOOKBACK=2: single-pass kernel for every shape it covers, not only those where
 // it was measured to be faster (used by the tests to reach its partial-row and partial-band code).
-bool lookback_any_shape() {
-    const char* e = getenv("BOXCONV_INTEGRAL_LOOKBACK");
-    return e != nullptr && atoi(e) == 2;
-}
-bool lookback_enabled() {
-    const char* e = getenv("BOXCONV_INTEGRAL_LOOKBACK");
-    return e == nullptr || atoi(e) != 0;
-}
+bool lookback_any_shape() { return switches().lookback_any_shape; }
+bool lookback_enabled() { return switches().lookback; }
 
 template <class TI, int WAVES>
 hipError_t launch_lookback(const TI* in, float* out, double* aux, int64_t planes, int h, int w,

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define BOXCONV_ABI_VERSION 1
+#define BOXCONV_ABI_VERSION 2
 
 #define BOXCONV_E_INVALID_ARGUMENT (-1) /* null pointer, non-positive size, ... */
 #define BOXCONV_E_WORKSPACE        (-2) /* workspace missing or smaller than *_workspace_bytes() */
@@ -42,6 +42,13 @@ int boxconv_abi_version(void);
 /* Message of the last error on this thread ("" if none). Never NULL; valid until the next call
  * on this thread. */
 const char* boxconv_last_error(void);
+
+/* The library's measurement and test switches (environment variables BOXCONV_*, listed in the
+ * integration notes) are read once, at the first call that needs them; no entry point calls getenv
+ * on its way to a launch. boxconv_reload_env() reads them again, for a test that changes one
+ * inside a running process. Not synchronised with calls in flight on other threads. No
+ * counterpart in the reference. */
+void boxconv_reload_env(void);
 
 /* ---- per-kernel timing (measurement aid; no counterpart in the reference) ---------------------
  * boxconv_profile_arm(name): from now on every launch of the kernel called `name` is bracketed by

@@ -18,9 +18,11 @@ def pytest_configure(config):
 def pytest_terminal_summary(terminalreporter):
     stats = getattr(sys.modules.get("test_gpu_parity"), "NOISE_STATS", None)
     if stats and stats["comparisons"]:
-        line = ("assert_parity: %(comparisons)d tensor comparisons, %(needed_noise_term)d passed only with the "
-                "rounding-noise term or the sibling scale (%(of_those_reference_all_zero)d of those have an "
-                "all-zero reference tensor)" % stats)
+        # (worded without "<number> passed" / "<number> failed": result parsers count those tokens)
+        line = ("assert_parity: of %(comparisons)d tensor comparisons, the rounding-noise term or the "
+                "sibling scale was needed in %(needed_noise_term)d (reference tensor zero, or a millionth of its "
+                "siblings, in %(of_those_reference_all_zero)d of those); largest diff / (tol * max|cpu|) among the "
+                "rest: %(worst_ratio).2f [%(worst_case)s]" % stats)
         terminalreporter.write_line(line)
         path = os.environ.get("BOXCONV_PARITY_REPORT")
         if path:
@@ -52,3 +54,26 @@ def hip():
     from box_convolution import _native
     _native.load()
     return _native
+
+
+@pytest.fixture
+def switches(hip):
+    """``switches(name, value)`` sets one of the library's BOXCONV_* environment switches (None
+    removes it) and makes the library read its environment again (it reads it once, at first
+    use); everything is put back, and re-read, when the test ends."""
+    saved = {}
+
+    def set_switch(name, value):
+        saved.setdefault(name, os.environ.get(name))
+        if value is None:
+            os.environ.pop(name, None)
+        else:
+            os.environ[name] = value
+        hip.reload_switches()
+    yield set_switch
+    for name, value in saved.items():
+        if value is None:
+            os.environ.pop(name, None)
+        else:
+            os.environ[name] = value
+    hip.reload_switches()

@@ -1,40 +1,51 @@
 """The five BASELINE workloads at full size on the GPU, through BoxConv2d (training mode, all
-five gradients), against the CPU oracle.
+five gradients), against the CPU oracle, on ALL input planes.
 
-Workloads 1 to 4 are compared in full. Workload 5 is compared on its first 16 of 128 input planes
-(box convolution is independent per input plane, and a parameter gradient only sums over the
-batch, so the oracle restricted to planes [0, c) reproduces exactly those slices of the full
-result), plus a size-independent property on the whole tensors: the adjoint identity
+Every workload also passes a size-independent property on the whole tensors: the adjoint identity
 <boxconv(x), g> = <x, grad_input(g)>.
 
 Every run prints its measured errors; with BOXCONV_PARITY_REPORT=<file> they are appended to that
 file as well (this is how profiles/parity_errors.txt is made).
 
-Tolerances: forward, grad_input 1e-4; parameter gradients 1e-3 (max|gpu-cpu| / max|cpu|).
+Tolerances, as max|gpu-cpu| / max|cpu| of the tensor itself, nothing added: forward and
+grad_input 1e-4, parameter gradients 1e-3.
 
-Workload 5 (inputs near 10.5, integral-image entries up to 2.2e7 where a float32 ulp is 2) is at
-the precision limit of the float32 reference itself: its parameter gradients are differences of
-two nearly equal terms (for a constant image the gradient of a normalised box vanishes), and the
-reference's float32 result deviates from the same algorithm run in float64 by about 2e-3
-(measured: y_max 1.8e-3), the GPU result by about 3e-4. There the GPU is held to 1e-3 against
-the float64 oracle and must be at least as close to it as the float32 oracle is; its distance to
-the float32 oracle is held to 1e-3 or, where the float32 oracle itself is further than that from
-float64, to the sum of the two distances to float64 (nothing but the reference's own rounding
-error may separate them).
+Workload 5 (128 planes of 1024 x 2048, inputs near 10.5, integral-image entries up to 2.2e7 where
+a float32 ulp is 2) is checked in chunks of 16 input planes (box convolution is independent per
+input plane, and a parameter gradient only sums over the batch, so the oracle restricted to
+planes [c0, c1) reproduces exactly those slices of the full result). There the reference's
+parameter gradients are dominated by the rounding of its own integral image (one float32 rounding
+per row, src/integral_image.cpp:28-31; the GPU stores correctly rounded sums), so the comparison
+is split into parts that each isolate one side:
+
+  (A) GPU step                         vs  oracle fed the GPU's integral image   1e-4 / 1e-3
+  (B) GPU backward fed the oracle's
+      float32 integral image           vs  oracle (the literal reference)        1e-4 / 1e-3
+  (C) GPU step                         vs  oracle (the literal reference)        1e-4 for forward and
+      grad_input; the parameter gradients are reported and bounded by 1e-3 plus what the oracle
+      itself moves by when its integral image is exchanged for the GPU's
+  (D) GPU step and oracle              vs  the oracle in float64                 GPU <= 1e-3 and at
+      least as close as the float32 oracle
+
+(A) and (B) are the statements "given the same integral image, GPU and reference agree to the
+stated tolerance", in both directions; tests/test_oracle_pins.py shows on the CPU alone that
+exchanging the reference's integral image for the correctly rounded one moves its parameter
+gradients by more than the tolerance at this workload's recipe.
 """
 import os
+from concurrent.futures import ThreadPoolExecutor
 
 import numpy as np
 import pytest
 import torch
 
-from baseline_workloads import make_workload
-from helpers import param_grad_floor, rel_err
+from baseline_workloads import make_workload, restrict
+from helpers import rel_err
 
 pytestmark = pytest.mark.gpu
 
-# planes the oracle is run on (None = all)
-ORACLE_PLANES = {1: None, 2: None, 3: None, 4: None, 5: 16}
+W5_CHUNK = 16      # input planes per oracle run of workload 5
+NAMES = ("x_min", "x_max", "y_min", "y_max")
 
 
 def report(line):
@@ -46,6 +57,7 @@ def report(line):
 
 
 def run_gpu(wl):
+    """One training step of BoxConv2d on the GPU; everything stays on the device."""
     from box_convolution import BoxConv2d
     dev = torch.device("cuda:0")
     module = BoxConv2d(wl.C, wl.F, wl.h, wl.w, wl.reparametrization_factor).to(dev)
@@ -61,55 +73,137 @@ def run_gpu(wl):
         assert torch.equal(p.detach().cpu(), v), "workload boxes must survive clipping unchanged"
     out.backward(g)
     torch.cuda.synchronize()
-    # adjoint identity on the full tensors, accumulated in float64 on the device
-    lhs = (out.detach().double() * g.double()).sum().item()
-    rhs = (x.detach().double() * x.grad.double()).sum().item()
-    scale = (out.detach().double().abs() * g.double().abs()).sum().item()
-    return (out.detach(), x.grad, [p.grad for p in (module.x_min, module.x_max, module.y_min, module.y_max)],
-            (lhs, rhs, scale))
+    # adjoint identity on the full tensors, accumulated in float64 on the device (chunked over the
+    # channel axis to bound the float64 temporaries)
+    lhs = rhs = scale = 0.0
+    F = wl.F
+    for c in range(wl.C):
+        o, gg = out.detach()[:, c * F:(c + 1) * F].double(), g[:, c * F:(c + 1) * F].double()
+        lhs += (o * gg).sum().item()
+        scale += (o.abs() * gg.abs()).sum().item()
+        rhs += (x.detach()[:, c].double() * x.grad[:, c].double()).sum().item()
+    return dict(out=out.detach(), gin=x.grad, x=x.detach(), g=g,
+                gpar=[p.grad for p in (module.x_min, module.x_max, module.y_min, module.y_max)],
+                adjoint=(lhs, rhs, scale))
 
 
-@pytest.mark.parametrize("k", [1, 2, 3, 4, 5])
+def real_boxes(wl, dtype=np.float32):
+    """Stored parameters times the reparametrization factor, rounded in float32 like the module's
+    `tensor * python float`."""
+    scales = (wl.reparametrization_h,) * 2 + (wl.reparametrization_w,) * 2
+    return [(p.numpy().astype(np.float32) * np.float32(s)).astype(dtype)
+            for p, s in zip((wl.x_min, wl.x_max, wl.y_min, wl.y_max), scales)]
+
+
+def oracle_step(oracle, integ, real, grad_out, wl):
+    out = oracle.box_forward(integ, *real, True, True)
+    grads = oracle.box_backward(integ, *real, grad_out, out, wl.reparametrization_h,
+                                wl.reparametrization_w, True, True)
+    return out, grads
+
+
+def fmt(errs):
+    return " ".join("%.2e" % e for e in errs)
+
+
+@pytest.mark.parametrize("k", [1, 2, 3, 4])
 def test_baseline_workload(oracle, k):
     wl = make_workload(k)
-    out, gin, gpar, (lhs, rhs, scale) = run_gpu(wl)
+    res = run_gpu(wl)
+    lhs, rhs, scale = res["adjoint"]
     assert abs(lhs - rhs) <= 2e-5 * scale, "adjoint identity <y,g> = <x,grad_input>: %r vs %r" % (lhs, rhs)
 
-    c = ORACLE_PLANES[k] or wl.C
-    sub = make_workload(k, in_planes=c)
-    args = [t.numpy() for t in (sub.x, sub.x_min, sub.x_max, sub.y_min, sub.y_max)]
-    out_c, saved = oracle.module_forward(*args, sub.reparametrization_h, sub.reparametrization_w, True, True)
-    grads_c = oracle.module_backward(saved, sub.grad_output.numpy(), sub.reparametrization_h,
-                                     sub.reparametrization_w, True, True)
-
-    F = wl.F
-    e_out = rel_err(out[:, :c * F].cpu().numpy(), out_c)
-    e_gin = rel_err(gin[:, :c].cpu().numpy(), grads_c[0])
-    floor = param_grad_floor(grads_c[1:])
-    e_par = [rel_err(gp[:c].cpu().numpy(), gc, floor) for gp, gc in zip(gpar, grads_c[1:])]
-    report("workload %d (%s), oracle on %d of %d input planes: adjoint identity |lhs-rhs|/sum|terms| %.2e; "
+    integ = oracle.integral_image(wl.x.numpy())
+    out_c, grads_c = oracle_step(oracle, integ, real_boxes(wl), wl.grad_output.numpy(), wl)
+    e_out = rel_err(res["out"].cpu().numpy(), out_c)
+    e_gin = rel_err(res["gin"].cpu().numpy(), grads_c[0])
+    e_par = [rel_err(gp.cpu().numpy(), gc) for gp, gc in zip(res["gpar"], grads_c[1:])]
+    report("workload %d (%s), oracle on all %d input planes: adjoint identity |lhs-rhs|/sum|terms| %.2e; "
            "max|gpu-cpu|/max|cpu|: forward %.2e grad_input %.2e grad_x_min %.2e grad_x_max %.2e "
            "grad_y_min %.2e grad_y_max %.2e"
-           % (k, wl.name, c, wl.C, abs(lhs - rhs) / scale, e_out, e_gin, *e_par))
+           % (k, wl.name, wl.C, abs(lhs - rhs) / scale, e_out, e_gin, *e_par))
     assert e_out <= 1e-4
     assert e_gin <= 1e-4
-    if k != 5:
-        assert max(e_par) <= 1e-3
-        return
+    assert max(e_par) <= 1e-3
 
-    # workload 5: the same algorithm in float64 on the same (float32-rounded) real-unit boxes
-    real = [(a.astype(np.float32) * np.float32(r)).astype(np.float64) for a, r in
-            zip(args[1:], (sub.reparametrization_h,) * 2 + (sub.reparametrization_w,) * 2)]
-    integ64 = oracle.integral_image(args[0].astype(np.float64))
-    out64 = oracle.box_forward(integ64, *real, True, True)
-    grads64 = oracle.box_backward(integ64, *real, sub.grad_output.numpy().astype(np.float64), out64,
-                                  sub.reparametrization_h, sub.reparametrization_w, True, True)
-    floor64 = param_grad_floor(grads64[1:])
-    e_gpu64 = [rel_err(gp[:c].cpu().numpy(), g64, floor64) for gp, g64 in zip(gpar, grads64[1:])]
-    e_cpu64 = [rel_err(gc, g64, floor64) for gc, g64 in zip(grads_c[1:], grads64[1:])]
-    report("workload 5 parameter gradients vs the float64 oracle (x_min x_max y_min y_max): gpu %s ; "
-           "float32 cpu oracle %s" % (" ".join("%.2e" % e for e in e_gpu64), " ".join("%.2e" % e for e in e_cpu64)))
-    assert max(e_gpu64) <= 1e-3
-    assert max(e_gpu64) <= max(max(e_cpu64), 1e-4)
-    for e, eg, ec in zip(e_par, e_gpu64, e_cpu64):
-        assert e <= max(1e-3, 1.05 * (eg + ec))
+
+# ---- workload 5 ---------------------------------------------------------------------------------
+@pytest.fixture(scope="module")
+def workload5(hip):
+    wl = make_workload(5)
+    res = run_gpu(wl)
+    res["integ"] = hip.integral_image(res["x"])       # what the module's forward integrated
+    torch.cuda.synchronize()
+    yield wl, res
+    res.clear()
+    torch.cuda.empty_cache()
+
+
+def test_workload5_adjoint_identity(workload5):
+    wl, res = workload5
+    lhs, rhs, scale = res["adjoint"]
+    report("workload 5 (%s): adjoint identity |lhs-rhs|/sum|terms| %.2e" % (wl.name, abs(lhs - rhs) / scale))
+    assert abs(lhs - rhs) <= 2e-5 * scale
+
+
+@pytest.mark.parametrize("c0", list(range(0, 128, W5_CHUNK)))
+def test_workload5_planes(hip, oracle, workload5, c0):
+    wl, res = workload5
+    c1, F = c0 + W5_CHUNK, wl.F
+    sub = restrict(wl, c0, c1)
+    x, g = sub.x.numpy(), sub.grad_output.numpy()
+    real = real_boxes(sub)
+    integ_gpu = res["integ"][:, c0:c1].cpu().numpy()
+    integ_own = oracle.integral_image(x)              # the reference's own float32 integral image
+
+    # (B)'s GPU side: the native backward on the oracle's integral image
+    real_dev = [torch.from_numpy(r).cuda() for r in real]
+    back_b = hip.box_convolution_backward(
+        torch.from_numpy(integ_own).cuda(), *real_dev, res["g"][:, c0 * F:c1 * F].contiguous(), None,
+        sub.reparametrization_h, sub.reparametrization_w, True, True, True, True, True, True, True)
+    back_b = [t.cpu().numpy() for t in back_b]
+
+    def in_double():
+        integ64 = oracle.integral_image(x.astype(np.float64))
+        return oracle_step(oracle, integ64, [r.astype(np.float64) for r in real], g.astype(np.float64), sub)
+    # the three oracle runs are independent and the checker releases the interpreter lock
+    with ThreadPoolExecutor(max_workers=3) as pool:
+        jobs = [pool.submit(oracle_step, oracle, integ_own, real, g, sub),
+                pool.submit(oracle_step, oracle, integ_gpu, real, g, sub),
+                pool.submit(in_double)]
+        (out_lit, grads_lit), (out_a, grads_a), (_, grads64) = [j.result() for j in jobs]
+
+    out = res["out"][:, c0 * F:c1 * F].cpu().numpy()
+    gin = res["gin"][:, c0:c1].cpu().numpy()
+    gpar = [gp[c0:c1].cpu().numpy() for gp in res["gpar"]]
+    tag = "workload 5 planes %3d..%3d" % (c0, c1 - 1)
+
+    # (A) same integral image (the GPU's) on both sides
+    e_a = [rel_err(out, out_a), rel_err(gin, grads_a[0])] + [rel_err(a, b) for a, b in zip(gpar, grads_a[1:])]
+    report("%s (A) gpu step vs oracle on the gpu's integral image: forward %.2e grad_input %.2e "
+           "grad_x_min %.2e grad_x_max %.2e grad_y_min %.2e grad_y_max %.2e" % (tag, *e_a))
+    # (B) same integral image (the reference's) on both sides
+    e_b = [rel_err(back_b[0], grads_lit[0])] + [rel_err(a, b) for a, b in zip(back_b[1:], grads_lit[1:])]
+    report("%s (B) gpu backward on the oracle's integral image vs oracle: grad_input %.2e "
+           "grad_x_min %.2e grad_x_max %.2e grad_y_min %.2e grad_y_max %.2e" % (tag, *e_b))
+    # (C) the literal comparison, and how far the oracle itself moves with the integral image
+    e_c = [rel_err(out, out_lit), rel_err(gin, grads_lit[0])] + [rel_err(a, b) for a, b in zip(gpar, grads_lit[1:])]
+    moved = [rel_err(a, b) for a, b in zip(grads_a[1:], grads_lit[1:])]
+    report("%s (C) gpu step vs oracle: forward %.2e grad_input %.2e grad_x_min %.2e grad_x_max %.2e "
+           "grad_y_min %.2e grad_y_max %.2e ; oracle on the gpu's integral image vs oracle on its own: %s"
+           % (tag, *e_c, fmt(moved)))
+    # (D) against the same algorithm in float64
+    e_gpu64 = [rel_err(a, b) for a, b in zip(gpar, grads64[1:])]
+    e_cpu64 = [rel_err(a, b) for a, b in zip(grads_lit[1:], grads64[1:])]
+    report("%s (D) parameter gradients vs the float64 oracle: gpu %s ; float32 oracle %s"
+           % (tag, fmt(e_gpu64), fmt(e_cpu64)))
+
+    assert e_a[0] <= 1e-4 and e_a[1] <= 1e-4, "(A) forward / grad_input"
+    assert max(e_a[2:]) <= 1e-3, "(A) parameter gradients"
+    assert e_b[0] <= 1e-4, "(B) grad_input"
+    assert max(e_b[1:]) <= 1e-3, "(B) parameter gradients"
+    assert e_c[0] <= 1e-4 and e_c[1] <= 1e-4, "(C) forward / grad_input"
+    for name, e, m in zip(NAMES, e_c[2:], moved):
+        assert e <= 1e-3 + m, "(C) grad_%s: beyond what the integral image's rounding accounts for" % name
+    assert max(e_gpu64) <= 1e-3, "(D)"
+    assert max(e_gpu64) <= max(max(e_cpu64), 1e-4), "(D) gpu further from float64 than the float32 oracle"

@@ -157,7 +157,7 @@ HALF_INTEGRAL_SHAPES = [(3, 96, 256), (2, 130, 1024), (2, 70, 2048), (3, 200, 36
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("planes,h,w", HALF_INTEGRAL_SHAPES)
-def test_integral_image_of_half_precision_input(hip, monkeypatch, planes, h, w, dtype):
+def test_integral_image_of_half_precision_input(hip, switches, planes, h, w, dtype):
     """float32 integral image straight from float16 / bfloat16: the same bits as converting the
     input to float32 first (which is pinned against the oracle in test_gpu_parity.py)."""
     x = (torch.randn(planes, h, w, device=DEV) * 3 + 0.5).to(dtype)
@@ -168,7 +168,7 @@ def test_integral_image_of_half_precision_input(hip, monkeypatch, planes, h, w, 
     flat = torch.empty(x.numel() + 1, device=DEV, dtype=dtype)
     shifted = flat[1:].view_as(x).copy_(x)
     assert shifted.data_ptr() % 8 != 0 and torch.equal(hip.integral_image(shifted), want)
-    monkeypatch.setenv("BOXCONV_INTEGRAL_LOOKBACK", "2")     # single pass wherever it applies
+    switches("BOXCONV_INTEGRAL_LOOKBACK", "2")     # single pass wherever it applies
     assert torch.equal(hip.integral_image(x), hip.integral_image(x.float()))
 
 

@@ -306,3 +306,47 @@ def test_split_identities(oracle):
         pi, pf = oracle.split(2, x0, x1, y0, y1, dtype=np.float64)
         assert np.array_equal(pi, ints - 1)
         assert np.allclose(pf, fr, atol=1e-12)
+
+
+# ---- what the rounding of the reference's integral image does to large-box gradients -----------
+def test_large_box_parameter_gradients_carry_the_integral_images_rounding(oracle):
+    """The recipe of the large-box workload (1024 x 2048 planes of uniform[0,1) + 10, boxes over
+    more than 80 % of the image): integral-image entries reach 2.2e7, where a float32 ulp is 2.
+    The reference rounds its integral image once per row (src/integral_image.cpp:28-31: the row
+    sum in double plus the float32 entry above, stored as float32), so an entry is off by up to a
+    few dozen ulps; the parameter gradients are differences of nearly equal sums of such entries.
+
+    Same float32 sampling code, same boxes, same grad_output, only the integral image exchanged
+    for the correctly rounded one (float64 sums rounded once): the y gradients move by more than
+    the 1e-3 they are compared at, towards the float64 result. This is why an implementation that
+    stores correctly rounded sums is compared with the reference on equal integral images at this
+    workload (tests/test_gpu_baseline_configs.py)."""
+    rng = np.random.default_rng(5)
+    C, F, h, w = 2, 2, 1024, 2048
+    x = rng.random((1, C, h, w), dtype=np.float32) + np.float32(10.0)
+    g = rng.standard_normal((1, C * F, h, w), dtype=np.float32)
+    boxes = make_boxes(rng, C, F, h, w, "large", away_from_integers=0.01)
+    own = oracle.integral_image(x)
+    i64 = oracle.integral_image(x.astype(np.float64))
+    rounded_once = i64.astype(np.float32)
+    ulp = np.spacing(np.float32(own.max()))
+    assert np.abs(own.astype(np.float64) - i64).max() > 8 * ulp          # the reference's drift
+    assert np.abs(rounded_once.astype(np.float64) - i64).max() <= 0.5 * ulp
+
+    def gradients(integ, dtype):
+        b = [p.astype(dtype) for p in boxes]
+        out = oracle.box_forward(integ, *b, True, True)
+        return oracle.box_backward(integ, *b, g.astype(dtype), out, 8.0 * h, 8.0 * w, True, True)[1:]
+    lit, once, dbl = gradients(own, np.float32), gradients(rounded_once, np.float32), gradients(i64, np.float64)
+    moved = [rel_err(a, b) for a, b in zip(lit, once)]
+    lit64 = [rel_err(a, b) for a, b in zip(lit, dbl)]
+    once64 = [rel_err(a, b) for a, b in zip(once, dbl)]
+    # the reference's own float32 result is more than the tolerance away from float64 ...
+    assert max(lit64) > 1.5e-3
+    # ... all of it from the integral image: with the correctly rounded one it is within 1e-4
+    assert max(once64) <= 1e-4
+    assert max(moved) > 1.5e-3
+    # and the x gradients hardly move: they sum differences of ADJACENT ROWS of the integral image,
+    # which are one rounding apart, while the y gradients sum differences of adjacent columns of
+    # box sums over some 900 rows, whose accumulated drifts are independent of each other
+    assert max(moved[:2]) <= 1e-4

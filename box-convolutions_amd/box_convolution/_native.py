@@ -102,11 +102,12 @@ def _require_device(t, what):
 
 
 def _stream(device):
-    """The current stream of `device` as a raw hipStream_t."""
+    """The current stream of `device` as a raw hipStream_t (an integer; 0 is the null stream,
+    which the C ABI takes as NULL)."""
     index = device.index
     if index is None:
         index = torch.cuda.current_device()
-    return ctypes.c_void_p(torch._C._cuda_getCurrentRawStream(index))
+    return torch._C._cuda_getCurrentRawStream(index) or None
 
 
 class _on_device:
@@ -130,13 +131,58 @@ class _on_device:
 
 
 def _ptr(t):
-    return None if t is None else ctypes.c_void_p(t.data_ptr())
+    """Device address as an integer (ctypes converts it to void*), None for a null pointer."""
+    return None if t is None else t.data_ptr()
 
 
-def _workspace(nbytes, device):
+# Scratch memory of the native calls. Every call needs it only until its own kernels have run, and
+# calls on one stream run in order, so one buffer per (device, stream), grown on demand, serves
+# them all: a training step then allocates no scratch (at the headline size the backward's is
+# 537 MB). While a stream is being captured into a graph the buffer comes from the allocator as
+# usual (the capture's own pool), because a cached buffer may be replaced, and so freed, by a
+# later, larger call while the graph still points at it.
+_workspaces = {}
+
+
+def _workspace(nbytes, device, stream):
     if nbytes == 0:
         return None
-    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+    if torch.cuda.is_current_stream_capturing():
+        return torch.empty(nbytes, dtype=torch.uint8, device=device)
+    key = (device.index, stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        _workspaces.pop(key, None)
+        ws = None                       # released before the larger one is requested
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def release_workspaces():
+    """Drop the cached scratch buffers (they are re-created on demand)."""
+    _workspaces.clear()
+
+
+# workspace sizes by call signature: the C ABI's *_workspace_bytes functions are pure
+_workspace_bytes = {}
+
+
+def _integral_workspace_bytes(lib, planes, h, w):
+    key = (planes, h, w)
+    n = _workspace_bytes.get(key)
+    if n is None:
+        n = _workspace_bytes[key] = lib.boxconv_integral_image_workspace_bytes(planes, h, w)
+    return n
+
+
+def _backward_workspace_bytes(lib, B, C, F, h, w, elem, want_input, want_params):
+    key = (B, C, F, h, w, elem, want_input, want_params)
+    n = _workspace_bytes.get(key)
+    if n is None:
+        n = _workspace_bytes[key] = lib.boxconv_backward_workspace_bytes(
+            B, C, F, h, w, elem, int(want_input), int(want_params))
+    return n
 
 
 _MAX_WIDENING_WIDTH = 2048     # widest row boxconv_integral_image_half_f32 reads directly
@@ -164,15 +210,16 @@ def integral_image(input):
         return output.zero_()
     planes = input.numel() // (h * w)
     with _on_device(input.device):
-        nbytes = lib.boxconv_integral_image_workspace_bytes(planes, h, w)
-        ws = _workspace(nbytes, input.device)
+        nbytes = _integral_workspace_bytes(lib, planes, h, w)
+        stream = _stream(input.device)
+        ws = _workspace(nbytes, input.device, stream)
         if half:
             rc = lib.boxconv_integral_image_half_f32(
                 _ptr(input), _FUSED_OUTPUT[input.dtype], _ptr(output), planes, h, w, _ptr(ws), nbytes,
-                _stream(input.device))
+                stream)
         else:
             rc = getattr(lib, "boxconv_integral_image_" + sfx)(
-                _ptr(input), _ptr(output), planes, h, w, _ptr(ws), nbytes, _stream(input.device))
+                _ptr(input), _ptr(output), planes, h, w, _ptr(ws), nbytes, stream)
     _check(rc, "integral_image")
     return output
 
@@ -195,7 +242,7 @@ def _same_kind(params, like, what):
         if p.dtype != like.dtype:
             raise RuntimeError("box_convolution: %s and parameters have different dtypes (%s, %s)"
                                % (what, like.dtype, p.dtype))
-        out.append(p.detach().contiguous())
+        out.append(p if p.is_contiguous() else p.contiguous())    # (only the address is used)
     return out
 
 
@@ -339,14 +386,18 @@ def box_convolution_backward(input_integrated, x_min, x_max, y_min, y_max, grad_
     grad_input = None
     if input_needs_grad:
         grad_input = (torch.empty if F > 0 else torch.zeros)((B, C, h, w), dtype=grad_output.dtype, device=dev)
-    grads = [torch.empty((C, F), dtype=dt, device=dev) if n else None for n in needs_p]
+    if all(needs_p):
+        grads = list(torch.empty((4, C, F), dtype=dt, device=dev).unbind(0))    # one allocation
+    else:
+        grads = [torch.empty((C, F), dtype=dt, device=dev) if n else None for n in needs_p]
     want_input = input_needs_grad and grad_input.numel() > 0 and F > 0
     want_params = any(needs_p) and C * F > 0
     if want_input or want_params:
         with _on_device(dev):
-            nbytes = lib.boxconv_backward_workspace_bytes(
-                B, C, F, h, w, input_integrated.element_size(), int(want_input), int(want_params))
-            ws = _workspace(nbytes, dev)
+            nbytes = _backward_workspace_bytes(lib, B, C, F, h, w, input_integrated.element_size(),
+                                               want_input, want_params)
+            stream = _stream(dev)
+            ws = _workspace(nbytes, dev, stream)
             if half:
                 rc = lib.boxconv_backward_half_f32(
                     _ptr(input_integrated), _ptr(x_min), _ptr(x_max), _ptr(y_min), _ptr(y_max),
@@ -354,7 +405,7 @@ def box_convolution_backward(input_integrated, x_min, x_max, y_min, y_max, grad_
                     float(reparametrization_h), float(reparametrization_w), int(bool(normalize)),
                     int(bool(exact)), _ptr(grad_input) if want_input else None,
                     *[_ptr(g) if want_params else None for g in grads],
-                    B, C, F, h, w, _ptr(ws), nbytes, _stream(dev))
+                    B, C, F, h, w, _ptr(ws), nbytes, stream)
             else:
                 rc = getattr(lib, "boxconv_backward_" + sfx)(
                     _ptr(input_integrated), _ptr(x_min), _ptr(x_max), _ptr(y_min), _ptr(y_max),
@@ -362,7 +413,7 @@ def box_convolution_backward(input_integrated, x_min, x_max, y_min, y_max, grad_
                     float(reparametrization_h), float(reparametrization_w), int(bool(normalize)),
                     int(bool(exact)), _ptr(grad_input) if want_input else None,
                     *[_ptr(g) if want_params else None for g in grads],
-                    B, C, F, h, w, _ptr(ws), nbytes, _stream(dev))
+                    B, C, F, h, w, _ptr(ws), nbytes, stream)
         _check(rc, "box_convolution_backward")
     return [grad_input] + grads
 
@@ -471,16 +522,17 @@ def training_forward(input, x_min, x_max, y_min, y_max, reparametrization_h, rep
     output = torch.empty((B, C * F, h, w), dtype=input.dtype, device=dev)
     real = torch.empty((4, C, F), dtype=input.dtype, device=dev)
     with _on_device(dev):
-        nbytes = lib.boxconv_integral_image_workspace_bytes(B * C, h, w)
-        ws = _workspace(nbytes, dev)
+        nbytes = _integral_workspace_bytes(lib, B * C, h, w)
+        stream = _stream(dev)
+        ws = _workspace(nbytes, dev, stream)
         rc = getattr(lib, "boxconv_training_forward_" + sfx)(
             _ptr(input), _ptr(x_min), _ptr(x_max), _ptr(y_min), _ptr(y_max), _ptr(real),
             _ptr(integrated), _ptr(output), B, C, F, h, w,
             float(reparametrization_h), float(reparametrization_w), float(max_input_h),
             float(max_input_w), int(bool(normalize)), int(bool(exact)), _ptr(ws), nbytes,
-            _stream(dev))
+            stream)
     _check(rc, "training_forward")
-    return integrated, output, (real[0], real[1], real[2], real[3])
+    return integrated, output, real.unbind(0)
 
 
 KERNEL_NAMES = ("band_colsum", "band_prefix", "band_scan", "forward_rows", "grad_output_stream",

@@ -68,8 +68,9 @@ class BoxConvolutionFunction(torch.autograd.Function):
             output = _native.box_convolution_forward_fused(
                 input_integrated, x_min, x_max, y_min, y_max, normalize, exact, input.dtype)
         elif clip_to is not None:
+            # (the native call only takes the parameters' addresses: nothing autograd could record)
             input_integrated, output, (x_min, x_max, y_min, y_max) = _native.training_forward(
-                input, x_min.detach(), x_max.detach(), y_min.detach(), y_max.detach(),
+                input, x_min, x_max, y_min, y_max,
                 reparametrization_h, reparametrization_w, clip_to[0], clip_to[1], normalize, exact)
         else:
             x_min, x_max, y_min, y_max = reparametrize(

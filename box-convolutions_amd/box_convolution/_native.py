@@ -544,6 +544,7 @@ def reload_switches():
     """Make the library read its BOXCONV_* environment switches again (it reads them once, at
     first use). For tests that change a switch inside a running process."""
     load().boxconv_reload_env()
+    _workspace_bytes.clear()        # the switches decide which kernels run, hence how much scratch
 
 
 def profile_arm(kernel_name, every=1):

@@ -177,6 +177,8 @@ inline bool force_gather_kernels() { return switches().force_gather; }
 // LDS bytes one workgroup may use on the current device (hipDeviceAttributeMaxSharedMemoryPerBlock,
 // looked up once per device; 0 if the query fails, which sends every shape to the gather kernels).
 size_t device_lds_limit();
+// Compute units of the current device (looked up once per device; 256 if the query fails).
+int compute_units();
 
 // Optional per-kernel timing (see boxconv_profile_arm in include/boxconv.h). When a kernel name is
 // armed, every launch of that kernel is bracketed by a pair of HIP events on its stream.

@@ -368,6 +368,16 @@ band_scan_rows_kernel(const TI* __restrict__ in, T* __restrict__ out, const doub
 constexpr int kLookbackRows = 32;     // band height limit: 32 rows x 4 columns per lane in registers
 constexpr int kLookbackBands = 64;
 constexpr unsigned long long kNotPublished = 0x7ff8deadbeef0001ull;
+// Scopes of the hand-over. All bands of a plane run on one XCD (see Progress below), so the
+// words only have to meet in that XCD's L2. The stores have workgroup scope: plain writes into the
+// L2 (the vector L1 is write-through); at agent scope every 8-byte store went through to memory
+// as a 32-byte write (measured: 16 MB of extra HBM writes per 4 MB of sums). The loads keep agent
+// scope, which is what makes them bypass the vector L1 (a workgroup-scope load may hit there and
+// would poll a stale line until its wait runs out). Should a publisher ever run on another XCD,
+// its words reach the poller late or never; the bounded wait then ends in the local
+// re-summation: slower, never wrong.
+constexpr int kPublishScope = __HIP_MEMORY_SCOPE_WORKGROUP;
+constexpr int kCollectScope = __HIP_MEMORY_SCOPE_AGENT;
 
 __global__ void __launch_bounds__(256) fill_marker_kernel(unsigned long long* dst, int64_t n) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
@@ -456,7 +466,7 @@ band_scan_lookback_kernel(const TI* __restrict__ in, float* __restrict__ out, do
         for (int v = 0; v < 4; ++v)
             if (c0 + v < w)
                 __hip_atomic_store(mine + v, static_cast<unsigned long long>(__double_as_longlong(own[v])),
-                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                   __ATOMIC_RELAXED, kPublishScope);
     }
 
     // -- column sums of the bands above, four bands per round trip: the first loads of a group
@@ -476,7 +486,7 @@ band_scan_lookback_kernel(const TI* __restrict__ in, float* __restrict__ out, do
 #pragma unroll
                 for (int v = 0; v < 4; ++v)
                     if (c0 + v < w)
-                        bits[u][v] = __hip_atomic_load(theirs + v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        bits[u][v] = __hip_atomic_load(theirs + v, __ATOMIC_RELAXED, kCollectScope);
             }
         }
 #pragma unroll
@@ -495,7 +505,7 @@ band_scan_lookback_kernel(const TI* __restrict__ in, float* __restrict__ out, do
 #pragma unroll
                 for (int v = 0; v < 4; ++v)
                     if (c0 + v < w) {
-                        bits[u][v] = __hip_atomic_load(theirs + v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        bits[u][v] = __hip_atomic_load(theirs + v, __ATOMIC_RELAXED, kCollectScope);
                         have[u] = have[u] && bits[u][v] != kNotPublished;
                     }
             }

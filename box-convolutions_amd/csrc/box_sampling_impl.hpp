@@ -57,7 +57,37 @@ struct FinalizeArgs {
     int n;                 // boxes
     float reparam_h, reparam_w;
     int normalize, exact;
+    const T* integ;        // integral image of the input, [batch][n / F planes][(h+1) x (w+1)]
+    const void* grad_out;  // [batch][n][h x w], elements of T (grad_dtype 0), f16_t (1) or bf16_t (2)
+    int grad_dtype, h, w, F;
 };
+
+// sum over batch and pixels of grad_output * (box sum with the FORWARD split, rounded mode), for
+// box k, by one wave; the total is valid in lane 63. Only used for the rare boxes described in
+// finalize_box: a plain loop over the pixels, 4 integral-image samples each.
+template <class T>
+__device__ __forceinline__ double forward_split_sum(const FinalizeArgs<T>& fa, const BoxParams<T>& prm,
+                                                 int k, int lane) {
+    const T xmin = prm.xmin[k], xmax = prm.xmax[k], ymin = prm.ymin[k], ymax = prm.ymax[k];
+    const BoxSplit<T> s = split_forward(xmin, xmax, ymin, ymax);
+    const int h = fa.h, w = fa.w;
+    const int64_t hw = static_cast<int64_t>(h) * w, ipl = static_cast<int64_t>(h + 1) * (w + 1);
+    const int c = k / fa.F, C = fa.n / fa.F;
+    double sum = 0.0;
+    for (int b = 0; b < fa.batch; ++b) {
+        const T* plane = fa.integ + (static_cast<int64_t>(b) * C + c) * ipl;
+        const int64_t g0 = (static_cast<int64_t>(b) * fa.n + k) * hw;
+        for (int64_t pix = lane; pix < hw; pix += 64) {
+            const int i = static_cast<int>(pix / w), j = static_cast<int>(pix % w);
+            T g;
+            if (fa.grad_dtype == 1)      g = static_cast<T>(widen(static_cast<const f16_t*>(fa.grad_out)[g0 + pix]));
+            else if (fa.grad_dtype == 2) g = static_cast<T>(widen(static_cast<const bf16_t*>(fa.grad_out)[g0 + pix]));
+            else                         g = static_cast<const T*>(fa.grad_out)[g0 + pix];
+            sum += static_cast<double>(g * gather_box<T, false>(plane, s, i, j, h, w));
+        }
+    }
+    return wave_sum_to_last(sum);
+}
 
 template <class T>
 __device__ __forceinline__ void finalize_box(const FinalizeArgs<T>& fa, const BoxParams<T>& prm,
@@ -77,9 +107,19 @@ __device__ __forceinline__ void finalize_box(const FinalizeArgs<T>& fa, const Bo
 #pragma unroll
         for (int m = 0; m < 5; ++m) sum[m] = fa.acc[k * 5 + m];
     }
-    if (lane != 63) return;
     const T xmin = prm.xmin[k], xmax = prm.xmax[k], ymin = prm.ymin[k], ymax = prm.ymax[k];
     const bool ex = fa.exact != 0;
+    // sum[4] = sum(grad_output * box sum) was taken with the split of the parameter-gradient pass
+    // (src/box_convolution.cpp:80-96); the reference multiplies grad_output with the saved forward
+    // OUTPUT (src/box_convolution_interface.cpp:355-358), i.e. the forward split (:22-38). The two
+    // cut a box at different whole pixels only when a lower bound lies so closely above an integer
+    // that `bound - 1` rounds to the integer below. In exact mode the border weights make up for
+    // it to the last digits; in rounded mode a whole row or column of the box is at stake, and the
+    // sum is taken again with the forward split (wave-uniform branch, next to never taken).
+    if (fa.normalize && !ex && fa.integ != nullptr && fa.grad_out != nullptr &&
+        (ceil(xmin) != ceil(xmin - T(1)) + T(1) || ceil(ymin) != ceil(ymin - T(1)) + T(1)))
+        sum[4] = forward_split_sum(fa, prm, k, lane);
+    if (lane != 63) return;
     const T inv_area = fa.normalize ? inverse_extent(xmin, xmax, ymin, ymax, ex, true, true) : T(1);
     const T s = fa.normalize ? static_cast<T>(sum[4]) * inv_area : T(0);   // sum(g * output)
 #pragma unroll
@@ -921,6 +961,8 @@ FinalizeArgs<T> finalize_args(const ParamFinish<T>& f) {
     for (int i = 0; i < 4; ++i) fa.g[i] = f.grad[i];
     fa.n = f.n_boxes; fa.reparam_h = f.reparam_h; fa.reparam_w = f.reparam_w;
     fa.normalize = f.normalize ? 1 : 0; fa.exact = f.exact ? 1 : 0;
+    fa.integ = f.integ; fa.grad_out = f.grad_out; fa.grad_dtype = f.grad_dtype; fa.h = f.h; fa.w = f.w;
+    fa.F = f.num_filters;
     return fa;
 }
 

@@ -325,8 +325,10 @@ int backward_impl(const T* integ, const T* x_min, const T* x_max, const T* y_min
         if (int rc = hip_result(boxconv::grad_params_begin(acc, n_boxes, s), "accumulator clear"))
             return rc;
 
+    const int grad_dtype = std::is_same<TG, T>::value ? 0 : std::is_same<TG, boxconv::f16_t>::value ? 1 : 2;
     const boxconv::ParamFinish<T> finish{acc, batch, L.acc_slots, {gx_min, gx_max, gy_min, gy_max},
-                                         n_boxes, reparam_h, reparam_w, normalize != 0, exact != 0};
+                                         n_boxes, reparam_h, reparam_w, normalize != 0, exact != 0,
+                                         integ, grad_output, grad_dtype, h, w, num_filters};
     bool finished = false;
     const int64_t planes = static_cast<int64_t>(batch) * in_planes;
     const boxconv::Dims d{in_planes, num_filters, h, w, planes, 0};

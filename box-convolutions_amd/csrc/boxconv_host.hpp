@@ -77,6 +77,13 @@ struct ParamFinish {
     int n_boxes;
     float reparam_h, reparam_w;
     bool normalize, exact;
+    // For the one case in which sum(grad_output * output) has to follow the FORWARD split of a
+    // box rather than the one the sums were taken with (see finalize_box): the integral image of
+    // the input, grad_output with its element type (0: T, 1: float16, 2: bfloat16), the image size.
+    const T* integ;
+    const void* grad_out;
+    int grad_dtype;
+    int h, w, num_filters;
 };
 
 // The column workspace M of the backward pass (written by grad_output_stream_launch, read by

@@ -255,13 +255,12 @@ def test_backward_lower_bound_one_ulp_above_an_integer(hip, oracle, h, w, exact)
     y_min = np.array([[just_above, just_above], [-7.25, np.nextafter(np.float32(-2.0), np.float32(0.0))]], np.float32)
     y_max = np.array([[6.4, 9.0], [3.75, 11.5]], np.float32)
     for normalize in (False, True):
-        # Rounded mode with normalisation: the reference's second summand uses the saved forward
-        # output (forward split), the GPU rebuilds sum(grad_output * output) with the split of the
-        # parameter-gradient pass; at these bounds the two differ by a whole row or column, so
-        # only the input gradient is compared there (in exact mode the border weight makes up for it).
-        needs = (True,) * 5 if (exact or not normalize) else (True, False, False, False, False)
+        # Rounded mode with normalisation: the reference's second summand multiplies grad_output with
+        # the saved forward output (forward split), while the sums of the grad_output pass follow the
+        # split of the parameter-gradient pass; at these bounds the two differ by a whole row or
+        # column, and the GPU takes that one sum again with the forward split (finalize_box).
         cpu, gpu, sc = run_both(hip, oracle, x, (x_min, x_max, y_min, y_max), 3.5 * h, 2.25 * w,
-                                normalize, exact, g, needs)
+                                normalize, exact, g)
         assert_parity(cpu, gpu, np.float32, "normalize=%s exact=%s" % (normalize, exact), **sc)
 
 

@@ -47,6 +47,7 @@ for _s in ("f32", "f64"):
 _SIGNATURES["boxconv_backward_half_f32"] = (
     _i, [_vp] * 6 + [_i, _f, _f, _i, _i] + [_vp] * 5 + [_i] * 5 + [_vp, _sz, _vp])
 _SIGNATURES["boxconv_integral_image_static_f32"] = (_i, [_vp, _vp, _i64, _i, _i, _vp])
+_SIGNATURES["boxconv_integral_image_int"] = (_i, [_vp, _vp, _i, _i64, _i, _i, _vp])
 _SIGNATURES["boxconv_integral_image_half_f32"] = (_i, [_vp, _i, _vp, _i64, _i, _i, _vp, _sz, _vp])
 _SIGNATURES["boxconv_forward_fused_f32"] = (_i, [_vp] * 6 + [_i] + [_vp] * 3 + [_i] * 8 + [_vp])
 
@@ -56,6 +57,8 @@ EXPORTED_SYMBOLS = tuple(sorted(_SIGNATURES))
 _FUSED_OUTPUT = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 
 _SUFFIX = {torch.float32: "f32", torch.float64: "f64"}
+# element type codes BOXCONV_U8 .. BOXCONV_I64
+_INT_DTYPE = {torch.uint8: 16, torch.int8: 17, torch.int16: 18, torch.int32: 19, torch.int64: 20}
 
 
 def load():
@@ -197,6 +200,8 @@ def integral_image(input):
     if input.dim() < 2:
         raise RuntimeError("integral image input must have >=2 dimensions")
     _require_device(input, "integral image input")
+    if input.dtype in _INT_DTYPE:
+        return _integral_image_int(input)
     half = input.dtype in (torch.float16, torch.bfloat16)
     h, w = input.shape[-2:]
     if half and (w > _MAX_WIDENING_WIDTH or (h + 1) * (w + 1) * 4 >= 2 ** 31):
@@ -220,6 +225,23 @@ def integral_image(input):
         else:
             rc = getattr(lib, "boxconv_integral_image_" + sfx)(
                 _ptr(input), _ptr(output), planes, h, w, _ptr(ws), nbytes, stream)
+    _check(rc, "integral_image")
+    return output
+
+
+def _integral_image_int(input):
+    """Integer tensors (the reference's CPU function takes every ATen type,
+    src/integral_image.cpp:14): exact sums, stored modulo 2^bits in the input's own type."""
+    lib = load()
+    input = input.contiguous()
+    h, w = input.shape[-2:]
+    output = torch.empty(tuple(input.shape[:-2]) + (h + 1, w + 1), dtype=input.dtype, device=input.device)
+    if h == 0 or w == 0:
+        return output.zero_()
+    planes = input.numel() // (h * w)
+    with _on_device(input.device):
+        rc = lib.boxconv_integral_image_int(_ptr(input), _ptr(output), _INT_DTYPE[input.dtype], planes,
+                                            h, w, _stream(input.device))
     _check(rc, "integral_image")
     return output
 
@@ -537,7 +559,8 @@ def training_forward(input, x_min, x_max, y_min, y_max, reparametrization_h, rep
 
 KERNEL_NAMES = ("band_colsum", "band_prefix", "band_scan", "forward_rows", "grad_output_stream",
                 "grad_input_cols", "param_grad_finalize", "fill_zero", "fill_marker", "clip",
-                "forward_gather", "grad_input_gather", "grad_params_gather")
+                "forward_gather", "grad_input_gather", "grad_params_gather", "int_row_prefix",
+                "int_col_prefix")
 
 
 def reload_switches():

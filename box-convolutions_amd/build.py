@@ -30,7 +30,8 @@ def _inst(tag, t, tg, part, same):
 
 
 SOURCES = [(s, s.replace(".hip", ".o"), []) for s in
-           ("box_sampling.hip", "box_forward.hip", "integral_image.hip", "box_misc.hip", "boxconv_c_abi.hip")]
+           ("box_sampling.hip", "box_forward.hip", "integral_image.hip", "integral_image_int.hip", "box_misc.hip",
+            "boxconv_c_abi.hip")]
 for _tag, _t, _tg in (("f32", "float", "float"), ("f64", "double", "double"),
                       ("f16", "float", "f16_t"), ("bf16", "float", "bf16_t")):
     for _part in (1, 2):

@@ -451,6 +451,24 @@ int boxconv_integral_image_f64(const double* in, double* out, int64_t planes, in
     return integral_image_impl<double>(in, out, planes, h, w, workspace, workspace_bytes, stream);
 }
 
+int boxconv_integral_image_int(const void* in, void* out, int dtype, int64_t planes, int h, int w,
+                               void* stream) {
+    if (planes < 0 || h < 1 || w < 1)
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "integral image: invalid sizes planes=%lld h=%d w=%d",
+                    static_cast<long long>(planes), h, w);
+    if (dtype < BOXCONV_U8 || dtype > BOXCONV_I64)
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "integral image: dtype %d is not one of BOXCONV_U8 .. BOXCONV_I64",
+                    dtype);
+    if (planes == 0) return 0;
+    if (in == nullptr || out == nullptr)
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "integral image: null tensor pointer");
+    if (planes * static_cast<int64_t>(h + 1) * (w + 1) > kMaxElems || planes * static_cast<int64_t>(h) > kMaxElems)
+        return fail(BOXCONV_E_TOO_LARGE, "integral image: output exceeds 2^31-1 elements");
+    return hip_result(boxconv::integral_image_int_launch(in, out, dtype, planes, h, w,
+                                                         static_cast<hipStream_t>(stream)),
+                      "integer integral image launch");
+}
+
 int boxconv_integral_image_static_f32(const float* in, float* out, int64_t planes, int h, int w,
                                       void* stream) {
     return integral_image_static_impl(in, out, planes, h, w, stream);

@@ -103,6 +103,16 @@ __device__ __forceinline__ double dpp_move(double keep, double v) {
     return __hiloint2double(hi, lo);
 }
 template <int Ctrl, int RowMask>
+__device__ __forceinline__ unsigned dpp_move(unsigned keep, unsigned v) {
+    return static_cast<unsigned>(dpp_move<Ctrl, RowMask>(static_cast<int>(keep), static_cast<int>(v)));
+}
+template <int Ctrl, int RowMask>
+__device__ __forceinline__ unsigned long long dpp_move(unsigned long long keep, unsigned long long v) {
+    const int lo = dpp_move<Ctrl, RowMask>(static_cast<int>(keep), static_cast<int>(v));
+    const int hi = dpp_move<Ctrl, RowMask>(static_cast<int>(keep >> 32), static_cast<int>(v >> 32));
+    return (static_cast<unsigned long long>(static_cast<unsigned>(hi)) << 32) | static_cast<unsigned>(lo);
+}
+template <int Ctrl, int RowMask>
 __device__ __forceinline__ float dpp_move(float keep, float v) {
     return __int_as_float(dpp_move<Ctrl, RowMask>(__float_as_int(keep), __float_as_int(v)));
 }

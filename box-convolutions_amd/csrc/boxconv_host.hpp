@@ -55,6 +55,12 @@ hipError_t integral_image_widening_launch(const TI* in, float* out, int64_t plan
                                           double* aux, const IntegralPlan& plan, hipStream_t stream);
 bool integral_image_widening_applies(int h, int w);
 
+// Integral image of an integer tensor (dtype: BOXCONV_U8 .. BOXCONV_I64 of include/boxconv.h),
+// every entry the exact sum modulo 2^bits; no workspace. The grid holds planes * h workgroups.
+constexpr int kIntU8 = 16, kIntI8 = 17, kIntI16 = 18, kIntI32 = 19, kIntI64 = 20;
+hipError_t integral_image_int_launch(const void* in, void* out, int dtype, int64_t planes, int h, int w,
+                                     hipStream_t stream);
+
 template <class T>
 hipError_t forward_launch(const T* integ, BoxParams<T> prm, T* out, Dims d, bool normalize,
                           bool exact, hipStream_t stream);

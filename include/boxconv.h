@@ -56,6 +56,7 @@ void boxconv_reload_env(void);
  * alone, whatever else the entry point launches). Names: "band_colsum", "band_prefix",
  * "band_scan", "forward_rows", "grad_output_stream", "grad_input_cols",
  * "param_grad_finalize", "fill_zero", "fill_marker", "clip", "forward_gather", "grad_input_gather",
+ * "int_row_prefix", "int_col_prefix",
  * "grad_params_gather".
  * NULL or "" disarms. Arming discards earlier measurements.
  * boxconv_profile_arm_every(name, n): the same, but only every n-th launch of that kernel (the
@@ -78,6 +79,19 @@ int boxconv_integral_image_f32(const float* in, float* out, int64_t planes, int 
                                void* workspace, size_t workspace_bytes, void* stream);
 int boxconv_integral_image_f64(const double* in, double* out, int64_t planes, int h, int w,
                                void* workspace, size_t workspace_bytes, void* stream);
+
+/* Integral image of an integer tensor. The reference's function takes every ATen type
+ * (AT_DISPATCH_ALL_TYPES, src/integral_image.cpp:14; wrapper src/integral_image_interface.cpp:8-27):
+ * the row sum runs in int64 and every entry is stored in the tensor's own type, so out holds the
+ * exact sums modulo 2^bits (src/integral_image.cpp:20-37). `dtype` selects the element type of
+ * both tensors. No workspace. Not used by BoxConv2d; two plain launches, not tuned. */
+#define BOXCONV_U8  16 /* uint8_t */
+#define BOXCONV_I8  17 /* int8_t */
+#define BOXCONV_I16 18 /* int16_t */
+#define BOXCONV_I32 19 /* int32_t */
+#define BOXCONV_I64 20 /* int64_t */
+int boxconv_integral_image_int(const void* in, void* out, int dtype, int64_t planes, int h, int w,
+                               void* stream);
 
 /* The same integral image for callers that cannot allocate or pass a workspace (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc). It has no counterpart in

@@ -38,8 +38,18 @@ inline int clampi(int v, int lo, int hi) { return std::max(lo, std::min(v, hi));
 // Integral image, src/integral_image.cpp:20-37. The running row sum lives in the accumulate type
 // (double for float and for double, at::acc_type<scalar_t,false>); the previous output row is
 // read back in scalar_t and the store rounds to scalar_t.
+// Integer tensors (AT_DISPATCH_ALL_TYPES, src/integral_image.cpp:14) accumulate in int64
+// (at::acc_type<integer, false>) and store back in their own type, i.e. modulo 2^bits.
+template <class T> struct AccumulateType { using type = double; };
+template <> struct AccumulateType<uint8_t> { using type = int64_t; };
+template <> struct AccumulateType<int8_t> { using type = int64_t; };
+template <> struct AccumulateType<int16_t> { using type = int64_t; };
+template <> struct AccumulateType<int32_t> { using type = int64_t; };
+template <> struct AccumulateType<int64_t> { using type = int64_t; };
+
 template <class T>
 void integral_image(const T* in, T* out, int64_t planes, int h, int w) {
+    using Acc = typename AccumulateType<T>::type;
     const int64_t W1 = w + 1;
     for (int64_t p = 0; p < planes; ++p) {
         const T* src = in + p * (int64_t)h * w;
@@ -49,7 +59,7 @@ void integral_image(const T* in, T* out, int64_t planes, int h, int w) {
             T* cur = dst + (int64_t)(row + 1) * W1;
             const T* prev = dst + (int64_t)row * W1;
             cur[0] = T(0);
-            double run = 0.0;
+            Acc run = 0;
             for (int col = 0; col < w; ++col) {
                 run += src[(int64_t)row * w + col];
                 cur[col + 1] = static_cast<T>(run + prev[col + 1]);
@@ -502,3 +512,15 @@ void grad_param_planes(const T* integ, const T* xmin, const T* xmax, const T* ym
 
 ORACLE_API(f32, float)
 ORACLE_API(f64, double)
+
+#define ORACLE_INT_INTEGRAL(SUFFIX, T)                                                            \
+    extern "C" int oracle_integral_image_##SUFFIX(const T* in, T* out, int64_t planes, int h,    \
+                                                  int w) {                                        \
+        integral_image<T>(in, out, planes, h, w);                                                 \
+        return 0;                                                                                 \
+    }
+ORACLE_INT_INTEGRAL(u8, uint8_t)
+ORACLE_INT_INTEGRAL(i8, int8_t)
+ORACLE_INT_INTEGRAL(i16, int16_t)
+ORACLE_INT_INTEGRAL(i32, int32_t)
+ORACLE_INT_INTEGRAL(i64, int64_t)

@@ -21,6 +21,9 @@ ORACLE_LIB = os.path.join(_HERE, "libboxconv_oracle.so")
 REF_LIB = os.path.join(_HERE, "_ref", "libboxconv_ref.so")
 
 _SUFFIX = {np.dtype(np.float32): "f32", np.dtype(np.float64): "f64"}
+# the integral image alone also takes the integer types (src/integral_image.cpp:14)
+_INT_SUFFIX = {np.dtype(np.uint8): "u8", np.dtype(np.int8): "i8", np.dtype(np.int16): "i16",
+               np.dtype(np.int32): "i32", np.dtype(np.int64): "i64"}
 
 
 def build(with_reference=True):
@@ -57,6 +60,14 @@ class CpuChecker:
 
     # -- the four functions of the reference's native module (src/bind.cpp:29-34) --------------
     def integral_image(self, x):
+        x = np.ascontiguousarray(x)
+        if x.dtype in _INT_SUFFIX:
+            h, w = x.shape[-2:]
+            planes = x.size // (h * w) if x.size else 0
+            out = np.empty(x.shape[:-2] + (h + 1, w + 1), dtype=x.dtype)
+            getattr(self.lib, "%sintegral_image_%s" % (self.prefix, _INT_SUFFIX[x.dtype]))(
+                _ptr(x), _ptr(out), ctypes.c_int64(planes), h, w)
+            return out
         x = _c(x)
         h, w = x.shape[-2:]
         planes = x.size // (h * w) if x.size else 0

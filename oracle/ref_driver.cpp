@@ -233,3 +233,18 @@ void split_impl(int variant, const T* p4, int* ints, T* fracs) {
 
 REF_API(f32, float)
 REF_API(f64, double)
+
+// the reference's integral image of integer tensors (AT_DISPATCH_ALL_TYPES)
+#define REF_INT_INTEGRAL(SUFFIX, T)                                                               \
+    extern "C" int ref_integral_image_##SUFFIX(const T* in, T* out, int64_t planes, int h,       \
+                                               int w) {                                           \
+        at::Tensor i = view_of(in, {planes, h, w});                                               \
+        at::Tensor o = view_of(out, {planes, h + 1, w + 1});                                      \
+        cpu::integral_image(i, o);                                                                \
+        return 0;                                                                                 \
+    }
+REF_INT_INTEGRAL(u8, uint8_t)
+REF_INT_INTEGRAL(i8, int8_t)
+REF_INT_INTEGRAL(i16, int16_t)
+REF_INT_INTEGRAL(i32, int32_t)
+REF_INT_INTEGRAL(i64, int64_t)

@@ -58,6 +58,10 @@ def test_argument_errors_are_reported_without_launching(lib):
     assert rc == -1 and b"null" in lib.boxconv_last_error()
     rc = lib.boxconv_integral_image_half_f32(null, 0, null, 1, 4, 4, null, 0, null)
     assert rc == -1 and b"input_dtype" in lib.boxconv_last_error()
+    rc = lib.boxconv_integral_image_int(null, null, 3, 1, 4, 4, null)
+    assert rc == -1 and b"BOXCONV_U8" in lib.boxconv_last_error()
+    rc = lib.boxconv_integral_image_int(null, null, 19, 1, 4, 4, null)
+    assert rc == -1 and b"null" in lib.boxconv_last_error()
     dummy16 = ctypes.c_void_p(256)
     rc = lib.boxconv_integral_image_half_f32(dummy16, 1, dummy16, 1, 4, 4096, null, 0, null)
     assert rc == -3 and b"2048" in lib.boxconv_last_error()

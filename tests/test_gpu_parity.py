@@ -84,6 +84,27 @@ def test_integral_image_single_pass_waits_are_bounded(hip, switches, planes, h, 
     assert torch.allclose(three, usual, rtol=2e-7, atol=0) and torch.allclose(hip.integral_image(x), usual, rtol=2e-7, atol=0)
 
 
+INT_TYPES = [(np.uint8, torch.uint8), (np.int8, torch.int8), (np.int16, torch.int16),
+             (np.int32, torch.int32), (np.int64, torch.int64)]
+
+
+@pytest.mark.parametrize("np_dtype,torch_dtype", INT_TYPES)
+@pytest.mark.parametrize("shape", [(1, 1, 1), (3, 5, 7), (2, 33, 257), (1, 70, 2500), (2, 2, 130, 1024), (1, 300, 3)])
+def test_integral_image_of_integer_tensors(hip, oracle, shape, np_dtype, torch_dtype):
+    """Integer tensors (src/integral_image.cpp:14): bit-exact against the oracle and against
+    numpy's wrapping cumulative sums, with values over the type's full range."""
+    rng = np.random.default_rng(sum(shape) + np.dtype(np_dtype).itemsize)
+    info = np.iinfo(np_dtype)
+    x = rng.integers(info.min, info.max, size=shape, dtype=np_dtype, endpoint=True)
+    got = hip.integral_image(torch.from_numpy(x).cuda())
+    assert got.dtype == torch_dtype and tuple(got.shape) == shape[:-2] + (shape[-2] + 1, shape[-1] + 1)
+    got = got.cpu().numpy()
+    want = np.zeros(got.shape, dtype=np_dtype)
+    want[..., 1:, 1:] = x.cumsum(-2, dtype=np_dtype).cumsum(-1, dtype=np_dtype)
+    assert np.array_equal(got, oracle.integral_image(x))
+    assert np.array_equal(got, want)
+
+
 def test_integral_image_leading_dims(hip, oracle):
     x = np.random.default_rng(5).random((2, 3, 2, 17, 19)).astype(np.float32)
     got = host(hip.integral_image(dev(x)))

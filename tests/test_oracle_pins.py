@@ -308,6 +308,28 @@ def test_split_identities(oracle):
         assert np.allclose(pf, fr, atol=1e-12)
 
 
+INT_DTYPES = [np.uint8, np.int8, np.int16, np.int32, np.int64]
+
+
+@pytest.mark.parametrize("dtype", INT_DTYPES)
+def test_integer_integral_image_is_wrapping_cumsum(oracle, dtype):
+    """Integer tensors (the reference dispatches on every ATen type, src/integral_image.cpp:14):
+    the exact sums modulo 2^bits, i.e. numpy's cumulative sums in the same type, full-range
+    values included. Where the compiled reference exists it gives the same bits."""
+    rng = np.random.default_rng(np.dtype(dtype).itemsize)
+    info = np.iinfo(dtype)
+    for shape in [(3, 37, 41), (1, 1, 1), (2, 5, 300), (2, 2, 130, 7)]:
+        x = rng.integers(info.min, info.max, size=shape, dtype=dtype, endpoint=True)
+        want = np.zeros(shape[:-2] + (shape[-2] + 1, shape[-1] + 1), dtype=dtype)
+        want[..., 1:, 1:] = x.cumsum(-2, dtype=dtype).cumsum(-1, dtype=dtype)
+        got = oracle.integral_image(x)
+        assert got.dtype == x.dtype and np.array_equal(got, want)
+        from oracle import cpu_checker
+        ref = cpu_checker.reference()
+        if ref is not None:
+            assert np.array_equal(ref.integral_image(x), want)
+
+
 # ---- what the rounding of the reference's integral image does to large-box gradients -----------
 def test_large_box_parameter_gradients_carry_the_integral_images_rounding(oracle):
     """The recipe of the large-box workload (1024 x 2048 planes of uniform[0,1) + 10, boxes over

@@ -83,6 +83,51 @@ def load():
     return lib
 
 
+GLUE_NAME = "_boxconv_glue"
+GLUE_PATH = os.path.join(_HERE, GLUE_NAME + ".so")
+_glue = None          # the module, or False once loading was tried without success
+
+
+def glue():
+    """The C++ autograd node of the training step (csrc/torch_glue.cpp), or None where that
+    extension was not built: an optional fast path for the HOST side of a step (checks,
+    allocations, autograd callbacks in C++ instead of Python). It calls the same entry points of
+    libboxconv_hip.so, handed over here as addresses, so results do not depend on it; set
+    BOXCONV_PYTHON_GLUE=1 to keep it out."""
+    global _glue
+    if _glue is None:
+        _glue = False
+        if os.path.isfile(GLUE_PATH) and os.environ.get("BOXCONV_PYTHON_GLUE") != "1":
+            import importlib.util
+            import warnings
+            lib = load()
+            try:
+                spec = importlib.util.spec_from_file_location(GLUE_NAME, GLUE_PATH)
+                module = importlib.util.module_from_spec(spec)
+                spec.loader.exec_module(module)
+            except (ImportError, OSError) as exc:      # e.g. built against another torch
+                warnings.warn("box_convolution: %s could not be loaded (%s); the training step keeps "
+                              "its Python glue (same kernels, more host time per step)" % (GLUE_PATH, exc))
+                return None
+            module.init(*[ctypes.cast(getattr(lib, name), ctypes.c_void_p).value for name in (
+                "boxconv_training_forward_f32", "boxconv_training_forward_f64", "boxconv_backward_f32",
+                "boxconv_backward_f64", "boxconv_integral_image_workspace_bytes",
+                "boxconv_backward_workspace_bytes", "boxconv_last_error")])
+            _glue = module
+    return _glue or None
+
+
+def training_step(input, x_min, x_max, y_min, y_max, reparametrization_h, reparametrization_w,
+                  max_input_h, max_input_w, normalize, exact):
+    """``BoxConv2d.forward`` in training mode through the C++ autograd node: clips the stored
+    parameters in place, returns the output; its backward gives the five gradients. Same native
+    calls as ``BoxConvolutionFunction`` with ``clip_to``. Requires ``glue()``."""
+    return _glue.training_step(
+        input, x_min, x_max, y_min, y_max, float(reparametrization_h), float(reparametrization_w),
+        float(max_input_h), float(max_input_w), bool(normalize), bool(exact),
+        _stream(input.device) or 0, torch.cuda.is_current_stream_capturing())
+
+
 def _check(rc, what):
     if rc != 0:
         msg = load().boxconv_last_error().decode("utf-8", "replace")
@@ -165,6 +210,8 @@ def _workspace(nbytes, device, stream):
 def release_workspaces():
     """Drop the cached scratch buffers (they are re-created on demand)."""
     _workspaces.clear()
+    if _glue:
+        _glue.release_workspaces()
 
 
 # workspace sizes by call signature: the C ABI's *_workspace_bytes functions are pure

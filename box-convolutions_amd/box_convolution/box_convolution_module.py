@@ -169,6 +169,7 @@ class BoxConv2d(torch.nn.Module):
         return self
 
     _HALF_TYPES = (torch.float16, torch.bfloat16)
+    _GLUE_TYPES = (torch.float32, torch.float64)
 
     def forward(self, input):
         if input.dtype in self._HALF_TYPES:
@@ -176,6 +177,12 @@ class BoxConv2d(torch.nn.Module):
         clip_to = None
         if self.training:
             if self.x_min.is_cuda and input.is_cuda and input.dim() == 4 and input.dtype == self.x_min.dtype:
+                if _native.glue() is not None and input.dtype in self._GLUE_TYPES:
+                    # the whole step's host side in C++ (same native calls, autograd node included)
+                    return _native.training_step(
+                        input, self.x_min, self.x_max, self.y_min, self.y_max,
+                        self.reparametrization_h, self.reparametrization_w,
+                        self.max_input_h, self.max_input_w, self.normalize, self.exact)
                 # the projection rides along in the native forward call
                 clip_to = (self.max_input_h, self.max_input_w)
             else:

@@ -62,6 +62,34 @@ def _stale(target, deps):
     return any(os.path.getmtime(d) > t for d in deps)
 
 
+GLUE_SRC = os.path.join(CSRC, "torch_glue.cpp")
+GLUE_PATH = os.path.join(HERE, "box_convolution", "_boxconv_glue.so")
+
+
+def build_glue(force=False, verbose=True):
+    """The C++ autograd node of the training step (csrc/torch_glue.cpp): a Python extension module
+    compiled with g++ against the installed torch's headers. It holds no kernels and does not link
+    to libboxconv_hip.so (it is handed that library's entry points as addresses at start-up)."""
+    if not (force or _stale(GLUE_PATH, [GLUE_SRC, os.path.abspath(__file__)])):
+        return GLUE_PATH
+    import sysconfig
+    import torch
+    from torch.utils import cpp_extension
+    cxx = shutil.which("g++") or "g++"
+    tdir = os.path.dirname(torch.__file__)
+    cmd = [cxx, "-O2", "-fPIC", "-std=c++17", "-shared", "-w",
+           "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI),
+           "-DTORCH_EXTENSION_NAME=_boxconv_glue", "-DTORCH_API_INCLUDE_EXTENSION_H"]
+    cmd += ["-I" + d for d in cpp_extension.include_paths()]
+    cmd += ["-I" + sysconfig.get_paths()["include"], GLUE_SRC, "-o", GLUE_PATH,
+            "-L" + os.path.join(tdir, "lib"), "-lc10", "-ltorch_cpu", "-ltorch", "-ltorch_python",
+            "-Wl,-rpath," + os.path.join(tdir, "lib")]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return GLUE_PATH
+
+
 def build(force=False, verbose=True):
     os.makedirs(OBJ_DIR, exist_ok=True)
     hipcc = _hipcc()
@@ -86,6 +114,7 @@ def build(force=False, verbose=True):
 
     if force or jobs or _stale(LIB_PATH, objs):
         run([hipcc, "-shared", "-fPIC", "--offload-arch=" + ARCH, "-o", LIB_PATH] + objs)
+    build_glue(force=force, verbose=verbose)
     return LIB_PATH
 
 

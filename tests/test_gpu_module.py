@@ -284,8 +284,9 @@ def test_noncontiguous_input_and_dtype_errors(hip):
     assert not x.is_contiguous()
     assert torch.equal(hip.integral_image(x), hip.integral_image(x.contiguous()))
     with pytest.raises(RuntimeError, match="float32 or float64"):
-        hip.integral_image(torch.zeros(1, 4, 4, device=DEV, dtype=torch.int32))
-    # (float16 / bfloat16 inputs are integrated into float32: test_gpu_fused_forward.py)
+        hip.integral_image(torch.zeros(1, 4, 4, device=DEV, dtype=torch.bool))
+    # (float16 / bfloat16 inputs are integrated into float32: test_gpu_fused_forward.py; integer
+    # tensors in their own type: test_gpu_parity.py)
     z = torch.zeros(2, 1, device=DEV)
     with pytest.raises(RuntimeError, match="as many rows"):
         hip.box_convolution_forward(torch.zeros(1, 3, 5, 5, device=DEV), z, z, z, z, True, True)
@@ -351,3 +352,63 @@ def test_training_forward_in_one_native_call(shape, dtype):
     for a, b in zip(got_real, real):
         assert torch.equal(a, b)
     assert torch.equal(got_integ, integ) and torch.equal(got_out, out)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("needs", [(True, True, True, True, True), (False, True, True, True, True),
+                                   (True, False, False, False, False), (True, True, False, False, True)])
+def test_cpp_autograd_node_matches_the_python_function(hip, dtype, needs):
+    """BoxConv2d.forward in training mode goes through the C++ autograd node where that extension
+    was built; BoxConvolutionFunction with `clip_to` is the same step in Python. Same native
+    calls, so output, clipped parameters and every requested gradient agree bit for bit, and
+    gradients that were not requested stay None."""
+    if hip.glue() is None:
+        pytest.skip("the C++ glue was not built")
+    B, C, F, h, w = 2, 3, 4, 40, 130
+    random.seed(5)
+    torch.manual_seed(5)
+    modules = [BoxConv2d(C, F, h, w).to(DEV, dtype) for _ in range(2)]
+    modules[1].load_state_dict(modules[0].state_dict())
+    x0 = torch.randn(B, C, h, w, device=DEV, dtype=dtype)
+    g = torch.randn(B, C * F, h, w, device=DEV, dtype=dtype)
+    results = []
+    for which, m in enumerate(modules):
+        with torch.no_grad():
+            m.x_min.mul_(2.0)          # some boxes out of bounds: the clip has work to do
+        names = ("x_min", "x_max", "y_min", "y_max")
+        for name, need in zip(names, needs[1:]):
+            getattr(m, name).requires_grad_(need)
+        x = x0.clone().requires_grad_(needs[0])
+        m.train()
+        if which == 0:
+            out = m(x)                                                      # C++ node
+            assert type(out.grad_fn).__name__ != "BoxConvolutionFunctionBackward"
+        else:
+            out = BoxConvolutionFunction.apply(
+                x, m.x_min, m.x_max, m.y_min, m.y_max, m.reparametrization_h, m.reparametrization_w,
+                m.normalize, m.exact, (m.max_input_h, m.max_input_w))      # Python function
+        out.backward(g)
+        results.append((out.detach(), x.grad, [getattr(m, n).grad for n in names],
+                        [getattr(m, n).detach().clone() for n in names]))
+    (out_a, gx_a, gp_a, p_a), (out_b, gx_b, gp_b, p_b) = results
+    assert torch.equal(out_a, out_b)
+    assert (gx_a is None) == (not needs[0]) and (gx_b is None) == (not needs[0])
+    if needs[0]:
+        assert torch.equal(gx_a, gx_b)
+    for a, b, need in zip(gp_a, gp_b, needs[1:]):
+        assert (a is None) == (not need) and (b is None) == (not need)
+        if need:
+            assert torch.equal(a, b)
+    for a, b in zip(p_a, p_b):
+        assert torch.equal(a, b)
+
+
+def test_cpp_autograd_node_reports_the_reference_errors(hip):
+    if hip.glue() is None:
+        pytest.skip("the C++ glue was not built")
+    m = BoxConv2d(2, 3, 8, 8).to(DEV)
+    m.train()
+    with pytest.raises(RuntimeError, match="as many rows as there are input channels"):
+        m(torch.zeros(1, 5, 8, 8, device=DEV))
+    with pytest.raises(AssertionError):
+        BoxConv2d(2, 3, 8, 8, stride_h=2)

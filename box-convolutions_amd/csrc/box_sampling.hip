@@ -28,6 +28,7 @@ Switches read_switches() {
     e = text("BOXCONV_INTEGRAL_LOOKBACK");
     s.lookback = e == nullptr || std::atoi(e) != 0;
     s.lookback_any_shape = e != nullptr && std::atoi(e) == 2;
+    s.stream_consecutive = flag_unless_zero("BOXCONV_STREAM_CONSEC");
     e = text("BOXCONV_INTEGRAL_SPIN");
     s.spin_limit = e != nullptr ? std::max(0, std::atoi(e)) : 64;
     s.fwd_threads = threads("BOXCONV_FWD_THREADS", 512);

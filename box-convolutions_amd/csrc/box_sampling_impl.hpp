@@ -887,6 +887,362 @@ grad_output_stream_kernel(SampleArgs<T> a) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// The same pass for float rows that fill the workgroup's column slots exactly (w == 4 * NT), both
+// products at once: a lane owns 4 CONSECUTIVE columns for everything, where
+// grad_output_stream_kernel gives it the columns lane, lane + 64, ... of its wave and moves the
+// weights W through LDS to get consecutive ones for the suffix sum. With consecutive columns
+//   * the taps of a lane's 4 columns are two runs of 5 adjacent row pairs in LDS (3 instructions
+//     each) instead of 16 separate pairs,
+//   * W is where the suffix sum needs it: no LDS round trip, no wave barrier in the middle of a
+//     row pair,
+//   * the integral rows and grad_output come as one 16-byte load per lane and row (the integral
+//     rows start at an odd element, so theirs are only dword-aligned, which global loads allow),
+//   * wave totals and tails travel as one 16-byte word per wave.
+// Same arithmetic, same order of additions inside a lane's row pair; the sums differ from the
+// other kernel's only in which columns share a lane. Everything said there about the math, the
+// two splits, the single barrier per row pair (MERGED) and the cache policy of the stores applies.
+typedef float f4_dword_aligned __attribute__((ext_vector_type(4), aligned(4)));
+__device__ __forceinline__ void load4_dword_aligned(const float* p, float (&v)[4]) {
+    const f4_dword_aligned q = *reinterpret_cast<const f4_dword_aligned*>(p);
+    v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+}
+
+// Two waves per SIMD on purpose, although the registers would allow three: with three, more
+// workgroups are resident per XCD than share one integral plane of the input, two planes compete
+// for its L2, and the kernel gets slower (226 against 217 us at 512 x 1024).
+template <class TG, int NT, bool EXACT>
+__global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2)))
+grad_output_stream_consec_kernel(SampleArgs<float> a) {
+    using T = float;
+    constexpr int K = 4;
+    constexpr int kPad = 8;                          // zero pairs in front of and behind a row in LDS
+    constexpr int GLEN = K * NT + 2 * kPad;
+    constexpr int WAVES = NT / 64;
+    constexpr bool MERGED = NT <= 256;
+    struct alignas(16) WaveSums { T tot0, tot1, tail0, tail1; };
+    struct alignas(16) LastColumn { T v, dt, db, unused; };      // V, DT, DB at column w
+    __shared__ __align__(16) RowPair<T> grow[2][GLEN];
+    __shared__ __align__(16) T delta[K * NT];
+    __shared__ WaveSums wsum[2][WAVES];
+    __shared__ LastColumn xw[2][2];
+    __shared__ double red[5 * WAVES];
+
+    const unsigned vid = xcd_contiguous_id(a.per_xcd);
+    if (vid >= a.total) return;                      // whole workgroup leaves together
+    const unsigned nbands = a.nb, nfilt = a.F;
+    const int band = static_cast<int>(vid % nbands);
+    const unsigned pf32 = vid / nbands;
+    const int f = static_cast<int>(pf32 % nfilt);
+    const int64_t pf = pf32, p = pf32 / nfilt;
+    const int k_par = static_cast<int>(static_cast<unsigned>(a.plane0 + p) % static_cast<unsigned>(a.C)) * a.F + f;
+    const int h = a.h, w = a.w, tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int c0 = K * tid;                          // the lane's first pixel column
+
+    const BoxOfWorkgroup<T> bx = load_box(a.prm, k_par);
+    const BoxSplit<T> s = split_grad_params(bx.xmin, bx.xmax, bx.ymin, bx.ymax);
+    const BoxSplit<T> sm = split_grad_input(bx.xmin, bx.xmax, bx.ymin, bx.ymax);
+    const int ylo_m = 1 - sm.yhi, yhi_m = 1 - sm.ylo;
+    const bool own_w = ylo_m != s.ylo || yhi_m != s.yhi;                        // workgroup-uniform
+
+    const int64_t pitch = w + 1;
+    const int64_t mpitch = a.mpitch;
+    const T* iplane = a.src + p * static_cast<int64_t>(h + 1) * pitch;        // integral of the input
+    const TG* gplane = reinterpret_cast<const TG*>(a.grad_out) + pf * static_cast<int64_t>(h) * w;
+    T* mrows = a.dst + pf * static_cast<int64_t>(h + 1) * mpitch;
+    const unsigned from_end = static_cast<unsigned>(a.per_xcd) - 1u - vid % static_cast<unsigned>(a.per_xcd);
+    const bool keep_in_cache =
+        static_cast<uint64_t>(from_end) * a.R * mpitch * sizeof(T) < static_cast<uint64_t>(a.keep_tail);
+    const Rows<T, true> mout(mrows, mpitch, static_cast<int>(mpitch), h + 1);
+
+    const int i0 = band * a.R;
+    const int i1 = min(h, i0 + a.R);
+
+    // integral row r, columns c0+1 .. c0+4; rows of grad_output, columns c0 .. c0+3 (a row past the
+    // band is read from a valid address and cleared afterwards)
+    auto load_i = [&](int r, T (&dst)[K]) {
+        load4_dword_aligned(iplane + static_cast<int64_t>(r) * pitch + 1 + c0, dst);
+    };
+    auto load_g = [&](int i, T (&dst)[K]) {
+        load_quad(gplane + static_cast<int64_t>(min(i, h - 1)) * w + c0, dst);
+    };
+    auto load_window = [&](int i, T (&t0)[K], T (&t1)[K], T (&b1)[K], T (&b2)[K]) {
+        load_i(clampi(i + s.xlo, 0, h), t0);
+        load_i(clampi(i + 1 + s.xlo, 0, h), t1);
+        load_i(clampi(i + 1 + s.xhi, 0, h), b1);
+        load_i(clampi(i + 2 + s.xhi, 0, h), b2);
+    };
+
+    T g0[K], g1[K];
+    load_g(i0, g0);
+    load_g(i0 + 1, g1);
+
+    // pads of both LDS rows, row 0 of the column workspace
+    if (tid < 2 * kPad) {
+        const int e = tid < kPad ? tid : K * NT + tid;
+        grow[0][e] = RowPair<T>{T(0), T(0)};
+        grow[1][e] = RowPair<T>{T(0), T(0)};
+    }
+    if (band == 0)
+        for (int c = tid; c < mpitch; c += NT) mrows[c] = T(0);
+
+    auto tail_weight = [&](int j, int ylo, int yhi, T fylo, T fyhi) {
+        const T one = T(1);
+        return (EXACT ? (one - fyhi) : one) * T(j > w - yhi)
+             + (EXACT ? fyhi : T(0)) * T(j > w - yhi - 1)
+             - (EXACT ? (one - fylo) : one) * T(j > w - ylo)
+             - (EXACT ? fylo : T(0)) * T(j > w - ylo + 1);
+    };
+    // first element (with the front pad counted in) of the runs of 5 row pairs that hold the taps
+    // of the lane's columns: right run g[c0 - yhi ..], left run g[c0 + 1 - ylo ..]
+    auto run_start = [&](int first) { return clampi(first, -kPad, w) + kPad; };
+    const int er = run_start(c0 - s.yhi), el = run_start(c0 + 1 - s.ylo);
+    const int er_m = run_start(c0 - yhi_m), el_m = run_start(c0 + 1 - ylo_m);
+    bool wave_has_tail = false;
+    {
+        T d[K];
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            d[k] = tail_weight(c0 + k, s.ylo, s.yhi, s.fylo, s.fyhi);
+            wave_has_tail = wave_has_tail || d[k] != T(0);
+        }
+        *reinterpret_cast<Quad<T>*>(&delta[c0]) = Quad<T>{{d[0], d[1], d[2], d[3]}};
+    }
+    wave_has_tail = __any(wave_has_tail) != 0 || own_w;                          // wave-uniform
+    const int j_ymax = w - s.yhi, j_ymin = w - s.ylo + 1;
+    const int idx_ymax = (j_ymax >= 0 && j_ymax < w) ? j_ymax + kPad : 0;        // element 0 is a zero pad
+    const int idx_ymin = (j_ymin >= 0 && j_ymin < w) ? j_ymin + kPad : 0;
+
+    double total[5] = {0.0, 0.0, 0.0, 0.0, 0.0};
+    T colacc[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) colacc[k] = T(0);
+
+    T ta[K], bc[K], t0[K], t1[K], b1[K], b2[K];
+    load_i(clampi(i0 + s.xlo - 1, 0, h), ta);
+    load_i(clampi(i0 + s.xhi, 0, h), bc);
+    load_window(i0, t0, t1, b1, b2);
+    __syncthreads();                                 // pads and tail weights are in place
+
+    // Rows i, i+1 of grad_output (GA, GB) into LDS buffer FL, the lane's share of their tails, and,
+    // from the lane that owns column w, V, DT, DB of that column for both rows.
+#define BOXCONV_PUBLISH_CONSEC(FL, I, GA, GB, TA, T0, T1, BC, B1, B2, TL0, TL1)                      \
+    {                                                                                               \
+        if ((I) + 1 >= i1) {                                                                        \
+            _Pragma("unroll")                                                                       \
+            for (int k = 0; k < K; ++k) GB[k] = T(0);                                               \
+        }                                                                                           \
+        Quad<T>* dst = reinterpret_cast<Quad<T>*>(&grow[FL][kPad + c0]);                            \
+        dst[0] = Quad<T>{{GA[0], GB[0], GA[1], GB[1]}};                                             \
+        dst[1] = Quad<T>{{GA[2], GB[2], GA[3], GB[3]}};                                             \
+        TL0 = T(0); TL1 = T(0);                                                                     \
+        if (wave_has_tail) {                                                                        \
+            const Quad<T> dq = *reinterpret_cast<const Quad<T>*>(&delta[c0]);                       \
+            _Pragma("unroll")                                                                       \
+            for (int k = 0; k < K; ++k) { TL0 += dq.v[k] * GA[k]; TL1 += dq.v[k] * GB[k]; }         \
+        }                                                                                           \
+        if (tid == NT - 1) {                                                                        \
+            const T dt0 = T0[K - 1] - TA[K - 1], db0 = B1[K - 1] - BC[K - 1];                       \
+            const T dt1 = T1[K - 1] - T0[K - 1], db1 = B2[K - 1] - B1[K - 1];                       \
+            T v0 = BC[K - 1] - T0[K - 1], v1 = B1[K - 1] - T1[K - 1];                               \
+            if (EXACT) {                                                                            \
+                v0 += s.fxhi * db0; v0 += s.fxlo * dt0;                                             \
+                v1 += s.fxhi * db1; v1 += s.fxlo * dt1;                                             \
+            }                                                                                       \
+            xw[FL][0] = LastColumn{v0, dt0, db0, T(0)};                                             \
+            xw[FL][1] = LastColumn{v1, dt1, db1, T(0)};                                             \
+        }                                                                                           \
+    }
+
+    T tl0 = T(0), tl1 = T(0);
+    if (MERGED) {
+        BOXCONV_PUBLISH_CONSEC(0, i0, g0, g1, ta, t0, t1, bc, b1, b2, tl0, tl1)
+        __syncthreads();
+    }
+
+    auto row_pair = [&](int i, auto prefetch_tag, auto flip_tag, auto own_w_tag) {
+        constexpr bool PREFETCH = decltype(prefetch_tag)::value;
+        constexpr int FLIP = decltype(flip_tag)::value;
+        constexpr bool OWN_W = decltype(own_w_tag)::value;
+        T n0[K] = {}, n1[K] = {}, n2[K] = {}, n3[K] = {}, m0[K] = {}, m1[K] = {};
+        if (PREFETCH) {
+            load_window(i + 2, n0, n1, n2, n3);
+            load_g(i + 2, m0);
+            load_g(i + 3, m1);
+        }
+        if (!MERGED) {
+            BOXCONV_PUBLISH_CONSEC(FLIP, i, g0, g1, ta, t0, t1, bc, b1, b2, tl0, tl1)
+            __syncthreads();                                                 // rows are in LDS
+        }
+        const RowPair<T>* G = grow[FLIP];
+        T tail0 = tl0, tail1 = tl1;
+        T tn0 = T(0), tn1 = T(0);
+
+        // W(i)[q], W(i+1)[q] of the lane's columns, and the five sums
+        T wq0[K], wq1[K];
+        {
+            RowPair<T> R[K + 1], L[K + 1];
+#pragma unroll
+            for (int m = 0; m <= K; ++m) { R[m] = G[er + m]; L[m] = G[el + m]; }
+            T sum[5] = {T(0), T(0), T(0), T(0), T(0)};
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                const RowPair<T> grA = R[k], gr = R[k + 1], gl = L[k], glA = L[k + 1];
+                const T dr0 = grA.r0 - gr.r0, dl0 = gl.r0 - glA.r0;
+                const T dr1 = grA.r1 - gr.r1, dl1 = gl.r1 - glA.r1;
+                wq0[k] = gr.r0 - gl.r0;
+                wq1[k] = gr.r1 - gl.r1;
+                if (EXACT) {
+                    wq0[k] += s.fyhi * dr0; wq0[k] += s.fylo * dl0;
+                    wq1[k] += s.fyhi * dr1; wq1[k] += s.fylo * dl1;
+                }
+                const T dt0 = t0[k] - ta[k], db0 = b1[k] - bc[k];
+                const T dt1 = t1[k] - t0[k], db1 = b2[k] - b1[k];
+                T v0 = bc[k] - t0[k], v1 = b1[k] - t1[k];
+                if (EXACT) {
+                    v0 += s.fxhi * db0; v0 += s.fxlo * dt0;
+                    v1 += s.fxhi * db1; v1 += s.fxlo * dt1;
+                }
+                sum[4] += v0 * wq0[k];
+                sum[1] += db0 * wq0[k];
+                sum[0] -= dt0 * wq0[k];
+                sum[3] += v0 * dr0;
+                sum[2] -= v0 * dl0;
+                sum[4] += v1 * wq1[k];
+                sum[1] += db1 * wq1[k];
+                sum[0] -= dt1 * wq1[k];
+                sum[3] += v1 * dr1;
+                sum[2] -= v1 * dl1;
+            }
+            if (wave_has_tail || wave == 0) {
+                const LastColumn x0 = xw[FLIP][0], x1 = xw[FLIP][1];
+                sum[4] += x0.v * tail0 + x1.v * tail1;
+                sum[1] += x0.db * tail0 + x1.db * tail1;
+                sum[0] -= x0.dt * tail0 + x1.dt * tail1;
+                if (tid == 0) {
+                    const RowPair<T> gmax = G[idx_ymax], gmin = G[idx_ymin];
+                    sum[3] += x0.v * gmax.r0 + x1.v * gmax.r1;
+                    sum[2] -= x0.v * gmin.r0 + x1.v * gmin.r1;
+                }
+            }
+#pragma unroll
+            for (int n = 0; n < 5; ++n) total[n] += static_cast<double>(sum[n]);
+        }
+
+        if (OWN_W) {
+            // rare: the mirrored split cuts the box at other whole pixels; weights and tails of
+            // the column workspace from that split
+            RowPair<T> R[K + 1], L[K + 1];
+#pragma unroll
+            for (int m = 0; m <= K; ++m) { R[m] = G[er_m + m]; L[m] = G[el_m + m]; }
+            tail0 = T(0); tail1 = T(0);
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                const RowPair<T> grA = R[k], gr = R[k + 1], gl = L[k], glA = L[k + 1];
+                wq0[k] = gr.r0 - gl.r0;
+                wq1[k] = gr.r1 - gl.r1;
+                if (EXACT) {
+                    wq0[k] += sm.fylo * (grA.r0 - gr.r0); wq0[k] += sm.fyhi * (gl.r0 - glA.r0);
+                    wq1[k] += sm.fylo * (grA.r1 - gr.r1); wq1[k] += sm.fyhi * (gl.r1 - glA.r1);
+                }
+                const T dlt = tail_weight(c0 + k, ylo_m, yhi_m, sm.fyhi, sm.fylo);
+                const RowPair<T> own = G[kPad + c0 + k];
+                tail0 += dlt * own.r0;
+                tail1 += dlt * own.r1;
+            }
+        }
+
+        // A[c] = (sum of all W + tail) - (W of the columns before c): exclusive prefix inside the
+        // lane, the lanes to the left by a wave scan, the other waves through LDS
+        T ex0[K], ex1[K];
+        T base0, base1;
+        {
+            T run0 = T(0), run1 = T(0);
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                ex0[k] = run0; run0 += wq0[k];
+                ex1[k] = run1; run1 += wq1[k];
+            }
+            const T inc0 = wave_inclusive_scan(run0);
+            const T inc1 = wave_inclusive_scan(run1);
+            base0 = run0 - inc0;                                             // -(lanes to the left)
+            base1 = run1 - inc1;
+            T wt0 = T(0), wt1 = T(0);
+            if (wave_has_tail) {
+                wt0 = wave_sum_to_last(tail0);
+                wt1 = wave_sum_to_last(tail1);
+            }
+            if (lane == 63) wsum[FLIP][wave] = WaveSums{inc0, inc1, wt0, wt1};
+        }
+        if (MERGED && PREFETCH) BOXCONV_PUBLISH_CONSEC(FLIP ^ 1, i + 2, m0, m1, t1, n0, n1, b2, n2, n3, tn0, tn1)
+        __syncthreads();                             // wave totals (and the next pair's rows) visible
+        {
+#pragma unroll
+            for (int wv = 0; wv < WAVES; ++wv) {
+                const WaveSums ws = wsum[FLIP][wv];
+                base0 += ws.tail0;
+                base1 += ws.tail1;
+                if (wv >= wave) {                    // `wave` is scalar
+                    base0 += ws.tot0;
+                    base1 += ws.tot1;
+                }
+            }
+            const bool second = i + 1 < i1;
+            const RowRef ob0 = mout.row(i + 1);
+            const RowRef ob1 = mout.row(min(i + 2, h), second);
+            T out0[K];
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                out0[k] = colacc[k] + (base0 - ex0[k]);
+                colacc[k] = out0[k] + (base1 - ex1[k]);
+            }
+            const int first = c0 * static_cast<int>(sizeof(T));
+            const int limit = static_cast<int>(mpitch * sizeof(T));
+            if (keep_in_cache) {
+                buffer_store_run<kCacheDefault, true>(out0, ob0, first, limit);
+                buffer_store_run<kCacheDefault, true>(colacc, ob1, first, limit);
+            } else {
+                buffer_store_run<kCacheStream, true>(out0, ob0, first, limit);
+                buffer_store_run<kCacheStream, true>(colacc, ob1, first, limit);
+            }
+        }
+        if (PREFETCH) {
+            if (MERGED) { tl0 = tn0; tl1 = tn1; }
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                ta[k] = t1[k]; bc[k] = b2[k];
+                t0[k] = n0[k]; t1[k] = n1[k]; b1[k] = n2[k]; b2[k] = n3[k];
+                g0[k] = m0[k]; g1[k] = m1[k];
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+#define BOXCONV_ALL_PAIRS(OWN_W_TAG)                                         \
+    {                                                                        \
+        int i = i0;                                                          \
+        for (; i + 4 < i1; i += 4) {                                         \
+            row_pair(i, std::true_type{}, Flip0{}, OWN_W_TAG{});             \
+            row_pair(i + 2, std::true_type{}, Flip1{}, OWN_W_TAG{});         \
+        }                                                                    \
+        if (i + 2 < i1) {                                                    \
+            row_pair(i, std::true_type{}, Flip0{}, OWN_W_TAG{});             \
+            row_pair(i + 2, std::false_type{}, Flip1{}, OWN_W_TAG{});        \
+        } else {                                                             \
+            row_pair(i, std::false_type{}, Flip0{}, OWN_W_TAG{});            \
+        }                                                                    \
+    }
+    if (own_w) BOXCONV_ALL_PAIRS(std::true_type)
+    else BOXCONV_ALL_PAIRS(std::false_type)
+#undef BOXCONV_ALL_PAIRS
+#undef BOXCONV_PUBLISH_CONSEC
+
+    __syncthreads();
+    block_accumulate5(total, a.acc + ((static_cast<int64_t>(a.plane0 + p) * a.F + f) * a.acc_slots + band) * 5,
+                      red, false);
+}
+
+// ---------------------------------------------------------------------------------------------
 // Gather kernels (helpers in box_sampling_common.hpp): one thread per output pixel.
 
 template <class T, bool EXACT>
@@ -1112,6 +1468,20 @@ hipError_t grad_output_stream_launch(const T* integ, const TG* grad_out, BoxPara
             return hipGetLastError();
         } else {
             return hipErrorInvalidValue;
+        }
+    }
+    // float rows of exactly four columns per lane, both products wanted, a slot per workgroup for
+    // the sums: the kernel with consecutive columns per lane
+    if constexpr (std::is_same<T, float>::value) {
+        const bool aligned = reinterpret_cast<uintptr_t>(grad_out) % (4 * sizeof(TG)) == 0 && d.w % 4 == 0;
+        if (switches().stream_consecutive && rc.full && rc.K == 4 && params && scan && acc_slots > 0 && aligned) {
+#define LAUNCH_GC(NT) \
+            if (exact) BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, true>), grid, dim3(NT), lds, stream, a); \
+            else       BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, false>), grid, dim3(NT), lds, stream, a)
+            if (rc.nt == 64) { LAUNCH_GC(64); } else if (rc.nt == 128) { LAUNCH_GC(128); }
+            else if (rc.nt == 256) { LAUNCH_GC(256); } else { LAUNCH_GC(512); }
+#undef LAUNCH_GC
+            return hipGetLastError();
         }
     }
 #pragma push_macro("BOXCONV_DISPATCH_WIDE")

@@ -174,6 +174,7 @@ struct Switches {
     bool gi_split_filters;    // BOXCONV_GI_SPLIT_FILTERS=0 clears it: no filter sharing in small grad-input launches
     bool lookback;            // BOXCONV_INTEGRAL_LOOKBACK=0 clears it: no single-pass integral image
     bool lookback_any_shape;  // BOXCONV_INTEGRAL_LOOKBACK=2: single pass for every shape it covers
+    bool stream_consecutive;  // BOXCONV_STREAM_CONSEC=0 clears it: no consecutive-column variant of the grad_output pass
     int spin_limit;           // BOXCONV_INTEGRAL_SPIN: polls of a hand-over word before re-summing (64)
     int fwd_threads;          // BOXCONV_FWD_THREADS: 256 or 512 (512)
     int stream_threads;       // BOXCONV_STREAM_THREADS: 256 or 512 (256)

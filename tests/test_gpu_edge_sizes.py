@@ -83,7 +83,10 @@ def test_tensors_that_are_not_16_byte_aligned(hip, shape):
     """Inputs whose data pointers are only 4-byte aligned (views into a larger buffer): the vector
     loads must not be used on them. Same bits as with aligned tensors for the integral image and
     the forward pass; the backward is compared to a tight tolerance (its column workspace is
-    private and aligned either way, only the loads of grad_output and of the integral differ)."""
+    private and aligned either way, only the loads of grad_output and of the integral differ; a
+    grad_output that is not 16-byte aligned also takes the variant of the grad_output pass with
+    wave-strided instead of consecutive columns per lane, whose float sums are associated
+    differently)."""
     B, C, F, h, w = shape
     gen = torch.Generator(device="cuda").manual_seed(11)
     x = torch.randn(B, C, h, w, device="cuda", generator=gen)
@@ -103,4 +106,4 @@ def test_tensors_that_are_not_16_byte_aligned(hip, shape):
                                        True, True, True, True, True)
     torch.cuda.synchronize()
     for a, b in zip(ref, got):
-        assert torch.allclose(a, b, rtol=1e-6, atol=1e-6 * float(a.abs().max()))
+        assert torch.allclose(a, b, rtol=1e-5, atol=4e-6 * float(a.abs().max()))

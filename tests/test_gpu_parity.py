@@ -324,6 +324,33 @@ def test_grad_input_filter_sharing_matches_one_set_per_workgroup(hip, switches, 
     assert (shared - single).abs().max().item() <= 4e-6 * scale
 
 
+@pytest.mark.parametrize("exact", [True, False])
+@pytest.mark.parametrize("h,w", [(67, 256), (130, 512), (70, 1024), (66, 2048)])
+def test_grad_output_pass_variants_agree(hip, oracle, switches, h, w, exact):
+    """Rows that fill a workgroup's column slots exactly (four columns per lane) run the
+    grad_output pass with consecutive columns per lane; BOXCONV_STREAM_CONSEC=0 sends them to the
+    kernel with wave-strided columns, as every other width. Both against the oracle, and against
+    each other to the last few bits (the sums differ only in which columns share a lane)."""
+    rng = np.random.default_rng(h + w + int(exact))
+    B, C, F = 1, 2, 3
+    x = rng.standard_normal((B, C, h, w)).astype(np.float32)
+    g = (rng.standard_normal((B, C * F, h, w)) + 0.25).astype(np.float32)
+    boxes = list(make_boxes(rng, C, F, h, w, "hanging", away_from_integers=0.05))
+    if not exact:
+        boxes[1] = np.maximum(boxes[1], np.ceil(boxes[0]) + 1).astype(np.float32)
+        boxes[3] = np.maximum(boxes[3], np.ceil(boxes[2]) + 1).astype(np.float32)
+    results = []
+    for variant in ("1", "0"):
+        switches("BOXCONV_STREAM_CONSEC", variant)
+        cpu, gpu, sc = run_both(hip, oracle, x, tuple(boxes), 3.5 * h, 2.25 * w, True, exact, g)
+        assert_parity(cpu, gpu, np.float32, "consecutive=%s %dx%d exact=%s" % (variant, h, w, exact), **sc)
+        results.append(gpu)
+    (_, back_a), (_, back_b) = results
+    assert np.abs(back_a[0] - back_b[0]).max() <= 2e-6 * np.abs(back_b[0]).max()
+    for a, b in zip(back_a[1:], back_b[1:]):
+        assert np.abs(a - b).max() <= 1e-5 * max(np.abs(b).max(), 1e-30) + 1e-6 * max(np.abs(t).max() for t in back_b[1:])
+
+
 def test_parameter_gradients_are_reproducible(hip):
     """The streaming backward adds the per-workgroup partial sums in a fixed order (no atomics),
     so repeated calls agree bit for bit."""

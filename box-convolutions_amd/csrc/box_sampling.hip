@@ -29,6 +29,8 @@ Switches read_switches() {
     s.lookback = e == nullptr || std::atoi(e) != 0;
     s.lookback_any_shape = e != nullptr && std::atoi(e) == 2;
     s.stream_consecutive = flag_unless_zero("BOXCONV_STREAM_CONSEC");
+    e = text("BOXCONV_STREAM_WGS");
+    s.stream_workgroups = e != nullptr ? std::max(1, std::atoi(e)) : 2048;
     e = text("BOXCONV_INTEGRAL_SPIN");
     s.spin_limit = e != nullptr ? std::max(0, std::atoi(e)) : 64;
     s.fwd_threads = threads("BOXCONV_FWD_THREADS", 512);
@@ -111,7 +113,7 @@ StreamPlan plan_grad_output_stream(int64_t planes_f, int h, int w, size_t elem_s
     const RowConfig rc = stream_row_config(std::max(w, 1));
     sp.usable = row_kernels_apply(h, w, elem_size) &&
                 stream_lds_bytes(rc.K, rc.nt, elem_size) <= kMaxDynamicLds;
-    int nb = bands_for(std::max<int64_t>(planes_f, 1), h, 32, 2048);
+    int nb = bands_for(std::max<int64_t>(planes_f, 1), h, 32, switches().stream_workgroups);
     int R = (h + nb - 1) / nb;
     R += R & 1;                                        // rows are handled in pairs
     sp.R = std::max(R, 2);

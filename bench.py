@@ -213,6 +213,51 @@ def event_pair_overhead_ms(n=50):
     return vals[len(vals) // 2]
 
 
+def machine_probes(dev):
+    """Rates of plain kernels on this machine, the yardsticks for the kernels' own rates."""
+    import torch
+    from box_convolution import _native
+
+    def timed(fn, reps=20):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(reps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            e1.synchronize()
+            times.append(e0.elapsed_time(e1) * 1e-3)
+        return sorted(times)[len(times) // 2]
+
+    print("plain kernels on one MI355X (median of 20 launches, HIP events around each; TB/s on the bytes named)")
+    n = 512 * (1 << 20) // 4
+    a = torch.randn(n, device=dev)
+    b = torch.empty_like(a)
+    c = torch.randn(n, device=dev)
+    for name, fn, nbytes in (("torch sum, 512 MiB read", lambda: a.sum(), 4 * n),
+                             ("torch copy_, 512 MiB read + 512 MiB written", lambda: b.copy_(a), 8 * n),
+                             ("torch add, 2 x 512 MiB read + 512 MiB written", lambda: torch.add(a, c, out=b), 12 * n),
+                             ("torch fill_, 512 MiB written", lambda: b.fill_(1.0), 4 * n)):
+        t = timed(fn)
+        print("%-72s %7.1f us  %.2f TB/s" % (name, t * 1e6, nbytes / t / 1e12))
+    del a, b, c
+    planes, h, w = 256, 512, 1024        # grad_output of the headline workload: 2 x 16 x 8 planes
+    src = torch.randn(planes, h, w, device=dev)
+    dst = torch.zeros(planes, h + 1, w, device=dev)
+    nbytes = 8 * planes * h * w
+    for rows, in_flight in ((64, 2), (64, 8), (32, 2), (16, 2), (8, 2), (8, 8)):
+        t = timed(lambda: _native.probe_copy_bands(src, dst, rows, in_flight))
+        print("%-72s %7.1f us  %.2f TB/s" % (
+            "band copy of 256 planes of 512 x 1024 floats, %2d rows per workgroup, %d in flight" % (rows, in_flight),
+            t * 1e6, nbytes / t / 1e12))
+    assert torch.equal(dst[:, 1:], src)
+    print("(the backward's streaming pass moves these 1074 MB plus 67 MB of integral images per launch, in "
+          "workgroups of 64 rows)")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -244,6 +289,11 @@ def main():
                     help="after the timed steps, run torch.neg on a float tensor of this many MiB "
                          "(reads MIB, writes MIB): the plain streaming kernel of known size that "
                          "the FETCH_SIZE / WRITE_SIZE counters are calibrated against")
+    ap.add_argument("--machine-probes", action="store_true",
+                    help="instead of a workload: what this machine's memory system gives plain kernels "
+                         "(torch's sum, copy, add, fill on 512 MiB, and the library's band-wise copy with "
+                         "the access pattern of the backward's streaming pass at the headline shape); "
+                         "prints a table, not the JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus %d is not supported (box convolution "
@@ -258,6 +308,9 @@ def main():
     _native.load()
 
     dev = torch.device("cuda:0")
+    if args.machine_probes:
+        machine_probes(dev)
+        return
     if args.shape:
         import random
         from baseline_workloads import Workload

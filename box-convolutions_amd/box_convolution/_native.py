@@ -31,6 +31,7 @@ _SIGNATURES = {
     "boxconv_profile_arm": (_i, [ctypes.c_char_p]),
     "boxconv_profile_arm_every": (_i, [ctypes.c_char_p, _i]),
     "boxconv_profile_collect": (_i, [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int)]),
+    "boxconv_probe_copy_bands": (_i, [_vp, _vp, _i64, _i, _i, _i, _i, _vp]),
     "boxconv_integral_image_workspace_bytes": (_sz, [_i64, _i, _i]),
     "boxconv_backward_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i, _i, _i]),
 }
@@ -622,6 +623,17 @@ def profile_arm(kernel_name, every=1):
     disarms)."""
     _check(load().boxconv_profile_arm_every(kernel_name.encode() if kernel_name else None, every),
            "profile_arm")
+
+
+def probe_copy_bands(src, dst, rows_per_group, rows_in_flight):
+    """Plain copy of `src` [planes, h, w] into rows 1..h of `dst` [planes, h+1, w] with the access
+    pattern of the backward's streaming pass (a measurement yardstick, see include/boxconv.h)."""
+    planes, h, w = src.shape
+    if (src.dtype != torch.float32 or dst.dtype != torch.float32 or not src.is_cuda or not dst.is_cuda
+            or tuple(dst.shape) != (planes, h + 1, w) or not src.is_contiguous() or not dst.is_contiguous()):
+        raise RuntimeError("probe_copy_bands: contiguous float32 device tensors [planes,h,w] -> [planes,h+1,w]")
+    _check(load().boxconv_probe_copy_bands(_ptr(src), _ptr(dst), planes, h, w, rows_per_group,
+                                           rows_in_flight, _stream(src.device)), "probe_copy_bands")
 
 
 def profile_collect():

@@ -46,7 +46,6 @@ Switches g_switches;
 
 constexpr int kLdsDevices = 64;
 std::atomic<int64_t> g_lds_limit[kLdsDevices];     // 0 = not looked up yet, -1 = query failed
-std::atomic<int> g_compute_units[kLdsDevices];     // 0 = not looked up yet
 
 }  // namespace
 
@@ -94,18 +93,6 @@ hipError_t grad_params_begin(double* acc, int n_boxes, hipStream_t stream) {
     BOXCONV_LAUNCH("fill_zero", fill_zero_kernel, dim3((n_boxes * 5 + 255) / 256), dim3(256), 0,
                    stream, acc, n_boxes * 5);
     return hipGetLastError();
-}
-
-int compute_units() {
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kLdsDevices) return 256;
-    int v = g_compute_units[dev].load(std::memory_order_relaxed);
-    if (v == 0) {
-        int n = 0;
-        v = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0 ? n : 256;
-        g_compute_units[dev].store(v, std::memory_order_relaxed);
-    }
-    return v;
 }
 
 StreamPlan plan_grad_output_stream(int64_t planes_f, int h, int w, size_t elem_size) {

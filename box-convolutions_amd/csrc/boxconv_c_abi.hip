@@ -469,6 +469,22 @@ int boxconv_integral_image_int(const void* in, void* out, int dtype, int64_t pla
                       "integer integral image launch");
 }
 
+int boxconv_probe_copy_bands(const float* src, float* dst, int64_t planes, int h, int w,
+                             int rows_per_group, int rows_in_flight, void* stream) {
+    if (planes < 1 || h < 1 || w < 256 || w > 4096 || w % 256 != 0 || rows_per_group < 1 ||
+        h % rows_per_group != 0 || (rows_in_flight != 2 && rows_in_flight != 4 && rows_in_flight != 8) ||
+        rows_per_group % rows_in_flight != 0)
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "copy probe: invalid sizes planes=%lld h=%d w=%d rows=%d in flight=%d",
+                    static_cast<long long>(planes), h, w, rows_per_group, rows_in_flight);
+    if (src == nullptr || dst == nullptr)
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "copy probe: null tensor pointer");
+    if (planes * static_cast<int64_t>(h + 1) * w > kMaxElems)
+        return fail(BOXCONV_E_TOO_LARGE, "copy probe: destination exceeds 2^31-1 elements");
+    return hip_result(boxconv::probe_copy_bands_launch(src, dst, planes, h, w, rows_per_group, rows_in_flight,
+                                                       static_cast<hipStream_t>(stream)),
+                      "copy probe launch");
+}
+
 int boxconv_integral_image_static_f32(const float* in, float* out, int64_t planes, int h, int w,
                                       void* stream) {
     return integral_image_static_impl(in, out, planes, h, w, stream);

@@ -61,6 +61,11 @@ constexpr int kIntU8 = 16, kIntI8 = 17, kIntI16 = 18, kIntI32 = 19, kIntI64 = 20
 hipError_t integral_image_int_launch(const void* in, void* out, int dtype, int64_t planes, int h, int w,
                                      hipStream_t stream);
 
+// Plain copy with the grad_output pass's access pattern (see boxconv_probe_copy_bands in
+// include/boxconv.h); the caller has checked the sizes.
+hipError_t probe_copy_bands_launch(const float* src, float* dst, int64_t planes, int h, int w, int rows,
+                                   int rows_in_flight, hipStream_t stream);
+
 template <class T>
 hipError_t forward_launch(const T* integ, BoxParams<T> prm, T* out, Dims d, bool normalize,
                           bool exact, hipStream_t stream);
@@ -192,8 +197,6 @@ inline bool force_gather_kernels() { return switches().force_gather; }
 // LDS bytes one workgroup may use on the current device (hipDeviceAttributeMaxSharedMemoryPerBlock,
 // looked up once per device; 0 if the query fails, which sends every shape to the gather kernels).
 size_t device_lds_limit();
-// Compute units of the current device (looked up once per device; 256 if the query fails).
-int compute_units();
 
 // Optional per-kernel timing (see boxconv_profile_arm in include/boxconv.h). When a kernel name is
 // armed, every launch of that kernel is bracketed by a pair of HIP events on its stream.

@@ -56,7 +56,7 @@ void boxconv_reload_env(void);
  * alone, whatever else the entry point launches). Names: "band_colsum", "band_prefix",
  * "band_scan", "forward_rows", "grad_output_stream", "grad_input_cols",
  * "param_grad_finalize", "fill_zero", "fill_marker", "clip", "forward_gather", "grad_input_gather",
- * "int_row_prefix", "int_col_prefix",
+ * "int_row_prefix", "int_col_prefix", "probe_copy_bands",
  * "grad_params_gather".
  * NULL or "" disarms. Arming discards earlier measurements.
  * boxconv_profile_arm_every(name, n): the same, but only every n-th launch of that kernel (the
@@ -67,6 +67,17 @@ void boxconv_reload_env(void);
 int boxconv_profile_arm(const char* kernel_name);
 int boxconv_profile_arm_every(const char* kernel_name, int every);
 int boxconv_profile_collect(double* total_ms, int* launches);
+
+/* A plain copy with the access pattern of the backward's streaming pass over grad_output
+ * (measurement aid; no counterpart in the reference): `planes` planes of h x w floats are copied
+ * into planes of (h+1) x w floats (rows 1..h; row 0 is not touched), a workgroup of w/4 lanes
+ * streaming `rows_per_group` consecutive rows, 16 bytes per lane and row, `rows_in_flight` (2, 4
+ * or 8) rows loaded before they are stored, non-temporal stores. Its rate is what the memory
+ * system gives a kernel that reads and writes with that pattern, the yardstick the benchmark
+ * prints beside the kernels' own rates. w a multiple of 256 up to 4096, h a multiple of
+ * rows_per_group, rows_per_group a multiple of rows_in_flight. */
+int boxconv_probe_copy_bands(const float* src, float* dst, int64_t planes, int h, int w,
+                             int rows_per_group, int rows_in_flight, void* stream);
 
 /* ---- integral image ------------------------------------------------------------------------
  * Replaces `integral_image(Tensor) -> Tensor`, reference src/integral_image_interface.cpp:8-27

@@ -63,6 +63,12 @@ def test_argument_errors_are_reported_without_launching(lib):
     rc = lib.boxconv_integral_image_int(null, null, 19, 1, 4, 4, null)
     assert rc == -1 and b"null" in lib.boxconv_last_error()
     dummy16 = ctypes.c_void_p(256)
+    rc = lib.boxconv_probe_copy_bands(dummy16, dummy16, 4, 64, 1000, 64, 2, null)     # w not a multiple of 256
+    assert rc == -1 and b"copy probe" in lib.boxconv_last_error()
+    rc = lib.boxconv_probe_copy_bands(dummy16, dummy16, 4, 64, 1024, 48, 2, null)     # bands do not tile h
+    assert rc == -1 and b"copy probe" in lib.boxconv_last_error()
+    rc = lib.boxconv_probe_copy_bands(null, null, 4, 64, 1024, 64, 2, null)
+    assert rc == -1 and b"null" in lib.boxconv_last_error()
     rc = lib.boxconv_integral_image_half_f32(dummy16, 1, dummy16, 1, 4, 4096, null, 0, null)
     assert rc == -3 and b"2048" in lib.boxconv_last_error()
     assert lib.boxconv_profile_arm_every(b"forward_rows", 0) == -1

@@ -412,3 +412,18 @@ def test_cpp_autograd_node_reports_the_reference_errors(hip):
         m(torch.zeros(1, 5, 8, 8, device=DEV))
     with pytest.raises(AssertionError):
         BoxConv2d(2, 3, 8, 8, stride_h=2)
+
+
+@pytest.mark.parametrize("w,rows,in_flight", [(256, 16, 2), (1024, 64, 8), (4096, 8, 4)])
+def test_copy_probe_copies(hip, w, rows, in_flight):
+    """The benchmark's yardstick kernel (a plain copy with the streaming pass's access pattern)
+    moves exactly the bytes it is priced on: rows 1..h of every plane, nothing else."""
+    planes, h = 5, 128
+    src = torch.randn(planes, h, w, device="cuda")
+    dst = torch.full((planes, h + 1, w), -7.0, device="cuda")
+    hip.probe_copy_bands(src, dst, rows, in_flight)
+    torch.cuda.synchronize()
+    assert torch.equal(dst[:, 1:], src)
+    assert bool((dst[:, 0] == -7.0).all())
+    with pytest.raises(RuntimeError):
+        hip.probe_copy_bands(src, dst, 48, 2)

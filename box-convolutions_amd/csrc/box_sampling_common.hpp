@@ -44,7 +44,23 @@ struct SampleArgs {
     int reverse;          // grad input only: walk the work items last to first
     int64_t keep_tail;    // grad_output pass only: bytes at the end of each XCD's share of the
                           // band-local integral that are stored with the ordinary cache policy
+    int m_bands;          // rows of M interleaved over this many bands (0: rows in their natural order)
+    int m_shift;          // log2 of the rows per band of M (interleaved layout only)
 };
+
+// Where row r (0..h) of a plane of the column workspace M lives. Natural order: row r. Interleaved
+// (planes of nb bands of exactly R = 2^m_shift rows): row 0 stays, row 1 + b*R + k (row k of band
+// b) goes to 1 + k*nb + b, so that the nb workgroups that write the bands of one plane side by
+// side, all at row k of their band at about the same time, write nb adjacent rows: the memory
+// system takes writes that cluster in address space faster than as many streams 256 KB apart
+// (a plain copy with either layout: 190 against 201 us for the headline's 1074 MB).
+template <class T>
+__device__ __forceinline__ int workspace_row(const SampleArgs<T>& a, int r) {
+    if (a.m_bands == 0) return r;
+    const int rr = r - 1;
+    const int il = 1 + (rr & ((1 << a.m_shift) - 1)) * a.m_bands + (rr >> a.m_shift);
+    return r == 0 ? 0 : il;
+}
 
 // Two rows of the same column, adjacent in LDS: every LDS access of the row kernels moves the
 // values of both rows of the current row pair at once.
@@ -276,6 +292,18 @@ SampleArgs<T> base_args(BoxParams<T> prm, const Dims& d) {
     SampleArgs<T> a{};
     a.prm = prm; a.C = d.C; a.F = d.F; a.h = d.h; a.w = d.w; a.plane0 = d.plane0;
     return a;
+}
+
+// The interleaved layout of M applies to planes that are cut into whole bands of a power-of-two
+// number of rows; both launches that touch M derive it from (h, rows per band) alone.
+template <class T>
+void set_workspace_layout(SampleArgs<T>& a, int h, int band_rows) {
+    a.m_bands = 0; a.m_shift = 0;
+    if (!switches().interleave_workspace || band_rows < 2 || (band_rows & (band_rows - 1)) != 0 ||
+        h % band_rows != 0 || h / band_rows < 2)
+        return;
+    a.m_bands = h / band_rows;
+    while ((1 << a.m_shift) < band_rows) ++a.m_shift;
 }
 
 template <class T>

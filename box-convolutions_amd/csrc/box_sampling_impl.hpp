@@ -226,7 +226,7 @@ grad_input_cols_kernel(SampleArgs<T> a, FinalizeArgs<T> fin) {
             ? inverse_extent(bx.xmin, bx.xmax, bx.ymin, bx.ymax, EXACT, true, true) : T(1);
         const T* plane = a.src + (p * a.F + f) * mplane + cl;
         auto load_row = [&](int row) {
-            return *reinterpret_cast<const Quad<T>*>(plane + static_cast<int64_t>(row) * mpitch);
+            return *reinterpret_cast<const Quad<T>*>(plane + static_cast<int64_t>(workspace_row(a, row)) * mpitch);
         };
 
         // rows of the two runs; rt[r+1], rb[r] are the plain and rt[r], rb[r+1] the advanced rows
@@ -812,8 +812,8 @@ grad_output_stream_kernel(SampleArgs<T> a) {
                 // is stored non-temporally so that it does not push the integral plane of the
                 // input, which all filters of a plane re-read, out of the L2.
                 const bool second = i + 1 < i1;
-                const RowRef ob0 = mout.row(i + 1);
-                const RowRef ob1 = mout.row(min(i + 2, h), second);
+                const RowRef ob0 = mout.row(workspace_row(a, i + 1));
+                const RowRef ob1 = mout.row(workspace_row(a, min(i + 2, h)), second);
                 T out0[K];
 #pragma unroll
                 for (int k = 0; k < K; ++k) {
@@ -1189,8 +1189,8 @@ grad_output_stream_consec_kernel(SampleArgs<float> a) {
                 }
             }
             const bool second = i + 1 < i1;
-            const RowRef ob0 = mout.row(i + 1);
-            const RowRef ob1 = mout.row(min(i + 2, h), second);
+            const RowRef ob0 = mout.row(workspace_row(a, i + 1));
+            const RowRef ob1 = mout.row(workspace_row(a, min(i + 2, h)), second);
             T out0[K];
 #pragma unroll
             for (int k = 0; k < K; ++k) {
@@ -1374,6 +1374,7 @@ hipError_t grad_input_launch(const T* gint, int band_rows, BoxParams<T> prm, TO*
 
     a.reverse = reverse_grad_input() ? 1 : 0;
     a.mpitch = column_workspace_pitch(d.w);
+    set_workspace_layout(a, d.h, band_rows);
     a.vec_out = (d.w % 4 == 0 && reinterpret_cast<uintptr_t>(grad_in) % (4 * sizeof(TO)) == 0) ? 1 : 0;
     const ColsConfig cc = cols_config(d.planes, d.F, d.h, d.w, split_filters_enabled());
     const int ntx = std::max(64, 1 << cc.lq), rg = ntx >> cc.lq;
@@ -1438,6 +1439,7 @@ hipError_t grad_output_stream_launch(const T* integ, const TG* grad_out, BoxPara
     a.mpitch = column_workspace_pitch(d.w);
     if (acc_slots != 0 && acc_slots != sp.nb * sp.parts) return hipErrorInvalidValue;
     a.nb = sp.nb; a.R = sp.R;
+    set_workspace_layout(a, d.h, sp.R);
     a.keep_tail = scan ? cached_tail_bytes() / kXcds : 0;
     finish_args(a, planes_f * a.nb);
     const RowConfig rc = stream_row_config(d.w);

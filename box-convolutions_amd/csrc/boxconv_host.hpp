@@ -180,6 +180,7 @@ struct Switches {
     bool lookback;            // BOXCONV_INTEGRAL_LOOKBACK=0 clears it: no single-pass integral image
     bool lookback_any_shape;  // BOXCONV_INTEGRAL_LOOKBACK=2: single pass for every shape it covers
     bool stream_consecutive;  // BOXCONV_STREAM_CONSEC=0 clears it: no consecutive-column variant of the grad_output pass
+    bool interleave_workspace;  // BOXCONV_M_INTERLEAVE=0 clears it: rows of the column workspace in their natural order
     int stream_workgroups;    // BOXCONV_STREAM_WGS: workgroups the grad_output pass aims for when it cuts planes into bands (2048)
     int spin_limit;           // BOXCONV_INTEGRAL_SPIN: polls of a hand-over word before re-summing (64)
     int fwd_threads;          // BOXCONV_FWD_THREADS: 256 or 512 (512)

@@ -352,6 +352,28 @@ def test_grad_output_pass_variants_agree(hip, oracle, switches, h, w, exact):
         assert np.abs(a - b).max() <= 1e-5 * max(np.abs(b).max(), 1e-30) + 1e-6 * max(np.abs(t).max() for t in back_b[1:])
 
 
+@pytest.mark.parametrize("h,w", [(64, 20), (96, 200), (128, 256), (256, 512), (64, 1024), (128, 2500)])
+def test_workspace_layouts_agree(hip, oracle, switches, h, w):
+    """Planes that are cut into whole bands of a power-of-two number of rows keep the rows of the
+    column workspace interleaved over the bands (row k of every band side by side);
+    BOXCONV_M_INTERLEAVE=0 keeps them in their natural order. Only the place of a row changes,
+    so the two give the same bits, and both meet the oracle."""
+    rng = np.random.default_rng(h * 7 + w)
+    B, C, F = 2, 2, 3
+    x = rng.standard_normal((B, C, h, w)).astype(np.float32)
+    g = (rng.standard_normal((B, C * F, h, w)) + 0.25).astype(np.float32)
+    boxes = tuple(make_boxes(rng, C, F, h, w, "hanging", away_from_integers=0.05))
+    results = []
+    for layout in ("1", "0"):
+        switches("BOXCONV_M_INTERLEAVE", layout)
+        cpu, gpu, sc = run_both(hip, oracle, x, boxes, 2.5 * h, 1.5 * w, True, True, g)
+        assert_parity(cpu, gpu, np.float32, "interleave=%s %dx%d" % (layout, h, w), **sc)
+        results.append(gpu)
+    (_, back_a), (_, back_b) = results
+    for a, b in zip(back_a, back_b):
+        assert np.array_equal(a, b)
+
+
 def test_parameter_gradients_are_reproducible(hip):
     """The streaming backward adds the per-workgroup partial sums in a fixed order (no atomics),
     so repeated calls agree bit for bit."""

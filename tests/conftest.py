@@ -21,8 +21,11 @@ def pytest_terminal_summary(terminalreporter):
         # (worded without "<number> passed" / "<number> failed": result parsers count those tokens)
         line = ("assert_parity: of %(comparisons)d tensor comparisons, the rounding-noise term or the "
                 "sibling scale was needed in %(needed_noise_term)d (reference tensor zero, or a millionth of its "
-                "siblings, in %(of_those_reference_all_zero)d of those); largest diff / (tol * max|cpu|) among the "
-                "rest: %(worst_ratio).2f [%(worst_case)s]" % stats)
+                "siblings, in %(of_those_reference_all_zero)d of those)" % stats)
+        if stats["worst_case"]:
+            line += "; largest diff / (tol * max|cpu|) among the rest: %(worst_ratio).2f [%(worst_case)s]" % stats
+        else:
+            line += "; every other comparison met tol * max|cpu| of the tensor itself"
         terminalreporter.write_line(line)
         path = os.environ.get("BOXCONV_PARITY_REPORT")
         if path:

@@ -16,7 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_NAME = "libboxconv_hip.so"
 LIB_PATH = os.path.join(_HERE, LIB_NAME)
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _lib = None
 
@@ -44,6 +44,8 @@ for _s in ("f32", "f64"):
     _SIGNATURES["boxconv_clip_reparametrize_" + _s] = (_i, [_vp] * 5 + [_i] + [_d] * 4 + [_i, _vp])
     _SIGNATURES["boxconv_training_forward_" + _s] = (
         _i, [_vp] * 8 + [_i] * 5 + [_d] * 4 + [_i, _i] + [_vp, _sz, _vp])
+    _SIGNATURES["boxconv_inference_forward_" + _s] = (
+        _i, [_vp] * 8 + [_i] * 5 + [_d] * 2 + [_i, _i] + [_vp, _sz, _vp])
 
 _SIGNATURES["boxconv_backward_half_f32"] = (
     _i, [_vp] * 6 + [_i, _f, _f, _i, _i] + [_vp] * 5 + [_i] * 5 + [_vp, _sz, _vp])
@@ -111,7 +113,8 @@ def glue():
                               "its Python glue (same kernels, more host time per step)" % (GLUE_PATH, exc))
                 return None
             module.init(*[ctypes.cast(getattr(lib, name), ctypes.c_void_p).value for name in (
-                "boxconv_training_forward_f32", "boxconv_training_forward_f64", "boxconv_backward_f32",
+                "boxconv_training_forward_f32", "boxconv_training_forward_f64",
+                "boxconv_inference_forward_f32", "boxconv_inference_forward_f64", "boxconv_backward_f32",
                 "boxconv_backward_f64", "boxconv_integral_image_workspace_bytes",
                 "boxconv_backward_workspace_bytes", "boxconv_last_error")])
             _glue = module
@@ -119,13 +122,14 @@ def glue():
 
 
 def training_step(input, x_min, x_max, y_min, y_max, reparametrization_h, reparametrization_w,
-                  max_input_h, max_input_w, normalize, exact):
-    """``BoxConv2d.forward`` in training mode through the C++ autograd node: clips the stored
-    parameters in place, returns the output; its backward gives the five gradients. Same native
-    calls as ``BoxConvolutionFunction`` with ``clip_to``. Requires ``glue()``."""
+                  max_input_h, max_input_w, normalize, exact, clip=True):
+    """``BoxConv2d.forward`` through the C++ autograd node. ``clip`` (training mode): clips the
+    stored parameters in place first; without it (eval mode) they are only read. Returns the
+    output; its backward gives the five gradients. Same native calls as
+    ``BoxConvolutionFunction`` (with ``clip_to`` in training mode). Requires ``glue()``."""
     return _glue.training_step(
         input, x_min, x_max, y_min, y_max, float(reparametrization_h), float(reparametrization_w),
-        float(max_input_h), float(max_input_w), bool(normalize), bool(exact),
+        float(max_input_h), float(max_input_w), bool(normalize), bool(exact), bool(clip),
         _stream(input.device) or 0, torch.cuda.is_current_stream_capturing())
 
 

@@ -175,14 +175,16 @@ class BoxConv2d(torch.nn.Module):
         if input.dtype in self._HALF_TYPES:
             return self._forward_half(input)
         clip_to = None
+        native = self.x_min.is_cuda and input.is_cuda and input.dim() == 4 and input.dtype == self.x_min.dtype
+        if native and _native.glue() is not None and input.dtype in self._GLUE_TYPES:
+            # the whole call's host side in C++ (same native calls, autograd node included); the
+            # parameters are clipped on the way in only in training mode
+            return _native.training_step(
+                input, self.x_min, self.x_max, self.y_min, self.y_max,
+                self.reparametrization_h, self.reparametrization_w,
+                self.max_input_h, self.max_input_w, self.normalize, self.exact, clip=self.training)
         if self.training:
-            if self.x_min.is_cuda and input.is_cuda and input.dim() == 4 and input.dtype == self.x_min.dtype:
-                if _native.glue() is not None and input.dtype in self._GLUE_TYPES:
-                    # the whole step's host side in C++ (same native calls, autograd node included)
-                    return _native.training_step(
-                        input, self.x_min, self.x_max, self.y_min, self.y_max,
-                        self.reparametrization_h, self.reparametrization_w,
-                        self.max_input_h, self.max_input_w, self.normalize, self.exact)
+            if native:
                 # the projection rides along in the native forward call
                 clip_to = (self.max_input_h, self.max_input_w)
             else:

@@ -68,10 +68,11 @@ hipError_t probe_copy_bands_launch(const float* src, float* dst, int64_t planes,
 
 template <class T>
 ClipArgs<T> clip_args(T* xmin, T* xmax, T* ymin, T* ymax, T* real, int n, double reparam_h,
-                      double reparam_w, double max_h, double max_w, bool exact) {
+                      double reparam_w, double max_h, double max_w, bool exact, bool project) {
     // float literals widened to double (src/box_convolution_interface.cpp:405-406)
     const double min_size = static_cast<double>(exact ? 1.001f : 2.001f);
-    return ClipArgs<T>{xmin, xmax, ymin, ymax, real, n, reparam_h, reparam_w, max_h, max_w, min_size};
+    return ClipArgs<T>{xmin, xmax, ymin, ymax, real, n, reparam_h, reparam_w, max_h, max_w, min_size,
+                       project ? 1 : 0};
 }
 
 template <class T>
@@ -89,8 +90,8 @@ template hipError_t clip_launch<float>(float*, float*, float*, float*, float*, i
 template hipError_t clip_launch<double>(double*, double*, double*, double*, double*, int, double,
                                         double, double, double, bool, hipStream_t);
 template ClipArgs<float> clip_args<float>(float*, float*, float*, float*, float*, int, double, double,
-                                          double, double, bool);
+                                          double, double, bool, bool);
 template ClipArgs<double> clip_args<double>(double*, double*, double*, double*, double*, int, double,
-                                            double, double, double, bool);
+                                            double, double, double, bool, bool);
 
 }  // namespace boxconv

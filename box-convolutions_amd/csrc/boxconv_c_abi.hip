@@ -219,7 +219,7 @@ int training_forward_impl(const T* input, T* x_min, T* x_max, T* y_min, T* y_max
                           T* integ, T* output, int batch, int in_planes, int num_filters, int h,
                           int w, double reparam_h, double reparam_w, double max_h, double max_w,
                           int normalize, int exact, void* workspace, size_t workspace_bytes,
-                          void* stream) {
+                          void* stream, bool project = true) {
     if (int rc = check_dims(batch, in_planes, num_filters, h, w)) return rc;
     const int n = in_planes * num_filters;
     if (n > 0 && (!x_min || !x_max || !y_min || !y_max || !real))
@@ -240,7 +240,7 @@ int training_forward_impl(const T* input, T* x_min, T* x_max, T* y_min, T* y_max
     bool prepared = false;
     if (int rc = hip_result(boxconv::clip_and_prepare_integral_launch<T>(
             boxconv::clip_args<T>(x_min, x_max, y_min, y_max, real, n, reparam_h, reparam_w, max_h,
-                                  max_w, exact != 0),
+                                  max_w, exact != 0, project),
             planes, w, aux, plan, &prepared, s), "clip launch"))
         return rc;
     if (planes == 0) return 0;
@@ -553,6 +553,32 @@ int boxconv_training_forward_f64(const double* input, double* x_min, double* x_m
                                          w, reparametrization_h, reparametrization_w, max_input_h,
                                          max_input_w, normalize, exact, workspace, workspace_bytes,
                                          stream);
+}
+
+int boxconv_inference_forward_f32(const float* input, const float* x_min, const float* x_max,
+                                  const float* y_min, const float* y_max, float* real_parameters,
+                                  float* input_integrated, float* output, int batch, int in_planes,
+                                  int num_filters, int h, int w, double reparametrization_h,
+                                  double reparametrization_w, int normalize, int exact, void* workspace,
+                                  size_t workspace_bytes, void* stream) {
+    // (the stored bounds are only read: the job does not project)
+    return training_forward_impl<float>(input, const_cast<float*>(x_min), const_cast<float*>(x_max),
+                                        const_cast<float*>(y_min), const_cast<float*>(y_max), real_parameters,
+                                        input_integrated, output, batch, in_planes, num_filters, h, w,
+                                        reparametrization_h, reparametrization_w, 0.0, 0.0, normalize, exact,
+                                        workspace, workspace_bytes, stream, false);
+}
+int boxconv_inference_forward_f64(const double* input, const double* x_min, const double* x_max,
+                                  const double* y_min, const double* y_max, double* real_parameters,
+                                  double* input_integrated, double* output, int batch, int in_planes,
+                                  int num_filters, int h, int w, double reparametrization_h,
+                                  double reparametrization_w, int normalize, int exact, void* workspace,
+                                  size_t workspace_bytes, void* stream) {
+    return training_forward_impl<double>(input, const_cast<double*>(x_min), const_cast<double*>(x_max),
+                                         const_cast<double*>(y_min), const_cast<double*>(y_max), real_parameters,
+                                         input_integrated, output, batch, in_planes, num_filters, h, w,
+                                         reparametrization_h, reparametrization_w, 0.0, 0.0, normalize, exact,
+                                         workspace, workspace_bytes, stream, false);
 }
 
 int boxconv_forward_fused_f32(const float* input_integrated, const float* x_min,

@@ -383,15 +383,18 @@ __device__ __forceinline__ void clip_pair(T& pmin, T& pmax, double reparam, doub
     pmax = static_cast<T>(hi);
 }
 
-// Box i of a clip job: both pairs clipped in place, and optionally written in real pixel units.
+// Box i of a clip job: both pairs clipped in place (if the job projects), and optionally written in
+// real pixel units.
 template <class T>
 __device__ __forceinline__ void clip_box(const ClipArgs<T>& c, int i) {
     T a = c.xmin[i], b = c.xmax[i];
-    clip_pair(a, b, c.reparam_h, c.min_size, c.max_h);
-    c.xmin[i] = a; c.xmax[i] = b;
     T lo = c.ymin[i], hi = c.ymax[i];
-    clip_pair(lo, hi, c.reparam_w, c.min_size, c.max_w);
-    c.ymin[i] = lo; c.ymax[i] = hi;
+    if (c.project) {                                   // (off: the bounds are only converted, nothing is stored to them)
+        clip_pair(a, b, c.reparam_h, c.min_size, c.max_h);
+        c.xmin[i] = a; c.xmax[i] = b;
+        clip_pair(lo, hi, c.reparam_w, c.min_size, c.max_w);
+        c.ymin[i] = lo; c.ymax[i] = hi;
+    }
     if (c.real != nullptr) {
         // a T tensor times a Python float: the scalar is rounded to T, then one T multiplication
         const T sh = static_cast<T>(c.reparam_h), sw = static_cast<T>(c.reparam_w);

@@ -151,10 +151,11 @@ struct ClipArgs {
     T* real;
     int n;
     double reparam_h, reparam_w, max_h, max_w, min_size;
+    int project;          // 0: the stored bounds are left as they are (only `real` is written)
 };
 template <class T>
 ClipArgs<T> clip_args(T* xmin, T* xmax, T* ymin, T* ymax, T* real, int n, double reparam_h,
-                      double reparam_w, double max_h, double max_w, bool exact);
+                      double reparam_w, double max_h, double max_w, bool exact, bool project = true);
 
 // The clip job and whatever the integral-image launch that follows needs done to `aux`
 // beforehand, in one launch. *prepared: pass it on to integral_image_launch.

@@ -1,11 +1,11 @@
-// Host-side fast path of BoxConv2d's training step: the autograd node in C++.
+// Host-side fast path of BoxConv2d's forward and backward: the autograd node in C++.
 //
 // What it replaces: the Python glue around the two native calls of a training step,
 //   box_convolution/box_convolution_function.py (BoxConvolutionFunction.forward / .backward, the
 //   counterpart of the reference's box_convolution/box_convolution_function.py:30-65) and the
 //   tensor-level checks and allocations of box_convolution/_native.py,
-// for the common case only: training mode (parameters clipped on the way in), float32 or
-// float64, everything on one GPU. On the layer shapes of the reference's model zoo the kernels of
+// for the common case only: float32 or float64, everything on one GPU; training mode (parameters
+// clipped on the way in) and eval mode (parameters only read). On the layer shapes of the reference's model zoo the kernels of
 // a step take under 100 us, and the Python versions of this glue cost more than that per step
 // (argument checks, seven tensor allocations, two ctypes calls with 22 and 24 arguments, and the
 // autograd engine calling back into Python from its own thread). Here the engine calls straight
@@ -31,6 +31,9 @@ using TrainingForwardFn = int (*)(const T*, T*, T*, T*, T*, T*, T*, T*, int, int
 template <class T>
 using BackwardFn = int (*)(const T*, const T*, const T*, const T*, const T*, const T*, const T*, float, float,
                            int, int, T*, T*, T*, T*, T*, int, int, int, int, int, void*, size_t, void*);
+template <class T>
+using InferenceForwardFn = int (*)(const T*, const T*, const T*, const T*, const T*, T*, T*, T*, int, int, int, int,
+                                   int, double, double, int, int, void*, size_t, void*);
 using IntegralWorkspaceFn = size_t (*)(int64_t, int, int);
 using BackwardWorkspaceFn = size_t (*)(int, int, int, int, int, int, int, int);
 using LastErrorFn = const char* (*)();
@@ -38,6 +41,8 @@ using LastErrorFn = const char* (*)();
 struct Abi {
     void* training_forward_f32 = nullptr;
     void* training_forward_f64 = nullptr;
+    void* inference_forward_f32 = nullptr;
+    void* inference_forward_f64 = nullptr;
     void* backward_f32 = nullptr;
     void* backward_f64 = nullptr;
     IntegralWorkspaceFn integral_workspace_bytes = nullptr;
@@ -51,6 +56,13 @@ template <> TrainingForwardFn<float> training_forward_fn<float>() {
 }
 template <> TrainingForwardFn<double> training_forward_fn<double>() {
     return reinterpret_cast<TrainingForwardFn<double>>(g_abi.training_forward_f64);
+}
+template <class T> InferenceForwardFn<T> inference_forward_fn();
+template <> InferenceForwardFn<float> inference_forward_fn<float>() {
+    return reinterpret_cast<InferenceForwardFn<float>>(g_abi.inference_forward_f32);
+}
+template <> InferenceForwardFn<double> inference_forward_fn<double>() {
+    return reinterpret_cast<InferenceForwardFn<double>>(g_abi.inference_forward_f64);
 }
 template <class T> BackwardFn<T> backward_fn();
 template <> BackwardFn<float> backward_fn<float>() { return reinterpret_cast<BackwardFn<float>>(g_abi.backward_f32); }
@@ -87,11 +99,13 @@ void* ptr_or_null(const at::Tensor& t) { return t.defined() ? t.data_ptr() : nul
 
 // ---- the autograd node -----------------------------------------------------------------------------
 struct TrainingStep : public torch::autograd::Function<TrainingStep> {
-    // Returns the output [B, C*F, h, w]. x_min .. y_max are the stored parameters, clipped in place.
+    // Returns the output [B, C*F, h, w]. x_min .. y_max are the stored parameters, clipped in place
+    // if `clip` (training mode), only read otherwise (eval mode).
     static at::Tensor forward(torch::autograd::AutogradContext* ctx, const at::Tensor& input,
                               const at::Tensor& x_min, const at::Tensor& x_max, const at::Tensor& y_min,
                               const at::Tensor& y_max, double reparam_h, double reparam_w, double max_h,
-                              double max_w, bool normalize, bool exact, int64_t stream, bool capturing) {
+                              double max_w, bool normalize, bool exact, bool clip, int64_t stream,
+                              bool capturing) {
         const at::Tensor in = input.contiguous();
         const int64_t B = in.size(0), C = in.size(1), h = in.size(2), w = in.size(3), F = x_min.size(1);
         const auto opts = in.options();
@@ -100,15 +114,25 @@ struct TrainingStep : public torch::autograd::Function<TrainingStep> {
         at::Tensor real = at::empty({4, C, F}, opts);
         const size_t nbytes = g_abi.integral_workspace_bytes(B * C, static_cast<int>(h), static_cast<int>(w));
         at::Tensor ws = workspace(nbytes, in.device(), static_cast<uint64_t>(stream), capturing);
-        AT_DISPATCH_FLOATING_TYPES(in.scalar_type(), "boxconv_training_forward", [&] {
-            check_rc(training_forward_fn<scalar_t>()(
-                         in.data_ptr<scalar_t>(), x_min.data_ptr<scalar_t>(), x_max.data_ptr<scalar_t>(),
-                         y_min.data_ptr<scalar_t>(), y_max.data_ptr<scalar_t>(), real.data_ptr<scalar_t>(),
-                         integrated.data_ptr<scalar_t>(), output.data_ptr<scalar_t>(), static_cast<int>(B),
-                         static_cast<int>(C), static_cast<int>(F), static_cast<int>(h), static_cast<int>(w),
-                         reparam_h, reparam_w, max_h, max_w, normalize ? 1 : 0, exact ? 1 : 0, ptr_or_null(ws),
-                         nbytes, reinterpret_cast<void*>(stream)),
-                     "training_forward");
+        AT_DISPATCH_FLOATING_TYPES(in.scalar_type(), "boxconv_module_forward", [&] {
+            if (clip)
+                check_rc(training_forward_fn<scalar_t>()(
+                             in.data_ptr<scalar_t>(), x_min.data_ptr<scalar_t>(), x_max.data_ptr<scalar_t>(),
+                             y_min.data_ptr<scalar_t>(), y_max.data_ptr<scalar_t>(), real.data_ptr<scalar_t>(),
+                             integrated.data_ptr<scalar_t>(), output.data_ptr<scalar_t>(), static_cast<int>(B),
+                             static_cast<int>(C), static_cast<int>(F), static_cast<int>(h), static_cast<int>(w),
+                             reparam_h, reparam_w, max_h, max_w, normalize ? 1 : 0, exact ? 1 : 0,
+                             ptr_or_null(ws), nbytes, reinterpret_cast<void*>(stream)),
+                         "training_forward");
+            else
+                check_rc(inference_forward_fn<scalar_t>()(
+                             in.data_ptr<scalar_t>(), x_min.data_ptr<scalar_t>(), x_max.data_ptr<scalar_t>(),
+                             y_min.data_ptr<scalar_t>(), y_max.data_ptr<scalar_t>(), real.data_ptr<scalar_t>(),
+                             integrated.data_ptr<scalar_t>(), output.data_ptr<scalar_t>(), static_cast<int>(B),
+                             static_cast<int>(C), static_cast<int>(F), static_cast<int>(h), static_cast<int>(w),
+                             reparam_h, reparam_w, normalize ? 1 : 0, exact ? 1 : 0, ptr_or_null(ws), nbytes,
+                             reinterpret_cast<void*>(stream)),
+                         "inference_forward");
         });
         // (as the reference: the integral image and the bounds in pixel units; the saved forward
         // output is not needed, the backward kernels rebuild the one sum that would use it)
@@ -173,7 +197,7 @@ struct TrainingStep : public torch::autograd::Function<TrainingStep> {
                          "box_convolution_backward");
             });
         }
-        torch::autograd::variable_list grads(13);             // one per argument of forward
+        torch::autograd::variable_list grads(14);             // one per argument of forward
         grads[0] = grad_input;
         if (any_param) {
             const auto parts = grad_params.unbind(0);
@@ -188,7 +212,7 @@ struct TrainingStep : public torch::autograd::Function<TrainingStep> {
 // reference (src/box_convolution_interface.cpp:19-34), same messages.
 at::Tensor training_step(const at::Tensor& input, const at::Tensor& x_min, const at::Tensor& x_max,
                          const at::Tensor& y_min, const at::Tensor& y_max, double reparam_h, double reparam_w,
-                         double max_h, double max_w, bool normalize, bool exact, int64_t stream,
+                         double max_h, double max_w, bool normalize, bool exact, bool clip, int64_t stream,
                          bool capturing) {
     TORCH_CHECK(g_abi.last_error != nullptr, "box_convolution: the native glue was not initialised");
     TORCH_CHECK(input.is_cuda(), "box_convolution: input is on '", input.device(),
@@ -201,7 +225,7 @@ at::Tensor training_step(const at::Tensor& input, const at::Tensor& x_min, const
         TORCH_CHECK(p->device() == input.device(), "BoxConv2d: input and parameters are on different devices");
         TORCH_CHECK(p->scalar_type() == input.scalar_type(), "box_convolution: input and parameters have different dtypes (",
                     input.scalar_type(), ", ", p->scalar_type(), ")");
-        TORCH_CHECK(p->is_contiguous(), "box_convolution: parameters must be contiguous to be clipped in place");
+        TORCH_CHECK(!clip || p->is_contiguous(), "box_convolution: parameters must be contiguous to be clipped in place");
         TORCH_CHECK(p->dim() == 2, "BoxConv2d: all parameters must have 2 dimensions");
         TORCH_CHECK(p->size(0) == input.size(1),
                     "BoxConv2d: all parameters must have as many rows as there are input channels");
@@ -209,15 +233,22 @@ at::Tensor training_step(const at::Tensor& input, const at::Tensor& x_min, const
     }
     TORCH_CHECK(input.size(2) >= 1 && input.size(3) >= 1, "BoxConv2d: input must be at least 1x1");
     TORCH_CHECK(reparam_h > 0 && reparam_w > 0, "box_convolution: reparametrization factors must be positive");
-    return TrainingStep::apply(input, x_min, x_max, y_min, y_max, reparam_h, reparam_w, max_h, max_w, normalize,
-                               exact, stream, capturing);
+    if (clip)
+        return TrainingStep::apply(input, x_min, x_max, y_min, y_max, reparam_h, reparam_w, max_h, max_w,
+                                   normalize, exact, clip, stream, capturing);
+    // only read: any layout will do (contiguous() is the tensor itself where it already is)
+    return TrainingStep::apply(input, x_min.contiguous(), x_max.contiguous(), y_min.contiguous(),
+                               y_max.contiguous(), reparam_h, reparam_w, max_h, max_w, normalize, exact, clip,
+                               stream, capturing);
 }
 
-void init(uint64_t training_forward_f32, uint64_t training_forward_f64, uint64_t backward_f32,
-          uint64_t backward_f64, uint64_t integral_workspace_bytes, uint64_t backward_workspace_bytes,
+void init(uint64_t training_forward_f32, uint64_t training_forward_f64, uint64_t inference_forward_f32,
+          uint64_t inference_forward_f64, uint64_t backward_f32, uint64_t backward_f64, uint64_t integral_workspace_bytes, uint64_t backward_workspace_bytes,
           uint64_t last_error) {
     g_abi.training_forward_f32 = reinterpret_cast<void*>(training_forward_f32);
     g_abi.training_forward_f64 = reinterpret_cast<void*>(training_forward_f64);
+    g_abi.inference_forward_f32 = reinterpret_cast<void*>(inference_forward_f32);
+    g_abi.inference_forward_f64 = reinterpret_cast<void*>(inference_forward_f64);
     g_abi.backward_f32 = reinterpret_cast<void*>(backward_f32);
     g_abi.backward_f64 = reinterpret_cast<void*>(backward_f64);
     g_abi.integral_workspace_bytes = reinterpret_cast<IntegralWorkspaceFn>(integral_workspace_bytes);
@@ -235,6 +266,7 @@ void release_workspaces() {
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("init", &init, "hand over the addresses of the C ABI entry points of libboxconv_hip.so");
     m.def("training_step", &training_step,
-          "BoxConv2d.forward in training mode with its backward as a C++ autograd node");
+          "BoxConv2d.forward (training mode: clip = true; eval mode: clip = false) with its backward as a C++ "
+          "autograd node");
     m.def("release_workspaces", &release_workspaces);
 }

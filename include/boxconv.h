@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define BOXCONV_ABI_VERSION 2
+#define BOXCONV_ABI_VERSION 3
 
 #define BOXCONV_E_INVALID_ARGUMENT (-1) /* null pointer, non-positive size, ... */
 #define BOXCONV_E_WORKSPACE        (-2) /* workspace missing or smaller than *_workspace_bytes() */
@@ -171,6 +171,25 @@ int boxconv_training_forward_f64(const double* input, double* x_min, double* x_m
                                  int w, double reparametrization_h, double reparametrization_w,
                                  double max_input_h, double max_input_w, int normalize, int exact,
                                  void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- eval-mode forward in one call --------------------------------------------------------------
+ * What `BoxConv2d.forward` does when `self.training` is false (reference
+ * box_convolution/box_convolution_module.py:208-214 and box_convolution_function.py:41-46): no
+ * clipping; stored -> real units, integral_image, box_convolution_forward. The stored bounds are
+ * only read. Same results as `stored * reparametrization`, boxconv_integral_image_* and
+ * boxconv_forward_* in turn; arguments as for boxconv_training_forward_* without the clip limits. */
+int boxconv_inference_forward_f32(const float* input, const float* x_min, const float* x_max,
+                                  const float* y_min, const float* y_max, float* real_parameters,
+                                  float* input_integrated, float* output, int batch, int in_planes,
+                                  int num_filters, int h, int w, double reparametrization_h,
+                                  double reparametrization_w, int normalize, int exact, void* workspace,
+                                  size_t workspace_bytes, void* stream);
+int boxconv_inference_forward_f64(const double* input, const double* x_min, const double* x_max,
+                                  const double* y_min, const double* y_max, double* real_parameters,
+                                  double* input_integrated, double* output, int batch, int in_planes,
+                                  int num_filters, int h, int w, double reparametrization_h,
+                                  double reparametrization_w, int normalize, int exact, void* workspace,
+                                  size_t workspace_bytes, void* stream);
 
 /* ---- forward, half-precision output and fused tail (inference) ------------------------------
  * The same box sums as boxconv_forward_f32 (reference src/box_convolution_interface.cpp:13-139),

@@ -77,6 +77,12 @@ def test_argument_errors_are_reported_without_launching(lib):
     rc = lib.boxconv_training_forward_f32(null, null, null, null, null, null, null, null, 1, 1, 1, 4, 4,
                                           f64(8.0), f64(8.0), f64(4.0), f64(4.0), 1, 1, null, 0, null)
     assert rc == -1 and b"null parameter pointer" in lib.boxconv_last_error()
+    rc = lib.boxconv_inference_forward_f32(null, null, null, null, null, null, null, null, 1, 1, 1, 4, 4,
+                                           f64(8.0), f64(8.0), 1, 1, null, 0, null)
+    assert rc == -1 and b"null parameter pointer" in lib.boxconv_last_error()
+    rc = lib.boxconv_inference_forward_f64(dummy16, dummy16, dummy16, dummy16, dummy16, dummy16, dummy16,
+                                           dummy16, 1, 1, 1, 4, 4, f64(8.0), f64(-1.0), 1, 1, null, 0, null)
+    assert rc == -1 and b"positive" in lib.boxconv_last_error()
     rc = lib.boxconv_training_forward_f32(dummy16, dummy16, dummy16, dummy16, dummy16, dummy16, dummy16,
                                           dummy16, 1, 1, 1, 4, 4, f64(0.0), f64(8.0), f64(4.0), f64(4.0),
                                           1, 1, null, 0, null)

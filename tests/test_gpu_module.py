@@ -403,6 +403,52 @@ def test_cpp_autograd_node_matches_the_python_function(hip, dtype, needs):
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("grad", [True, False])
+def test_cpp_autograd_node_in_eval_mode(hip, dtype, grad):
+    """In eval mode the module's forward goes through the same C++ node without the clip
+    (reference box_convolution/box_convolution_module.py:203-214: clip_parameters only when
+    training): parameters that are out of bounds stay as they are, and output and gradients are
+    those of BoxConvolutionFunction without `clip_to`, bit for bit; under no_grad there is no
+    graph."""
+    if hip.glue() is None:
+        pytest.skip("the C++ glue was not built")
+    B, C, F, h, w = 2, 3, 4, 33, 70
+    random.seed(6)
+    torch.manual_seed(6)
+    m = BoxConv2d(C, F, h, w).to(DEV, dtype)
+    m.eval()
+    with torch.no_grad():
+        m.x_min.mul_(3.0)              # out of bounds on purpose; eval mode must not touch them
+    names = ("x_min", "x_max", "y_min", "y_max")
+    before = [getattr(m, n).detach().clone() for n in names]
+    x = torch.randn(B, C, h, w, device=DEV, dtype=dtype, requires_grad=grad)
+    g = torch.randn(B, C * F, h, w, device=DEV, dtype=dtype)
+    if grad:
+        out = m(x)
+        assert type(out.grad_fn).__name__ != "BoxConvolutionFunctionBackward"
+        out.backward(g)
+        got = (out.detach(), x.grad, [getattr(m, n).grad.clone() for n in names])
+        for n in names:
+            getattr(m, n).grad = None
+        x2 = x.detach().clone().requires_grad_(True)
+        ref = BoxConvolutionFunction.apply(x2, m.x_min, m.x_max, m.y_min, m.y_max, m.reparametrization_h,
+                                           m.reparametrization_w, m.normalize, m.exact, None)
+        ref.backward(g)
+        assert torch.equal(got[0], ref.detach()) and torch.equal(got[1], x2.grad)
+        for a, n in zip(got[2], names):
+            assert torch.equal(a, getattr(m, n).grad)
+    else:
+        with torch.no_grad():
+            out = m(x)
+            ref = BoxConvolutionFunction.apply(x, m.x_min, m.x_max, m.y_min, m.y_max, m.reparametrization_h,
+                                               m.reparametrization_w, m.normalize, m.exact, None)
+        assert out.grad_fn is None and not out.requires_grad
+        assert torch.equal(out, ref)
+    for a, n in zip(before, names):
+        assert torch.equal(a, getattr(m, n).detach())
+
+
 def test_cpp_autograd_node_reports_the_reference_errors(hip):
     if hip.glue() is None:
         pytest.skip("the C++ glue was not built")

@@ -279,6 +279,57 @@ def test_module_trains_end_to_end():
     assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in m.parameters())
 
 
+def test_training_trajectory_matches_the_cpu_twin(oracle):
+    """Twenty steps of SGD with momentum on a BoxConv2d layer (GPU, the module as a user calls
+    it: clip, unit conversion, integral image, sampling, backward) against the same loop on the
+    host with the CPU oracle in the place of every native call (clip_parameters at the start of
+    each training forward, reference box_convolution/box_convolution_module.py:203-206). Losses
+    and the final parameters must agree: a difference in any gradient, in the clip or in the
+    units would compound over the steps."""
+    random.seed(11)
+    torch.manual_seed(11)
+    B, C, F, h, w = 2, 3, 4, 30, 44
+    m = BoxConv2d(C, F, h, w).to(DEV)
+    names = ("x_min", "x_max", "y_min", "y_max")
+    twin = [getattr(m, n).detach().cpu().numpy().copy() for n in names]
+    x = torch.randn(B, C, h, w)
+    target = torch.randn(B, C * F, h, w) * 0.1 + x.repeat_interleave(F, dim=1) * 0.5
+    lr, mom, steps = 2e-3, 0.9, 20
+    opt = torch.optim.SGD(m.parameters(), lr=lr, momentum=mom)
+    xg, tg = x.to(DEV), target.to(DEV)
+    m.train()
+    losses_gpu, losses_cpu = [], []
+    velocity = [np.zeros_like(p) for p in twin]
+    moved = 0.0
+    start = [p.copy() for p in twin]
+    for step in range(steps):
+        opt.zero_grad()
+        out = m(xg)
+        loss = ((out - tg) ** 2).mean()
+        loss.backward()
+        opt.step()
+        losses_gpu.append(loss.item())
+        # the twin: clip in place, forward, loss, backward, the same momentum update in float32
+        oracle.clip_parameters(*twin, m.reparametrization_h, m.reparametrization_w, m.max_input_h, m.max_input_w, True)
+        out_c, saved = oracle.module_forward(x.numpy(), *twin, m.reparametrization_h, m.reparametrization_w, True, True)
+        diff = out_c - target.numpy()
+        losses_cpu.append(float((diff.astype(np.float64) ** 2).mean()))
+        grad_out = (2.0 / diff.size * diff).astype(np.float32)
+        grads = oracle.module_backward(saved, grad_out, m.reparametrization_h, m.reparametrization_w, True, True,
+                                       (False, True, True, True, True))
+        for k in range(4):
+            velocity[k] = (mom * velocity[k] + grads[1 + k]).astype(np.float32) if step else grads[1 + k].copy()
+            twin[k] = (twin[k] - np.float32(lr) * velocity[k]).astype(np.float32)
+    for a, b in zip(losses_gpu, losses_cpu):
+        assert abs(a - b) <= 1e-4 * abs(b), (losses_gpu, losses_cpu)
+    for n, want, first in zip(names, twin, start):
+        got = getattr(m, n).detach().cpu().numpy()
+        moved = max(moved, float(np.abs(want - first).max()))
+        assert np.abs(got - want).max() <= 1e-4 * np.abs(want).max(), n
+    assert moved > 1e-3, "the parameters hardly moved: the test would not notice a wrong gradient"
+    assert losses_gpu[-1] < losses_gpu[0]
+
+
 def test_noncontiguous_input_and_dtype_errors(hip):
     x = torch.randn(2, 2, 9, 20, device=DEV)[..., ::2]
     assert not x.is_contiguous()

@@ -178,6 +178,7 @@ def time_steps(step, steps, repeats):
 def small_workload_extra(k, dev, steps=200):
     """Eager and captured-graph step time of a small workload (its kernels take tens of
     microseconds, so the eager figure is what the host can enqueue)."""
+    import torch
     from baseline_workloads import algorithmic_bytes, make_workload
     wl = make_workload(k)
     module, x, g, eager_step = make_step(wl, dev)
@@ -190,6 +191,17 @@ def small_workload_extra(k, dev, steps=200):
         replay()
     graph, _, _ = time_steps(replay, steps, 3)
     del keep
+    # the inference forward of the same layer: module.eval(), no autograd
+    module.eval()
+    x_eval = x.detach()
+
+    def eval_forward():
+        with torch.no_grad():
+            module(x_eval)
+    for _ in range(20):
+        eval_forward()
+    infer, _, _ = time_steps(eval_forward, steps, 3)
+    module.train()
     return {
         "workload": wl.name,
         "eager_ms_per_step": round(1e3 * eager / steps, 4),
@@ -197,6 +209,7 @@ def small_workload_extra(k, dev, steps=200):
         "eager_GBps": round(ab["alg"] / (eager / steps) / 1e9, 1),
         "graph_GBps": round(ab["alg"] / (graph / steps) / 1e9, 1),
         "eager_over_graph": round(eager / graph, 2),
+        "eval_forward_ms": round(1e3 * infer / steps, 4),
     }
 
 

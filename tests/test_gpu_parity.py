@@ -352,14 +352,15 @@ def test_grad_output_pass_variants_agree(hip, oracle, switches, h, w, exact):
         assert np.abs(a - b).max() <= 1e-5 * max(np.abs(b).max(), 1e-30) + 1e-6 * max(np.abs(t).max() for t in back_b[1:])
 
 
-@pytest.mark.parametrize("h,w", [(64, 20), (96, 200), (128, 256), (256, 512), (64, 1024), (128, 2500)])
-def test_workspace_layouts_agree(hip, oracle, switches, h, w):
+@pytest.mark.parametrize("h,w,F", [(64, 20, 3), (64, 40, 5), (96, 200, 3), (128, 256, 2), (256, 512, 3),
+                                   (64, 1024, 3), (128, 2500, 2)])
+def test_workspace_layouts_agree(hip, oracle, switches, h, w, F):
     """Planes that are cut into whole bands of a power-of-two number of rows keep the rows of the
     column workspace interleaved over the bands (row k of every band side by side);
     BOXCONV_M_INTERLEAVE=0 keeps them in their natural order. Only the place of a row changes,
     so the two give the same bits, and both meet the oracle."""
     rng = np.random.default_rng(h * 7 + w)
-    B, C, F = 2, 2, 3
+    B, C = 2, 2
     x = rng.standard_normal((B, C, h, w)).astype(np.float32)
     g = (rng.standard_normal((B, C * F, h, w)) + 0.25).astype(np.float32)
     boxes = tuple(make_boxes(rng, C, F, h, w, "hanging", away_from_integers=0.05))

@@ -171,7 +171,25 @@ class BoxConv2d(torch.nn.Module):
     _HALF_TYPES = (torch.float16, torch.bfloat16)
     _GLUE_TYPES = (torch.float32, torch.float64)
 
+    # The native library indexes a tensor with 32 bits: batch * in_planes * num_filters *
+    # (h+1) * (w+1) must stay below 2^31 (include/boxconv.h, BOXCONV_E_TOO_LARGE).
+    _MAX_ELEMENTS = 2 ** 31 - 1
+
+    def _batch_limit(self, input):
+        """How many batch items one native call can take (None: no limit applies)."""
+        if input.dim() != 4 or not input.is_cuda:
+            return None
+        per_item = self.in_planes * max(self.num_filters, 1) * (input.size(2) + 1) * (input.size(3) + 1)
+        limit = self._MAX_ELEMENTS // max(per_item, 1)
+        return limit if 1 <= limit < input.size(0) else None
+
     def forward(self, input):
+        limit = self._batch_limit(input)
+        if limit is not None:
+            # A batch too large for one native call goes through in slices: box convolution is
+            # independent per batch item, and autograd adds the slices' parameter gradients up.
+            # (The clip of a training-mode forward is a projection: repeating it changes nothing.)
+            return torch.cat([self.forward(part) for part in input.split(limit, dim=0)], dim=0)
         if input.dtype in self._HALF_TYPES:
             return self._forward_half(input)
         clip_to = None

@@ -524,3 +524,76 @@ def test_copy_probe_copies(hip, w, rows, in_flight):
     assert bool((dst[:, 0] == -7.0).all())
     with pytest.raises(RuntimeError):
         hip.probe_copy_bands(src, dst, 48, 2)
+
+
+def test_batches_too_large_for_one_native_call_go_through_in_slices(monkeypatch):
+    """The library indexes with 32 bits and refuses batch * planes * filters * (h+1) * (w+1) >=
+    2^31; the module then feeds the batch through in slices. Here with the limit lowered so that a
+    small batch is cut into three uneven slices: output, grad_input and the parameter gradients
+    are those of the single call."""
+    random.seed(8)
+    torch.manual_seed(8)
+    B, C, F, h, w = 7, 2, 3, 20, 33
+    m = BoxConv2d(C, F, h, w).to(DEV)
+    m.train()
+    x = torch.randn(B, C, h, w, device=DEV, requires_grad=True)
+    g = torch.randn(B, C * F, h, w, device=DEV)
+    m(x).backward(g)
+    whole = (x.grad.clone(), [p.grad.clone() for p in m.parameters()])
+    out_whole = m(x).detach()
+    x.grad = None
+    for p in m.parameters():
+        p.grad = None
+    per_item = C * F * (h + 1) * (w + 1)
+    monkeypatch.setattr(BoxConv2d, "_MAX_ELEMENTS", 3 * per_item + 5)      # slices of 3, 3 and 1
+    assert m._batch_limit(x) == 3
+    out = m(x)
+    out.backward(g)
+    assert torch.equal(out.detach(), out_whole)
+    assert torch.equal(x.grad, whole[0])
+    for p, want in zip(m.parameters(), whole[1]):
+        assert torch.allclose(p.grad, want, rtol=1e-5, atol=1e-6 * float(want.abs().max()))
+
+
+def test_output_of_more_than_2_31_elements(hip):
+    """The real thing: 130 x 4 planes x 8 filters of 512 x 1024 (8.7 GB of output, 2^31 elements
+    are reached at batch 128). A single native call is refused; the module's forward and
+    backward work, and agree with the batch items run one at a time."""
+    free, _ = torch.cuda.mem_get_info()
+    if free < 60 * 2 ** 30:
+        pytest.skip("needs 60 GB of free device memory")
+    random.seed(9)
+    torch.manual_seed(9)
+    B, C, F, h, w = 130, 4, 8, 512, 1024
+    m = BoxConv2d(C, F, h, w).to(DEV)
+    m.train()
+    x = torch.randn(B, C, h, w, device=DEV, requires_grad=True)
+    with pytest.raises(RuntimeError, match="2\\^31"):
+        hip.integral_image(torch.empty(B * C * F, h, w, device=DEV))
+    assert m._batch_limit(x) == 127
+    g = torch.randn(B, C * F, h, w, device=DEV)
+    out = m(x)
+    assert out.shape == (B, C * F, h, w)
+    out.backward(g)
+    gin = x.grad
+    gpar = [p.grad.clone() for p in m.parameters()]
+    for p in m.parameters():
+        p.grad = None
+    acc = [torch.zeros(C, F, device=DEV, dtype=torch.float64) for _ in range(4)]
+    worst_out = worst_gin = 0.0
+    for b in range(B):
+        xb = x.detach()[b:b + 1].clone().requires_grad_(True)
+        ob = m(xb)
+        ob.backward(g[b:b + 1])
+        for a, p in zip(acc, m.parameters()):
+            a += p.grad.double()
+            p.grad = None
+        if b in (0, 1, 63, 126, 127, 129):
+            worst_out = max(worst_out, float((ob.detach() - out.detach()[b:b + 1]).abs().max() / ob.detach().abs().max()))
+            worst_gin = max(worst_gin, float((xb.grad - gin[b:b + 1]).abs().max() / xb.grad.abs().max()))
+    assert worst_out <= 2e-6 and worst_gin <= 2e-6, (worst_out, worst_gin)
+    for got, want in zip(gpar, acc):
+        assert float((got.double() - want).abs().max()) <= 1e-4 * float(want.abs().max())
+    del out, gin, g, x
+    torch.cuda.empty_cache()
+    hip.release_workspaces()

@@ -127,10 +127,13 @@ def training_step(input, x_min, x_max, y_min, y_max, reparametrization_h, repara
     stored parameters in place first; without it (eval mode) they are only read. Returns the
     output; its backward gives the five gradients. Same native calls as
     ``BoxConvolutionFunction`` (with ``clip_to`` in training mode). Requires ``glue()``."""
-    return _glue.training_step(
-        input, x_min, x_max, y_min, y_max, float(reparametrization_h), float(reparametrization_w),
-        float(max_input_h), float(max_input_w), bool(normalize), bool(exact), bool(clip),
-        _stream(input.device) or 0, torch.cuda.is_current_stream_capturing())
+    # (the backward runs on the autograd engine's thread for input's device, which makes that
+    # device current itself)
+    with _on_device(input.device):
+        return _glue.training_step(
+            input, x_min, x_max, y_min, y_max, float(reparametrization_h), float(reparametrization_w),
+            float(max_input_h), float(max_input_w), bool(normalize), bool(exact), bool(clip),
+            _stream(input.device) or 0, torch.cuda.is_current_stream_capturing())
 
 
 def _check(rc, what):

@@ -855,8 +855,21 @@ grad_output_stream_kernel(SampleArgs<T> a) {
     };
     // (written out twice rather than through another lambda: arrays captured through two levels
     // of closures end up in scratch memory)
+    // double: one loop body serves every pair of pairs, also a band's last two (the second then
+    // prefetches rows that nothing uses: clamped integral rows, and rows of grad_output past the
+    // band, which read as zeros). With the band's end written out as a third and a fourth copy of
+    // the pair body, as for the other types, the copy for "two pairs left" returned wrong
+    // parameter sums for double rows of 1537 to 2047 columns in rounded mode (the kernel spills
+    // some 500 registers at that size); the loop body itself never did.
 #define BOXCONV_ALL_PAIRS(OWN_W_TAG)                                         \
-    {                                                                        \
+    if constexpr (sizeof(T) == 8) {                                          \
+        int i = i0;                                                          \
+        for (; i + 2 < i1; i += 4) {                                         \
+            row_pair(i, std::true_type{}, Flip0{}, OWN_W_TAG{});             \
+            row_pair(i + 2, std::true_type{}, Flip1{}, OWN_W_TAG{});         \
+        }                                                                    \
+        if (i < i1) row_pair(i, std::false_type{}, Flip0{}, OWN_W_TAG{});    \
+    } else {                                                                 \
         int i = i0;                                                          \
         for (; i + 4 < i1; i += 4) {                                         \
             row_pair(i, std::true_type{}, Flip0{}, OWN_W_TAG{});             \

@@ -199,6 +199,9 @@ SMALL_CASES = [
     (1, 1, 2, 12, 1100), (1, 1, 1, 9, 2100), (1, 1, 2, 1, 1), (1, 1, 2, 1, 70), (1, 1, 2, 70, 1),
     (1, 1, 2, 12, 700), (1, 2, 1, 10, 768), (1, 1, 2, 11, 1300), (1, 1, 1, 9, 1536),   # three columns per lane
     (1, 1, 2, 40, 2048), (1, 2, 2, 21, 1800), (1, 1, 1, 10, 2047),      # 512 threads, four columns per lane
+    # the same shape with an even number of row pairs per band (a band then ends in the second LDS
+    # buffer; float64 in rounded mode once returned wrong parameter gradients exactly there)
+    (1, 1, 2, 4, 1538), (2, 1, 3, 32, 1537), (1, 1, 4, 8, 1800), (1, 1, 2, 16, 2047), (1, 1, 2, 12, 1300),
     # narrow images with four filters or more: the waves of a grad-input workgroup share the
     # filters (one turn with idle waves, two turns with the second partial, full-width rows)
     (1, 2, 4, 9, 20), (1, 2, 11, 19, 33), (2, 1, 16, 12, 64),

@@ -526,6 +526,48 @@ def test_copy_probe_copies(hip, w, rows, in_flight):
         hip.probe_copy_bands(src, dst, 48, 2)
 
 
+def test_modules_on_concurrent_streams_give_the_serial_bits():
+    """Three layers stepping at the same time on streams of their own (one of them at a shape that
+    takes the single-pass integral image, whose workgroups wait for each other): every call keeps
+    its scratch per stream and the results are those of the calls run one after the other, bit
+    for bit."""
+    random.seed(12)
+    torch.manual_seed(12)
+    shapes = [(2, 8, 4, 256, 512), (4, 16, 4, 64, 128), (1, 4, 8, 128, 1024)]
+    mods, xs, gs, refs = [], [], [], []
+    for (B, C, F, h, w) in shapes:
+        m = BoxConv2d(C, F, h, w).to(DEV)
+        m.train()
+        x = torch.randn(B, C, h, w, device=DEV, requires_grad=True)
+        g = torch.randn(B, C * F, h, w, device=DEV)
+        out = m(x)
+        out.backward(g)
+        refs.append((out.detach().clone(), x.grad.clone(), [p.grad.clone() for p in m.parameters()]))
+        x.grad = None
+        for p in m.parameters():
+            p.grad = None
+        mods.append(m), xs.append(x), gs.append(g)
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in shapes]
+    for _ in range(5):
+        outs = []
+        for s, m, x, g in zip(streams, mods, xs, gs):
+            s.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(s):
+                out = m(x)
+                out.backward(g)
+                outs.append(out)
+        for s in streams:
+            torch.cuda.current_stream().wait_stream(s)
+        torch.cuda.synchronize()
+        for m, x, out, ref in zip(mods, xs, outs, refs):
+            assert torch.equal(out.detach(), ref[0]) and torch.equal(x.grad, ref[1])
+            for p, want in zip(m.parameters(), ref[2]):
+                assert torch.equal(p.grad, want)
+                p.grad = None
+            x.grad = None
+
+
 def test_batches_too_large_for_one_native_call_go_through_in_slices(monkeypatch):
     """The library indexes with 32 bits and refuses batch * planes * filters * (h+1) * (w+1) >=
     2^31; the module then feeds the batch through in slices. Here with the limit lowered so that a

@@ -261,24 +261,33 @@ def test_backward_across_row_bands(hip, oracle, h, w, kind):
     assert_parity(cpu, gpu, np.float32, "%s %dx%d" % (kind, h, w), **sc)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("exact", [True, False])
-@pytest.mark.parametrize("h,w", [(12, 40), (70, 300), (40, 1024)])
-def test_backward_lower_bound_one_ulp_above_an_integer(hip, oracle, h, w, exact):
+@pytest.mark.parametrize("h,w", [(12, 40), (70, 300), (40, 1024), (16, 512), (9, 700), (33, 1500), (36, 1800),
+                                 (40, 2048), (18, 3000)])
+def test_backward_lower_bound_one_ulp_above_an_integer(hip, oracle, h, w, exact, dtype):
     """A lower bound so close above an integer that `bound - 1` rounds to the integer below: the
     split the reference uses for the parameter gradients (src/box_convolution.cpp:80-96) and the
     mirrored split it uses for the input gradient (:51-67) then cut the box at different whole
     pixels. The grad_output pass computes separate column weights for the two in that case; in
-    rounded mode a shared set would put a whole column of grad_input off."""
+    rounded mode a shared set would put a whole column of grad_input off. The widths reach every
+    workgroup shape of that pass; the heights give bands with odd and with even numbers of row
+    pairs."""
     rng = np.random.default_rng(h * 31 + w + int(exact))
     B, C, F = 1, 2, 2
-    x = rng.standard_normal((B, C, h, w)).astype(np.float32)
-    g = rng.standard_normal((B, C * F, h, w)).astype(np.float32)
-    just_above = np.nextafter(np.float32(-1.0), np.float32(0.0))     # -0.99999994
-    assert np.float32(just_above - np.float32(1.0)) == np.float32(-2.0)
-    x_min = np.array([[just_above, -3.3], [np.nextafter(np.float32(-3.0), np.float32(0.0)), -0.4]], np.float32)
-    x_max = np.array([[4.6, 2.2], [5.0, 3.5]], np.float32)
-    y_min = np.array([[just_above, just_above], [-7.25, np.nextafter(np.float32(-2.0), np.float32(0.0))]], np.float32)
-    y_max = np.array([[6.4, 9.0], [3.75, 11.5]], np.float32)
+    x = rng.standard_normal((B, C, h, w)).astype(dtype)
+    g = rng.standard_normal((B, C * F, h, w)).astype(dtype)
+    one = dtype(1.0)
+
+    def above(v):
+        return np.nextafter(dtype(v), dtype(0.0))
+
+    just_above = above(-1.0)                                         # float32: -0.99999994
+    assert dtype(just_above - one) == dtype(-2.0)
+    x_min = np.array([[just_above, -3.3], [above(-3.0), -0.4]], dtype)
+    x_max = np.array([[4.6, 2.2], [5.0, 3.5]], dtype)
+    y_min = np.array([[just_above, just_above], [-7.25, above(-2.0)]], dtype)
+    y_max = np.array([[6.4, 9.0], [3.75, 11.5]], dtype)
     for normalize in (False, True):
         # Rounded mode with normalisation: the reference's second summand multiplies grad_output with
         # the saved forward output (forward split), while the sums of the grad_output pass follow the
@@ -286,7 +295,7 @@ def test_backward_lower_bound_one_ulp_above_an_integer(hip, oracle, h, w, exact)
         # column, and the GPU takes that one sum again with the forward split (finalize_box).
         cpu, gpu, sc = run_both(hip, oracle, x, (x_min, x_max, y_min, y_max), 3.5 * h, 2.25 * w,
                                 normalize, exact, g)
-        assert_parity(cpu, gpu, np.float32, "normalize=%s exact=%s" % (normalize, exact), **sc)
+        assert_parity(cpu, gpu, dtype, "normalize=%s exact=%s" % (normalize, exact), **sc)
 
 
 @pytest.mark.parametrize("w", [48, 100, 200])

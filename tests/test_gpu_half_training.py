@@ -67,6 +67,35 @@ def test_backward_reads_and_writes_half_precision(hip, oracle, shape, kind, dtyp
             assert np.abs(got[i].cpu().numpy() - want[i]).max() <= 1e-3 * scale + noise, (normalize, exact, i)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("h,w", [(14, 60), (24, 1024)])
+def test_half_grad_output_with_a_bound_one_ulp_above_an_integer(hip, oracle, h, w, dtype):
+    """Rounded mode with normalisation and a lower bound one ulp above an integer: the one sum
+    that is then taken again with the forward split (finalize_box) reads grad_output in its own
+    half type."""
+    rng = np.random.default_rng(h + w)
+    B, C, F = 1, 2, 2
+    x = rng.standard_normal((B, C, h, w)).astype(np.float32)
+    g_half = torch.from_numpy(rng.standard_normal((B, C * F, h, w)).astype(np.float32)).to(dtype)
+    g32 = g_half.float().numpy()
+    just_above = np.nextafter(np.float32(-1.0), np.float32(0.0))
+    boxes = (np.array([[just_above, -3.3], [np.nextafter(np.float32(-3.0), np.float32(0.0)), -0.4]], np.float32),
+             np.array([[4.6, 2.2], [5.0, 3.5]], np.float32),
+             np.array([[just_above, just_above], [-7.25, np.nextafter(np.float32(-2.0), np.float32(0.0))]], np.float32),
+             np.array([[6.4, 9.0], [3.75, 11.5]], np.float32))
+    integ_c = oracle.integral_image(x)
+    out_c = oracle.box_forward(integ_c, *boxes, True, False)
+    want = oracle.box_backward(integ_c, *boxes, g32, out_c, 3.0 * h, 2.0 * w, True, False, (True,) * 5)
+    integ = hip.integral_image(torch.from_numpy(x).to(DEV))
+    got = hip.box_convolution_backward(integ, *[torch.from_numpy(b).to(DEV) for b in boxes], g_half.to(DEV), None,
+                                       3.0 * h, 2.0 * w, True, False, True, True, True, True, True)
+    gi, ref = got[0].float().cpu().numpy(), want[0]
+    assert np.all(np.abs(gi - ref) <= HALF_ULP[dtype] * np.abs(ref) + 1e-4 * np.abs(ref).max())
+    floor = param_grad_floor(want[1:])
+    for i in range(1, 5):
+        assert np.abs(got[i].cpu().numpy() - want[i]).max() <= 1e-3 * max(np.abs(want[i]).max(), floor), i
+
+
 def make_module(C, F, h, w, seed):
     random.seed(seed)
     return BoxConv2d(C, F, h, w).to(DEV)

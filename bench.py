@@ -269,6 +269,22 @@ def machine_probes(dev):
     assert torch.equal(dst[:, 1:], src)
     print("(the backward's streaming pass moves these 1074 MB plus 67 MB of integral images per launch, in "
           "workgroups of 64 rows)")
+    del src, dst
+    # the grad-input pass's loads and stores without its arithmetic, with the headline workload's boxes
+    from baseline_workloads import make_workload
+    wl = make_workload(3)
+    x_lo = torch.ceil(-wl.x_max * wl.reparametrization_h).to(torch.int32).to(dev)
+    x_hi = (torch.floor(-wl.x_min * wl.reparametrization_h) + 1).to(torch.int32).to(dev)
+    planes = wl.B * wl.C
+    m = torch.randn(planes, wl.F, wl.h + 1, wl.w, device=dev)
+    out = torch.empty(planes, wl.h, wl.w, device=dev)
+    m_bytes, out_bytes = 4 * m.numel(), 4 * out.numel()
+    for mode, what in ((0, "both runs of 9 rows per filter (the kernel's pattern)"),
+                       (1, "one run per filter: every row of the workspace read once"),
+                       (2, "one run from the workspace, the other from a few MB resident in the L2")):
+        t = timed(lambda: _native.probe_grad_input_pattern(m, out, x_lo, x_hi, mode))
+        print("%-72s %7.1f us  %.2f TB/s" % ("grad-input pattern, " + what, t * 1e6, (m_bytes + out_bytes) / t / 1e12))
+    print("(TB/s on the 537 MB of the column workspace read once plus the 67 MB written)")
 
 
 def main():

@@ -32,6 +32,7 @@ _SIGNATURES = {
     "boxconv_profile_arm_every": (_i, [ctypes.c_char_p, _i]),
     "boxconv_profile_collect": (_i, [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int)]),
     "boxconv_probe_copy_bands": (_i, [_vp, _vp, _i64, _i, _i, _i, _i, _vp]),
+    "boxconv_probe_grad_input_pattern": (_i, [_vp, _vp, _vp, _vp, _i64, _i, _i, _i, _i, _vp]),
     "boxconv_integral_image_workspace_bytes": (_sz, [_i64, _i, _i]),
     "boxconv_backward_workspace_bytes": (_sz, [_i, _i, _i, _i, _i, _i, _i, _i]),
 }
@@ -641,6 +642,22 @@ def probe_copy_bands(src, dst, rows_per_group, rows_in_flight):
         raise RuntimeError("probe_copy_bands: contiguous float32 device tensors [planes,h,w] -> [planes,h+1,w]")
     _check(load().boxconv_probe_copy_bands(_ptr(src), _ptr(dst), planes, h, w, rows_per_group,
                                            rows_in_flight, _stream(src.device)), "probe_copy_bands")
+
+
+def probe_grad_input_pattern(column_workspace, out, x_lo, x_hi, mode):
+    """The grad-input pass's loads and stores without its arithmetic (a measurement yardstick, see
+    include/boxconv.h): column_workspace [planes, F, h+1, 1024] float32, out [planes, h, 1024],
+    x_lo / x_hi [C, F] int32 row offsets of the two runs."""
+    planes, F, h1, w = column_workspace.shape
+    C = x_lo.shape[0]
+    ok = (w == 1024 and tuple(out.shape) == (planes, h1 - 1, w) and tuple(x_lo.shape) == (C, F)
+          and tuple(x_hi.shape) == (C, F) and x_lo.dtype == torch.int32 and x_hi.dtype == torch.int32
+          and column_workspace.dtype == torch.float32 and out.dtype == torch.float32
+          and all(t.is_cuda and t.is_contiguous() for t in (column_workspace, out, x_lo, x_hi)))
+    if not ok:
+        raise RuntimeError("probe_grad_input_pattern: float32 [planes,F,h+1,1024] -> [planes,h,1024], int32 [C,F] offsets")
+    _check(load().boxconv_probe_grad_input_pattern(_ptr(column_workspace), _ptr(out), _ptr(x_lo), _ptr(x_hi), planes,
+                                                   C, F, h1 - 1, mode, _stream(out.device)), "probe_grad_input_pattern")
 
 
 def profile_collect():

@@ -44,7 +44,72 @@ probe_copy_bands_kernel(const float* __restrict__ src, float* __restrict__ dst, 
     }
 }
 
+// The loads and stores of the grad-input pass without its arithmetic: a workgroup of 256 lanes
+// owns 8 output rows of one plane (rows of 1024 floats, 16 bytes per lane) and reads, for each of
+// F filters, the 9 rows from i0 + xlo[f] - 1 and the 9 rows from i0 + xhi[f] of that filter's
+// plane of M (h + 1 rows), clamped to [0, h]; it writes the 8 rows of their blend.
+// mode 0: both runs (the kernel's pattern); 1: the bottom run only (every row of M is then read
+// once); 2: the bottom run from M, the top run from the first 97 rows of the XCD's first planes
+// (a few MB that stay in the L2: what the second read costs when it always hits).
+template <int MODE>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3)))
+probe_grad_input_pattern_kernel(const float* __restrict__ M, float* __restrict__ out, const int* __restrict__ xlo,
+                                const int* __restrict__ xhi, int C, int F, int h, int64_t per_xcd, int64_t total) {
+    unsigned vid = xcd_contiguous_id(per_xcd);
+    if (vid >= total) return;
+    vid = static_cast<unsigned>(total) - 1u - vid;                  // last to first, like the kernel
+    const unsigned groups = static_cast<unsigned>(h / 8);
+    const int i0 = static_cast<int>(vid % groups) * 8;
+    const int64_t p = vid / groups;
+    const int c = static_cast<int>(p % C);
+    probe_f4 acc[8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) acc[r] = probe_f4{0.f, 0.f, 0.f, 0.f};
+    const int64_t mplane = static_cast<int64_t>(h + 1) * 1024;
+#pragma unroll 1
+    for (int f = 0; f < F; ++f) {
+        const int lo = xlo[c * F + f], hi = xhi[c * F + f];
+        const float* plane = M + (p * F + f) * mplane + 4 * threadIdx.x;
+        const float* resident = M + (static_cast<int64_t>(blockIdx.x % kXcds) * F + f) * mplane + 4 * threadIdx.x;
+        probe_f4 T[9], B[9];
+#pragma unroll
+        for (int r = 0; r <= 8; ++r) {
+            const int rt = min(max(i0 + r + lo - 1, 0), h), rb = min(max(i0 + r + hi, 0), h);
+            if (MODE == 0) T[r] = *reinterpret_cast<const probe_f4*>(plane + static_cast<int64_t>(rt) * 1024);
+            if (MODE == 2) T[r] = *reinterpret_cast<const probe_f4*>(resident + static_cast<int64_t>((rt * 7) % 97) * 1024);
+            B[r] = *reinterpret_cast<const probe_f4*>(plane + static_cast<int64_t>(rb) * 1024);
+        }
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            if (MODE == 1) acc[r] += B[r] + 0.25f * (B[r + 1] - B[r]);
+            else acc[r] += (B[r] - T[r + 1]) + 0.25f * (B[r + 1] - B[r]) + 0.5f * (T[r + 1] - T[r]);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 8; ++r)
+        *reinterpret_cast<probe_f4*>(out + (p * h + i0 + r) * 1024 + 4 * threadIdx.x) = acc[r];
+}
+
 }  // namespace
+
+hipError_t probe_grad_input_pattern_launch(const float* M, float* out, const int* xlo, const int* xhi,
+                                           int64_t planes, int C, int F, int h, int mode, hipStream_t stream) {
+    const int64_t total = planes * (h / 8);
+    const int64_t per_xcd = (total + kXcds - 1) / kXcds;
+    const dim3 grid(static_cast<unsigned>(per_xcd * kXcds)), block(256);
+    if (mode == 0)
+        BOXCONV_LAUNCH("probe_grad_input_pattern", (probe_grad_input_pattern_kernel<0>), grid, block, 0, stream, M, out,
+                       xlo, xhi, C, F, h, per_xcd, total);
+    else if (mode == 1)
+        BOXCONV_LAUNCH("probe_grad_input_pattern", (probe_grad_input_pattern_kernel<1>), grid, block, 0, stream, M, out,
+                       xlo, xhi, C, F, h, per_xcd, total);
+    else if (mode == 2)
+        BOXCONV_LAUNCH("probe_grad_input_pattern", (probe_grad_input_pattern_kernel<2>), grid, block, 0, stream, M, out,
+                       xlo, xhi, C, F, h, per_xcd, total);
+    else
+        return hipErrorInvalidValue;
+    return hipGetLastError();
+}
 
 hipError_t probe_copy_bands_launch(const float* src, float* dst, int64_t planes, int h, int w, int rows,
                                    int rows_in_flight, hipStream_t stream) {

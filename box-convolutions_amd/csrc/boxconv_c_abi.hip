@@ -485,6 +485,23 @@ int boxconv_probe_copy_bands(const float* src, float* dst, int64_t planes, int h
                       "copy probe launch");
 }
 
+int boxconv_probe_grad_input_pattern(const float* column_workspace, float* out, const int* x_lo,
+                                     const int* x_hi, int64_t planes, int in_planes, int num_filters, int h,
+                                     int mode, void* stream) {
+    if (planes < 1 || in_planes < 1 || num_filters < 1 || h < 8 || h % 8 != 0 || mode < 0 || mode > 2)
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "grad-input pattern probe: invalid sizes planes=%lld in_planes=%d "
+                    "num_filters=%d h=%d mode=%d", static_cast<long long>(planes), in_planes, num_filters, h, mode);
+    if (mode == 2 && (h < 97 || planes < 8))
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "grad-input pattern probe: mode 2 needs h >= 97 and 8 planes");
+    if (!column_workspace || !out || !x_lo || !x_hi)
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "grad-input pattern probe: null pointer");
+    if (planes * num_filters * static_cast<int64_t>(h + 1) * 1024 > kMaxElems)
+        return fail(BOXCONV_E_TOO_LARGE, "grad-input pattern probe: workspace exceeds 2^31-1 elements");
+    return hip_result(boxconv::probe_grad_input_pattern_launch(column_workspace, out, x_lo, x_hi, planes, in_planes,
+                                                               num_filters, h, mode, static_cast<hipStream_t>(stream)),
+                      "grad-input pattern probe launch");
+}
+
 int boxconv_integral_image_static_f32(const float* in, float* out, int64_t planes, int h, int w,
                                       void* stream) {
     return integral_image_static_impl(in, out, planes, h, w, stream);

@@ -66,6 +66,11 @@ hipError_t integral_image_int_launch(const void* in, void* out, int dtype, int64
 hipError_t probe_copy_bands_launch(const float* src, float* dst, int64_t planes, int h, int w, int rows,
                                    int rows_in_flight, hipStream_t stream);
 
+// The grad-input pass's loads and stores without its arithmetic (see
+// boxconv_probe_grad_input_pattern in include/boxconv.h); the caller has checked the sizes.
+hipError_t probe_grad_input_pattern_launch(const float* M, float* out, const int* xlo, const int* xhi,
+                                           int64_t planes, int C, int F, int h, int mode, hipStream_t stream);
+
 template <class T>
 hipError_t forward_launch(const T* integ, BoxParams<T> prm, T* out, Dims d, bool normalize,
                           bool exact, hipStream_t stream);

@@ -56,7 +56,7 @@ void boxconv_reload_env(void);
  * alone, whatever else the entry point launches). Names: "band_colsum", "band_prefix",
  * "band_scan", "forward_rows", "grad_output_stream", "grad_input_cols",
  * "param_grad_finalize", "fill_zero", "fill_marker", "clip", "forward_gather", "grad_input_gather",
- * "int_row_prefix", "int_col_prefix", "probe_copy_bands",
+ * "int_row_prefix", "int_col_prefix", "probe_copy_bands", "probe_grad_input_pattern",
  * "grad_params_gather".
  * NULL or "" disarms. Arming discards earlier measurements.
  * boxconv_profile_arm_every(name, n): the same, but only every n-th launch of that kernel (the
@@ -78,6 +78,18 @@ int boxconv_profile_collect(double* total_ms, int* launches);
  * rows_per_group, rows_per_group a multiple of rows_in_flight. */
 int boxconv_probe_copy_bands(const float* src, float* dst, int64_t planes, int h, int w,
                              int rows_per_group, int rows_in_flight, void* stream);
+
+/* The loads and stores of the backward's grad-input pass without its arithmetic (measurement aid;
+ * no counterpart in the reference), for rows of 1024 floats: column_workspace holds
+ * planes * num_filters planes of (h+1) x 1024 floats, out planes of h x 1024. A workgroup owns 8
+ * output rows i0.. of a plane and reads, per filter f of input plane c = plane % in_planes, the 9
+ * rows from i0 + x_lo[c*F+f] - 1 and the 9 rows from i0 + x_hi[c*F+f] (clamped to [0, h]) of that
+ * filter's plane, 16 bytes per lane and row, as the kernel does. mode 0: both runs; 1: the second
+ * run only (every row is then read once); 2: the first run from a few MB that stay in the L2
+ * (what the second read of a row costs when it always hits). h a multiple of 8. */
+int boxconv_probe_grad_input_pattern(const float* column_workspace, float* out, const int* x_lo,
+                                     const int* x_hi, int64_t planes, int in_planes, int num_filters, int h,
+                                     int mode, void* stream);
 
 /* ---- integral image ------------------------------------------------------------------------
  * Replaces `integral_image(Tensor) -> Tensor`, reference src/integral_image_interface.cpp:8-27

@@ -69,6 +69,10 @@ def test_argument_errors_are_reported_without_launching(lib):
     assert rc == -1 and b"copy probe" in lib.boxconv_last_error()
     rc = lib.boxconv_probe_copy_bands(null, null, 4, 64, 1024, 64, 2, null)
     assert rc == -1 and b"null" in lib.boxconv_last_error()
+    rc = lib.boxconv_probe_grad_input_pattern(dummy16, dummy16, dummy16, dummy16, 8, 2, 3, 100, 0, null)   # h % 8
+    assert rc == -1 and b"pattern probe" in lib.boxconv_last_error()
+    rc = lib.boxconv_probe_grad_input_pattern(dummy16, dummy16, null, dummy16, 8, 2, 3, 104, 0, null)
+    assert rc == -1 and b"null" in lib.boxconv_last_error()
     rc = lib.boxconv_integral_image_half_f32(dummy16, 1, dummy16, 1, 4, 4096, null, 0, null)
     assert rc == -3 and b"2048" in lib.boxconv_last_error()
     assert lib.boxconv_profile_arm_every(b"forward_rows", 0) == -1

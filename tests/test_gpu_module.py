@@ -639,3 +639,35 @@ def test_output_of_more_than_2_31_elements(hip):
     del out, gin, g, x
     torch.cuda.empty_cache()
     hip.release_workspaces()
+
+
+def test_grad_input_pattern_probe_reads_the_rows_it_is_priced_on(hip):
+    """The benchmark's second yardstick (the grad-input pass's loads and stores without its
+    arithmetic): with every plane of the workspace holding its own constant the blend of the two
+    runs cancels (mode 0) and the single run returns the sum of the constants (mode 1); with rows
+    that hold their row index, mode 1 returns the clamped row positions."""
+    planes, C, F, h = 8, 2, 3, 104
+    x_lo = torch.tensor([[-5, -40, 2], [-1, -90, -7]], dtype=torch.int32, device="cuda")
+    x_hi = torch.tensor([[6, 3, 30], [1, 80, -2]], dtype=torch.int32, device="cuda")
+    consts = torch.arange(1, planes * F + 1, device="cuda", dtype=torch.float32).view(planes, F, 1, 1)
+    m = consts.expand(planes, F, h + 1, 1024).contiguous()
+    out = torch.full((planes, h, 1024), -1.0, device="cuda")
+    hip.probe_grad_input_pattern(m, out, x_lo, x_hi, 0)
+    assert bool((out == 0).all())
+    hip.probe_grad_input_pattern(m, out, x_lo, x_hi, 1)
+    assert torch.equal(out, consts.sum(1).expand(planes, h, 1024))
+    rows = torch.arange(h + 1, device="cuda", dtype=torch.float32).view(1, 1, h + 1, 1)
+    m = rows.expand(planes, F, h + 1, 1024).contiguous()
+    hip.probe_grad_input_pattern(m, out, x_lo, x_hi, 1)
+    i = torch.arange(h, device="cuda").view(1, h, 1)
+    want = torch.zeros(planes, h, 1, device="cuda")
+    for p in range(planes):
+        for f in range(F):
+            b0 = (i[0] + int(x_hi[p % C, f])).clamp(0, h).float()
+            b1 = (i[0] + 1 + int(x_hi[p % C, f])).clamp(0, h).float()
+            want[p] += b0 + 0.25 * (b1 - b0)
+    assert torch.allclose(out, want.expand(planes, h, 1024), rtol=0, atol=1e-4)
+    hip.probe_grad_input_pattern(m, out, x_lo, x_hi, 2)          # (runs; its values are not meaningful)
+    torch.cuda.synchronize()
+    with pytest.raises(RuntimeError):
+        hip.probe_grad_input_pattern(m, out, x_lo, x_hi, 3)

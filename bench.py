@@ -257,6 +257,13 @@ def machine_probes(dev):
         t = timed(fn)
         print("%-72s %7.1f us  %.2f TB/s" % (name, t * 1e6, nbytes / t / 1e12))
     del a, b, c
+    # the size of the headline's integral image: input planes in, integral planes out
+    small_in = torch.randn(32, 512, 1024, device=dev)
+    small_out = torch.empty_like(small_in)
+    t = timed(lambda: small_out.copy_(small_in))
+    print("%-72s %7.1f us  %.2f TB/s" % ("torch copy_, 64 MiB read + 64 MiB written (the integral image's bytes)",
+                                         t * 1e6, 8 * small_in.numel() / t / 1e12))
+    del small_in, small_out
     planes, h, w = 256, 512, 1024        # grad_output of the headline workload: 2 x 16 x 8 planes
     src = torch.randn(planes, h, w, device=dev)
     dst = torch.zeros(planes, h + 1, w, device=dev)

@@ -29,6 +29,10 @@ Switches read_switches() {
     s.lookback = e == nullptr || std::atoi(e) != 0;
     s.lookback_any_shape = e != nullptr && std::atoi(e) == 2;
     s.stream_consecutive = flag_unless_zero("BOXCONV_STREAM_CONSEC");
+    {
+        const char* e = text("BOXCONV_STREAM_CONSEC");
+        s.stream_consecutive_partial = e == nullptr || (e[0] != '0' && e[0] != '1');
+    }
     s.interleave_workspace = flag_unless_zero("BOXCONV_M_INTERLEAVE");
     e = text("BOXCONV_STREAM_WGS");
     s.stream_workgroups = e != nullptr ? std::max(1, std::atoi(e)) : 2048;

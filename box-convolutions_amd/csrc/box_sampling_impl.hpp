@@ -900,7 +900,7 @@ grad_output_stream_kernel(SampleArgs<T> a) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// The same pass for float rows that fill the workgroup's column slots exactly (w == 4 * NT), both
+// The same pass for float rows of a multiple of four columns (w <= 4 * NT; FULL: w == 4 * NT), both
 // products at once: a lane owns 4 CONSECUTIVE columns for everything, where
 // grad_output_stream_kernel gives it the columns lane, lane + 64, ... of its wave and moves the
 // weights W through LDS to get consecutive ones for the suffix sum. With consecutive columns
@@ -914,6 +914,9 @@ grad_output_stream_kernel(SampleArgs<T> a) {
 // Same arithmetic, same order of additions inside a lane's row pair; the sums differ from the
 // other kernel's only in which columns share a lane. Everything said there about the math, the
 // two splits, the single barrier per row pair (MERGED) and the cache policy of the stores applies.
+// !FULL: the lanes past the row's end (whole lanes, since w is a multiple of four) load from the
+// row's first columns and drop what they loaded where it would be used: they put zeros into LDS
+// (the row's right-hand padding), hold zero weights and a zero V, and store nothing.
 typedef float f4_dword_aligned __attribute__((ext_vector_type(4), aligned(4)));
 __device__ __forceinline__ void load4_dword_aligned(const float* p, float (&v)[4]) {
     const f4_dword_aligned q = *reinterpret_cast<const f4_dword_aligned*>(p);
@@ -923,7 +926,7 @@ __device__ __forceinline__ void load4_dword_aligned(const float* p, float (&v)[4
 // Two waves per SIMD on purpose, although the registers would allow three: with three, more
 // workgroups are resident per XCD than share one integral plane of the input, two planes compete
 // for its L2, and the kernel gets slower (226 against 217 us at 512 x 1024).
-template <class TG, int NT, bool EXACT>
+template <class TG, int NT, bool EXACT, bool FULL>
 __global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2)))
 grad_output_stream_consec_kernel(SampleArgs<float> a) {
     using T = float;
@@ -952,6 +955,9 @@ grad_output_stream_consec_kernel(SampleArgs<float> a) {
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int c0 = K * tid;                          // the lane's first pixel column
+    const bool lane_in = FULL || c0 < w;             // (w is a multiple of K: a lane is in or out as a whole)
+    const int cl = lane_in ? c0 : 0;                 // idle lanes load the row's first columns
+    const int owner = FULL ? NT - 1 : w / K - 1;     // the lane whose last column is column w
 
     const BoxOfWorkgroup<T> bx = load_box(a.prm, k_par);
     const BoxSplit<T> s = split_grad_params(bx.xmin, bx.xmax, bx.ymin, bx.ymax);
@@ -974,11 +980,13 @@ grad_output_stream_consec_kernel(SampleArgs<float> a) {
 
     // integral row r, columns c0+1 .. c0+4; rows of grad_output, columns c0 .. c0+3 (a row past the
     // band is read from a valid address and cleared afterwards)
+    // (what an idle lane loads is discarded where it would be used, not here: a select right
+    // behind a load makes the lane wait for it at once)
     auto load_i = [&](int r, T (&dst)[K]) {
-        load4_dword_aligned(iplane + static_cast<int64_t>(r) * pitch + 1 + c0, dst);
+        load4_dword_aligned(iplane + static_cast<int64_t>(r) * pitch + 1 + cl, dst);
     };
     auto load_g = [&](int i, T (&dst)[K]) {
-        load_quad(gplane + static_cast<int64_t>(min(i, h - 1)) * w + c0, dst);
+        load_quad(gplane + static_cast<int64_t>(min(i, h - 1)) * w + cl, dst);
     };
     auto load_window = [&](int i, T (&t0)[K], T (&t1)[K], T (&b1)[K], T (&b2)[K]) {
         load_i(clampi(i + s.xlo, 0, h), t0);
@@ -1017,7 +1025,7 @@ grad_output_stream_consec_kernel(SampleArgs<float> a) {
         T d[K];
 #pragma unroll
         for (int k = 0; k < K; ++k) {
-            d[k] = tail_weight(c0 + k, s.ylo, s.yhi, s.fylo, s.fyhi);
+            d[k] = lane_in ? tail_weight(c0 + k, s.ylo, s.yhi, s.fylo, s.fyhi) : T(0);
             wave_has_tail = wave_has_tail || d[k] != T(0);
         }
         *reinterpret_cast<Quad<T>*>(&delta[c0]) = Quad<T>{{d[0], d[1], d[2], d[3]}};
@@ -1046,6 +1054,10 @@ grad_output_stream_consec_kernel(SampleArgs<float> a) {
             _Pragma("unroll")                                                                       \
             for (int k = 0; k < K; ++k) GB[k] = T(0);                                               \
         }                                                                                           \
+        if (!FULL && !lane_in) {                                                                    \
+            _Pragma("unroll")                                                                       \
+            for (int k = 0; k < K; ++k) { GA[k] = T(0); GB[k] = T(0); }                             \
+        }                                                                                           \
         Quad<T>* dst = reinterpret_cast<Quad<T>*>(&grow[FL][kPad + c0]);                            \
         dst[0] = Quad<T>{{GA[0], GB[0], GA[1], GB[1]}};                                             \
         dst[1] = Quad<T>{{GA[2], GB[2], GA[3], GB[3]}};                                             \
@@ -1055,7 +1067,7 @@ grad_output_stream_consec_kernel(SampleArgs<float> a) {
             _Pragma("unroll")                                                                       \
             for (int k = 0; k < K; ++k) { TL0 += dq.v[k] * GA[k]; TL1 += dq.v[k] * GB[k]; }         \
         }                                                                                           \
-        if (tid == NT - 1) {                                                                        \
+        if (tid == owner) {                                                                         \
             const T dt0 = T0[K - 1] - TA[K - 1], db0 = B1[K - 1] - BC[K - 1];                       \
             const T dt1 = T1[K - 1] - T0[K - 1], db1 = B2[K - 1] - B1[K - 1];                       \
             T v0 = BC[K - 1] - T0[K - 1], v1 = B1[K - 1] - T1[K - 1];                               \
@@ -1110,6 +1122,7 @@ grad_output_stream_consec_kernel(SampleArgs<float> a) {
                     wq0[k] += s.fyhi * dr0; wq0[k] += s.fylo * dl0;
                     wq1[k] += s.fyhi * dr1; wq1[k] += s.fylo * dl1;
                 }
+                if (!FULL && !lane_in) { wq0[k] = T(0); wq1[k] = T(0); }    // (no column q > w)
                 const T dt0 = t0[k] - ta[k], db0 = b1[k] - bc[k];
                 const T dt1 = t1[k] - t0[k], db1 = b2[k] - b1[k];
                 T v0 = bc[k] - t0[k], v1 = b1[k] - t1[k];
@@ -1117,6 +1130,9 @@ grad_output_stream_consec_kernel(SampleArgs<float> a) {
                     v0 += s.fxhi * db0; v0 += s.fxlo * dt0;
                     v1 += s.fxhi * db1; v1 += s.fxlo * dt1;
                 }
+                // (an idle lane: its weights are zero, which takes care of the products with dt and
+                // db; its V must go as well, since the taps of its columns are not zero)
+                if (!FULL && !lane_in) { v0 = T(0); v1 = T(0); }
                 sum[4] += v0 * wq0[k];
                 sum[1] += db0 * wq0[k];
                 sum[0] -= dt0 * wq0[k];
@@ -1159,7 +1175,8 @@ grad_output_stream_consec_kernel(SampleArgs<float> a) {
                     wq0[k] += sm.fylo * (grA.r0 - gr.r0); wq0[k] += sm.fyhi * (gl.r0 - glA.r0);
                     wq1[k] += sm.fylo * (grA.r1 - gr.r1); wq1[k] += sm.fyhi * (gl.r1 - glA.r1);
                 }
-                const T dlt = tail_weight(c0 + k, ylo_m, yhi_m, sm.fyhi, sm.fylo);
+                if (!FULL && !lane_in) { wq0[k] = T(0); wq1[k] = T(0); }
+                const T dlt = lane_in ? tail_weight(c0 + k, ylo_m, yhi_m, sm.fyhi, sm.fylo) : T(0);
                 const RowPair<T> own = G[kPad + c0 + k];
                 tail0 += dlt * own.r0;
                 tail1 += dlt * own.r1;
@@ -1212,12 +1229,16 @@ grad_output_stream_consec_kernel(SampleArgs<float> a) {
             }
             const int first = c0 * static_cast<int>(sizeof(T));
             const int limit = static_cast<int>(mpitch * sizeof(T));
-            if (keep_in_cache) {
-                buffer_store_run<kCacheDefault, true>(out0, ob0, first, limit);
-                buffer_store_run<kCacheDefault, true>(colacc, ob1, first, limit);
-            } else {
-                buffer_store_run<kCacheStream, true>(out0, ob0, first, limit);
-                buffer_store_run<kCacheStream, true>(colacc, ob1, first, limit);
+            // (the rows are addressed by offset into one descriptor for the plane: a lane past the
+            // row's end must not store at all)
+            if (FULL || lane_in) {
+                if (keep_in_cache) {
+                    buffer_store_run<kCacheDefault, true>(out0, ob0, first, limit);
+                    buffer_store_run<kCacheDefault, true>(colacc, ob1, first, limit);
+                } else {
+                    buffer_store_run<kCacheStream, true>(out0, ob0, first, limit);
+                    buffer_store_run<kCacheStream, true>(colacc, ob1, first, limit);
+                }
             }
         }
         if (PREFETCH) {
@@ -1489,12 +1510,26 @@ hipError_t grad_output_stream_launch(const T* integ, const TG* grad_out, BoxPara
     // the sums: the kernel with consecutive columns per lane
     if constexpr (std::is_same<T, float>::value) {
         const bool aligned = reinterpret_cast<uintptr_t>(grad_out) % (4 * sizeof(TG)) == 0 && d.w % 4 == 0;
-        if (switches().stream_consecutive && rc.full && rc.K == 4 && params && scan && acc_slots > 0 && aligned) {
+        // the smallest workgroup whose lanes, four columns each, cover the row. Rows that would
+        // leave more than two fifths of its lanes idle stay with the other kernel, and so do rows
+        // that fill that kernel's column slots exactly at three columns per lane (measured, 16 x 8
+        // planes: 1920 columns 649 -> 490 us, 1280: 331 -> 295, 960: 261 -> 230, 640: 201 -> 181,
+        // 480: 165 -> 137; but 768: 196 -> 205 and 1536: 200 -> 219).
+        const int lanes = d.w / 4;
+        const int cnt = lanes <= 64 ? 64 : lanes <= 128 ? 128 : lanes <= 256 ? 256 : 512;
+        const bool covers = d.w <= 2048 &&
+            (lanes == cnt || (switches().stream_consecutive_partial && lanes * 5 >= cnt * 3 && !(rc.full && rc.K == 3)));
+        if (switches().stream_consecutive && covers && params && scan && acc_slots > 0 && aligned) {
 #define LAUNCH_GC(NT) \
-            if (exact) BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, true>), grid, dim3(NT), lds, stream, a); \
-            else       BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, false>), grid, dim3(NT), lds, stream, a)
-            if (rc.nt == 64) { LAUNCH_GC(64); } else if (rc.nt == 128) { LAUNCH_GC(128); }
-            else if (rc.nt == 256) { LAUNCH_GC(256); } else { LAUNCH_GC(512); }
+            if (lanes == NT) { \
+                if (exact) BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, true, true>), grid, dim3(NT), lds, stream, a); \
+                else       BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, false, true>), grid, dim3(NT), lds, stream, a); \
+            } else { \
+                if (exact) BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, true, false>), grid, dim3(NT), lds, stream, a); \
+                else       BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, false, false>), grid, dim3(NT), lds, stream, a); \
+            }
+            if (cnt == 64) { LAUNCH_GC(64) } else if (cnt == 128) { LAUNCH_GC(128) }
+            else if (cnt == 256) { LAUNCH_GC(256) } else { LAUNCH_GC(512) }
 #undef LAUNCH_GC
             return hipGetLastError();
         }

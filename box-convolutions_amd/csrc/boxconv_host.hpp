@@ -185,7 +185,8 @@ struct Switches {
     bool gi_split_filters;    // BOXCONV_GI_SPLIT_FILTERS=0 clears it: no filter sharing in small grad-input launches
     bool lookback;            // BOXCONV_INTEGRAL_LOOKBACK=0 clears it: no single-pass integral image
     bool lookback_any_shape;  // BOXCONV_INTEGRAL_LOOKBACK=2: single pass for every shape it covers
-    bool stream_consecutive;  // BOXCONV_STREAM_CONSEC=0 clears it: no consecutive-column variant of the grad_output pass
+    bool stream_consecutive;  // BOXCONV_STREAM_CONSEC=0 clears it: no consecutive-column variant of the grad_output pass at all
+    bool stream_consecutive_partial;  // BOXCONV_STREAM_CONSEC=1 clears it: that variant only for rows that fill its workgroup exactly
     bool interleave_workspace;  // BOXCONV_M_INTERLEAVE=0 clears it: rows of the column workspace in their natural order
     int stream_workgroups;    // BOXCONV_STREAM_WGS: workgroups the grad_output pass aims for when it cuts planes into bands (2048)
     int spin_limit;           // BOXCONV_INTEGRAL_SPIN: polls of a hand-over word before re-summing (64)

@@ -26,7 +26,8 @@ HALF_ULP = {torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}
 SHAPES = [(2, 2, 5, 20, 33), (1, 2, 2, 150, 90), (1, 1, 2, 40, 1024), (1, 2, 1, 18, 1536),
           (1, 1, 2, 12, 2048), (1, 1, 1, 9, 2100), (1, 1, 2, 8, 4096), (1, 1, 1, 6, 4100),
           (1, 2, 2, 131, 256), (1, 1, 3, 70, 512),    # rows that fill one and two waves exactly
-          (1, 2, 2, 128, 256), (2, 1, 3, 64, 100)]    # whole power-of-two bands: interleaved workspace rows
+          (1, 2, 2, 128, 256), (2, 1, 3, 64, 100),    # whole power-of-two bands: interleaved workspace rows
+          (1, 2, 2, 30, 960), (1, 1, 2, 20, 1920), (1, 1, 3, 25, 640)]   # consecutive columns per lane with idle lanes
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])

@@ -338,12 +338,16 @@ def test_grad_input_filter_sharing_matches_one_set_per_workgroup(hip, switches, 
 
 
 @pytest.mark.parametrize("exact", [True, False])
-@pytest.mark.parametrize("h,w", [(67, 256), (130, 512), (70, 1024), (66, 2048)])
+@pytest.mark.parametrize("h,w", [(67, 256), (130, 512), (70, 1024), (66, 2048),
+                                 # rows that leave lanes of that workgroup idle (whole waves, half a wave, one lane)
+                                 (36, 240), (30, 640), (40, 960), (64, 1000), (18, 1280), (22, 1800), (34, 1920),
+                                 (20, 2044), (50, 160), (33, 44)])
 def test_grad_output_pass_variants_agree(hip, oracle, switches, h, w, exact):
-    """Rows that fill a workgroup's column slots exactly (four columns per lane) run the
-    grad_output pass with consecutive columns per lane; BOXCONV_STREAM_CONSEC=0 sends them to the
-    kernel with wave-strided columns, as every other width. Both against the oracle, and against
-    each other to the last few bits (the sums differ only in which columns share a lane)."""
+    """Rows of a multiple of four columns that fill at least three fifths of a workgroup at four
+    columns per lane run the grad_output pass with consecutive columns per lane (the lanes past
+    the row's end idle along); BOXCONV_STREAM_CONSEC=0 sends them to the kernel with wave-strided
+    columns, as every other width. Both against the oracle, and against each other to the last
+    few bits (the sums differ only in which columns share a lane)."""
     rng = np.random.default_rng(h + w + int(exact))
     B, C, F = 1, 2, 3
     x = rng.standard_normal((B, C, h, w)).astype(np.float32)
@@ -353,7 +357,7 @@ def test_grad_output_pass_variants_agree(hip, oracle, switches, h, w, exact):
         boxes[1] = np.maximum(boxes[1], np.ceil(boxes[0]) + 1).astype(np.float32)
         boxes[3] = np.maximum(boxes[3], np.ceil(boxes[2]) + 1).astype(np.float32)
     results = []
-    for variant in ("1", "0"):
+    for variant in (None, "0"):
         switches("BOXCONV_STREAM_CONSEC", variant)
         cpu, gpu, sc = run_both(hip, oracle, x, tuple(boxes), 3.5 * h, 2.25 * w, True, exact, g)
         assert_parity(cpu, gpu, np.float32, "consecutive=%s %dx%d exact=%s" % (variant, h, w, exact), **sc)
@@ -361,7 +365,8 @@ def test_grad_output_pass_variants_agree(hip, oracle, switches, h, w, exact):
     (_, back_a), (_, back_b) = results
     assert np.abs(back_a[0] - back_b[0]).max() <= 2e-6 * np.abs(back_b[0]).max()
     for a, b in zip(back_a[1:], back_b[1:]):
-        assert np.abs(a - b).max() <= 1e-5 * max(np.abs(b).max(), 1e-30) + 1e-6 * max(np.abs(t).max() for t in back_b[1:])
+        # (float32 sums of a few hundred thousand products in two different orders)
+        assert np.abs(a - b).max() <= 1e-4 * max(np.abs(b).max(), 1e-30) + 1e-5 * max(np.abs(t).max() for t in back_b[1:])
 
 
 @pytest.mark.parametrize("h,w,F", [(64, 20, 3), (64, 40, 5), (96, 200, 3), (128, 256, 2), (256, 512, 3),

@@ -1368,6 +1368,14 @@ inline ColsConfig cols_config(int64_t planes, int F, int h, int w, bool allow_sp
     const int quads = (w + 3) / 4;
     c.lq = 3;
     while (c.lq < 8 && (1 << c.lq) < quads) ++c.lq;          // 8 .. 256 lanes per row group
+    // Rows wider than one strip: the strip width (one, two or four waves) that leaves the fewest
+    // lanes idle; the kernel is local to a column, so narrower strips cost nothing else
+    // (720 x 1280, 16 x 8 planes: two strips of 1024 columns 144 us, five of 256 columns 112 us).
+    if (quads > 256) {
+        auto lanes_launched = [&](int lq) { return ((quads + (1 << lq) - 1) >> lq) << lq; };
+        for (int lq = 7; lq >= 6; --lq)
+            if (lanes_launched(lq) < lanes_launched(c.lq)) c.lq = lq;
+    }
     c.rb = 8;
     c.fs = 1;
     // Small problems: more, shorter-lived waves (2 rows per lane), and the filters of a plane

@@ -926,8 +926,10 @@ __device__ __forceinline__ void load4_dword_aligned(const float* p, float (&v)[4
 // Two waves per SIMD on purpose, although the registers would allow three: with three, more
 // workgroups are resident per XCD than share one integral plane of the input, two planes compete
 // for its L2, and the kernel gets slower (226 against 217 us at 512 x 1024).
+// (Workgroups of five and six waves may run three waves per SIMD: two of them then share a CU,
+// where at two per SIMD one would leave three or two of its eight wave slots empty.)
 template <class TG, int NT, bool EXACT, bool FULL>
-__global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, 2)))
+__global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, (NT == 320 || NT == 384) ? 3 : 2)))
 grad_output_stream_consec_kernel(SampleArgs<float> a) {
     using T = float;
     constexpr int K = 4;
@@ -1518,15 +1520,14 @@ hipError_t grad_output_stream_launch(const T* integ, const TG* grad_out, BoxPara
     // the sums: the kernel with consecutive columns per lane
     if constexpr (std::is_same<T, float>::value) {
         const bool aligned = reinterpret_cast<uintptr_t>(grad_out) % (4 * sizeof(TG)) == 0 && d.w % 4 == 0;
-        // the smallest workgroup whose lanes, four columns each, cover the row. Rows that would
-        // leave more than two fifths of its lanes idle stay with the other kernel, and so do rows
-        // that fill that kernel's column slots exactly at three columns per lane (measured, 16 x 8
-        // planes: 1920 columns 649 -> 490 us, 1280: 331 -> 295, 960: 261 -> 230, 640: 201 -> 181,
-        // 480: 165 -> 137; but 768: 196 -> 205 and 1536: 200 -> 219).
+        // the smallest workgroup (whole waves) whose lanes, four columns each, cover the row. Rows
+        // that would leave more than two fifths of its lanes idle stay with the other kernel
+        // (measured, 16 x 8 planes: 1920 columns 649 -> 490 us, 960: 261 -> 230, 480: 165 -> 137).
         const int lanes = d.w / 4;
-        const int cnt = lanes <= 64 ? 64 : lanes <= 128 ? 128 : lanes <= 256 ? 256 : 512;
-        const bool covers = d.w <= 2048 &&
-            (lanes == cnt || (switches().stream_consecutive_partial && lanes * 5 >= cnt * 3 && !(rc.full && rc.K == 3)));
+        const int cnt = (lanes + 63) / 64 * 64;
+        const bool exact_fit = lanes == cnt && (cnt == 64 || cnt == 128 || cnt == 256 || cnt == 512);
+        const bool covers = d.w <= 2048 && lanes >= 1 &&
+                            (exact_fit || (switches().stream_consecutive_partial && lanes * 5 >= cnt * 3));
         if (switches().stream_consecutive && covers && params && scan && acc_slots > 0 && aligned) {
 #define LAUNCH_GC(NT) \
             if (lanes == NT) { \
@@ -1536,8 +1537,16 @@ hipError_t grad_output_stream_launch(const T* integ, const TG* grad_out, BoxPara
                 if (exact) BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, true, false>), grid, dim3(NT), lds, stream, a); \
                 else       BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, false, false>), grid, dim3(NT), lds, stream, a); \
             }
-            if (cnt == 64) { LAUNCH_GC(64) } else if (cnt == 128) { LAUNCH_GC(128) }
-            else if (cnt == 256) { LAUNCH_GC(256) } else { LAUNCH_GC(512) }
+            switch (cnt) {
+                case 64: LAUNCH_GC(64) break;
+                case 128: LAUNCH_GC(128) break;
+                case 192: LAUNCH_GC(192) break;
+                case 256: LAUNCH_GC(256) break;
+                case 320: LAUNCH_GC(320) break;
+                case 384: LAUNCH_GC(384) break;
+                case 448: LAUNCH_GC(448) break;
+                default: LAUNCH_GC(512) break;
+            }
 #undef LAUNCH_GC
             return hipGetLastError();
         }

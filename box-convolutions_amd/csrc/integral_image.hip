@@ -558,7 +558,10 @@ band_scan_lookback_kernel(const TI* __restrict__ in, float* __restrict__ out, do
 #pragma unroll
             for (int v = 0; v < 4; ++v) res[v] = static_cast<T>(left + pre[rb][v]);
             const RowRef orow = orows.row(min(row + 1, h), row < r1);
-            buffer_store_run<kCacheDefault, FULL>(res, orow, out_off, (w + 1) * static_cast<int>(sizeof(T)));
+            // (FULL: the rows are addressed by offset into one descriptor for the plane, without a
+            // bounds check of their own, so a lane past the row's end must not store)
+            if (!FULL || lane_in)
+                buffer_store_run<kCacheDefault, FULL>(res, orow, out_off, (w + 1) * static_cast<int>(sizeof(T)));
             if (tid == 0 && row < r1) dst[static_cast<int64_t>(row + 1) * W1] = T(0);
         }
     }
@@ -630,7 +633,8 @@ hipError_t launch_lookback(const TI* in, float* out, double* aux, int64_t planes
     const int spin = lookback_spin_limit();
     const dim3 grid(static_cast<unsigned>(per_xcd * kXcds));
     const dim3 block(WAVES * 64);
-    const bool vec = aligned_for_vec4(in, w), full = (w == WAVES * 256);
+    // full: every lane holds four columns of the row or none (rows of a multiple of four columns)
+    const bool vec = aligned_for_vec4(in, w), full = vec;
 #define LAUNCH_LOOKBACK(VEC, FULL)                                                                 \
     BOXCONV_LAUNCH("band_scan", (band_scan_lookback_kernel<TI, WAVES, 4, VEC, FULL>), grid, block, 0,  \
                    stream, in, out, aux, h, w, nb, R, planes, per_xcd, rev, spin)
@@ -650,10 +654,17 @@ template <class TI>
 struct LookbackByWidth<float, TI> {
     static hipError_t run(const TI* in, float* out, double* aux, int64_t planes, int h, int w, int nb,
                           int R, bool reverse, bool prepared, hipStream_t stream) {
-        if (w <= 256)       return launch_lookback<TI, 1>(in, out, aux, planes, h, w, nb, R, reverse, prepared, stream);
-        else if (w <= 512)  return launch_lookback<TI, 2>(in, out, aux, planes, h, w, nb, R, reverse, prepared, stream);
-        else if (w <= 1024) return launch_lookback<TI, 4>(in, out, aux, planes, h, w, nb, R, reverse, prepared, stream);
-        else                return launch_lookback<TI, 8>(in, out, aux, planes, h, w, nb, R, reverse, prepared, stream);
+        // as many waves as the row needs at 256 columns each
+        switch ((w + 255) / 256) {
+            case 1: return launch_lookback<TI, 1>(in, out, aux, planes, h, w, nb, R, reverse, prepared, stream);
+            case 2: return launch_lookback<TI, 2>(in, out, aux, planes, h, w, nb, R, reverse, prepared, stream);
+            case 3: return launch_lookback<TI, 3>(in, out, aux, planes, h, w, nb, R, reverse, prepared, stream);
+            case 4: return launch_lookback<TI, 4>(in, out, aux, planes, h, w, nb, R, reverse, prepared, stream);
+            case 5: return launch_lookback<TI, 5>(in, out, aux, planes, h, w, nb, R, reverse, prepared, stream);
+            case 6: return launch_lookback<TI, 6>(in, out, aux, planes, h, w, nb, R, reverse, prepared, stream);
+            case 7: return launch_lookback<TI, 7>(in, out, aux, planes, h, w, nb, R, reverse, prepared, stream);
+            default: return launch_lookback<TI, 8>(in, out, aux, planes, h, w, nb, R, reverse, prepared, stream);
+        }
     }
 };
 
@@ -693,9 +704,18 @@ IntegralPlan plan_integral(int64_t planes, int h, int w, int64_t want) {
     // planes of more than 32 bands in the first case.
     const int bands32 = (h + kLookbackRows - 1) / kLookbackRows;
     const int64_t groups = planes * bands32;                          // workgroups of the launch
-    const int64_t resident = w > 0 ? 256 * (8 / std::max(1, w / 256)) : 0;   // two waves per SIMD each
-    const bool measured_faster = (w == 256 || w == 512 || w == 1024 || w == 2048) &&
-                                 ((groups <= resident && bands32 <= 32) || groups >= 4096);
+    // workgroups that are on the chip at once: eight wave slots per CU at two waves per SIMD;
+    // workgroups of five waves and more, of which only one would fit, get three per SIMD
+    const int waves = std::max(1, (w + 255) / 256);
+    const int64_t resident = 256 * (waves <= 4 ? 8 / waves : 12 / waves);
+    // (rows of a multiple of four columns: every lane holds four columns or none. Measured on
+    // 16 x 8 or 32 x 8 planes, single pass against two: 720 x 1280 43 against 59 us, 512 x 768 27
+    // against 44, 256 x 1536 26 against 37, 512 x 1000 40 against 50, 480 x 640 35 against 41;
+    // but 540 x 960, one workgroup in sixteen too many to be resident, 63 against 51, and
+    // 1080 x 1920, 34 bands per plane, 117 against 80.)
+    // Narrower rows leave most of a wave idle in either kernel; the two passes are faster there
+    // (64 x 128: 20 against 24 us, 135 x 240: 21 against 25).
+    const bool measured_faster = w % 4 == 0 && w >= 256 && ((groups <= resident && bands32 <= 32) || groups >= 4096);
     const bool single_pass = wanted >= 2 && h > kLookbackRows && w <= 2048 && scan_by_rows(h, w, sizeof(float)) &&
                              bands32 <= kLookbackBands && (lookback_any_shape() || measured_faster);
     if (single_pass) nb = (h + kLookbackRows - 1) / kLookbackRows;

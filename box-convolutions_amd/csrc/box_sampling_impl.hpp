@@ -926,10 +926,12 @@ __device__ __forceinline__ void load4_dword_aligned(const float* p, float (&v)[4
 // Two waves per SIMD on purpose, although the registers would allow three: with three, more
 // workgroups are resident per XCD than share one integral plane of the input, two planes compete
 // for its L2, and the kernel gets slower (226 against 217 us at 512 x 1024).
-// (Workgroups of five and six waves may run three waves per SIMD: two of them then share a CU,
-// where at two per SIMD one would leave three or two of its eight wave slots empty.)
+// (Workgroups of three, five and six waves may run three waves per SIMD: four or two of them then
+// share a CU, where at two per SIMD two, three or two of its eight wave slots would stay empty.
+// Measured at three waves: 480 x 640 170 -> 149 us; rows of 960 and 1000 columns, four waves with
+// idle lanes, got slower with three per SIMD like the full rows: 230 -> 235 us.)
 template <class TG, int NT, bool EXACT, bool FULL>
-__global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, (NT == 320 || NT == 384) ? 3 : 2)))
+__global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, (NT == 192 || NT == 320 || NT == 384) ? 3 : 2)))
 grad_output_stream_consec_kernel(SampleArgs<float> a) {
     using T = float;
     constexpr int K = 4;

@@ -1518,8 +1518,8 @@ hipError_t grad_output_stream_launch(const T* integ, const TG* grad_out, BoxPara
             return hipErrorInvalidValue;
         }
     }
-    // float rows of exactly four columns per lane, both products wanted, a slot per workgroup for
-    // the sums: the kernel with consecutive columns per lane
+    // float rows of a multiple of four columns, both products wanted, a slot per workgroup for the
+    // sums: the kernel with four consecutive columns per lane
     if constexpr (std::is_same<T, float>::value) {
         const bool aligned = reinterpret_cast<uintptr_t>(grad_out) % (4 * sizeof(TG)) == 0 && d.w % 4 == 0;
         // the smallest workgroup (whole waves) whose lanes, four columns each, cover the row. Rows

@@ -1,6 +1,7 @@
 // Shared by the translation units that hold the box-sampling kernels: lane/slot addressing, row
 // loads, the LDS row-pair layout, the gather helpers, and the host-side choice of workgroup shape.
-// Everything here lives in an unnamed namespace: each translation unit gets its own copy.
+// Apart from the argument block SampleArgs, which crosses translation units, everything here
+// lives in an unnamed namespace: each translation unit gets its own copy.
 #pragma once
 
 #include <cstdlib>
@@ -13,7 +14,6 @@ namespace boxconv {
 
 namespace {
 
-
 extern __shared__ __align__(16) unsigned char smem_raw[];
 
 // Largest workgroup of the row-streaming kernels (16 waves, for rows of 2049 to 4096 columns;
@@ -22,6 +22,8 @@ extern __shared__ __align__(16) unsigned char smem_raw[];
 // columns per lane, and these kernels hide HBM latency with occupancy.
 constexpr int kMaxRowThreads = 1024;
 constexpr int kMaxRowWaves = kMaxRowThreads / 64;
+
+}  // namespace
 
 template <class T>
 struct SampleArgs {
@@ -47,6 +49,8 @@ struct SampleArgs {
     int m_bands;          // rows of M interleaved over this many bands (0: rows in their natural order)
     int m_shift;          // log2 of the rows per band of M (interleaved layout only)
 };
+
+namespace {
 
 // Where row r (0..h) of a plane of the column workspace M lives. Natural order: row r. Interleaved
 // (planes of nb bands of exactly R = 2^m_shift rows): row 0 stays, row 1 + b*R + k (row k of band

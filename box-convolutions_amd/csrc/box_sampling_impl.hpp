@@ -1471,6 +1471,40 @@ hipError_t grad_input_launch(const T* gint, int band_rows, BoxParams<T> prm, TO*
 // policy (the memory-side cache holds 256 MB; the grad-input kernel reads that part first).
 inline int64_t cached_tail_bytes() { return switches().keep_tail_bytes; }
 
+// The launches of grad_output_stream_consec_kernel (`lanes` busy lanes of a workgroup of `cnt`).
+// Its instantiations are a translation unit of their own (BOXCONV_INST_PART 3): some hundred
+// kernels that would otherwise double the compile time of the unit with the other variant.
+template <class TG>
+hipError_t grad_output_stream_consec_launch(const SampleArgs<float>& a, int lanes, int cnt, bool exact,
+                                            dim3 grid, hipStream_t stream);
+#if defined(BOXCONV_INST_PART) && BOXCONV_INST_PART == 3
+template <class TG>
+hipError_t grad_output_stream_consec_launch(const SampleArgs<float>& a, int lanes, int cnt, bool exact,
+                                            dim3 grid, hipStream_t stream) {
+    const size_t lds = 0;                              // the kernel's LDS is statically sized
+#define LAUNCH_GC(NT) \
+    if (lanes == NT) { \
+        if (exact) BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, true, true>), grid, dim3(NT), lds, stream, a); \
+        else       BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, false, true>), grid, dim3(NT), lds, stream, a); \
+    } else { \
+        if (exact) BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, true, false>), grid, dim3(NT), lds, stream, a); \
+        else       BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, false, false>), grid, dim3(NT), lds, stream, a); \
+    }
+    switch (cnt) {
+        case 64: LAUNCH_GC(64) break;
+        case 128: LAUNCH_GC(128) break;
+        case 192: LAUNCH_GC(192) break;
+        case 256: LAUNCH_GC(256) break;
+        case 320: LAUNCH_GC(320) break;
+        case 384: LAUNCH_GC(384) break;
+        case 448: LAUNCH_GC(448) break;
+        default: LAUNCH_GC(512) break;
+    }
+#undef LAUNCH_GC
+    return hipGetLastError();
+}
+#endif
+
 template <class T, class TG>
 hipError_t grad_output_stream_launch(const T* integ, const TG* grad_out, BoxParams<T> prm,
                                      double* acc, int acc_slots, T* column_workspace,
@@ -1531,26 +1565,7 @@ hipError_t grad_output_stream_launch(const T* integ, const TG* grad_out, BoxPara
         const bool covers = d.w <= 2048 && lanes >= 1 &&
                             (exact_fit || (switches().stream_consecutive_partial && lanes * 5 >= cnt * 3));
         if (switches().stream_consecutive && covers && params && scan && acc_slots > 0 && aligned) {
-#define LAUNCH_GC(NT) \
-            if (lanes == NT) { \
-                if (exact) BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, true, true>), grid, dim3(NT), lds, stream, a); \
-                else       BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, false, true>), grid, dim3(NT), lds, stream, a); \
-            } else { \
-                if (exact) BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, true, false>), grid, dim3(NT), lds, stream, a); \
-                else       BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, false, false>), grid, dim3(NT), lds, stream, a); \
-            }
-            switch (cnt) {
-                case 64: LAUNCH_GC(64) break;
-                case 128: LAUNCH_GC(128) break;
-                case 192: LAUNCH_GC(192) break;
-                case 256: LAUNCH_GC(256) break;
-                case 320: LAUNCH_GC(320) break;
-                case 384: LAUNCH_GC(384) break;
-                case 448: LAUNCH_GC(448) break;
-                default: LAUNCH_GC(512) break;
-            }
-#undef LAUNCH_GC
-            return hipGetLastError();
+            return grad_output_stream_consec_launch<TG>(a, lanes, cnt, exact, grid, stream);
         }
     }
 #pragma push_macro("BOXCONV_DISPATCH_WIDE")

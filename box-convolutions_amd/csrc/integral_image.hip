@@ -376,6 +376,8 @@ constexpr unsigned long long kNotPublished = 0x7ff8deadbeef0001ull;
 // would poll a stale line until its wait runs out). Should a publisher ever run on another XCD,
 // its words reach the poller late or never; the bounded wait then ends in the local
 // re-summation: slower, never wrong.
+// Hand-over words per band of a plane: four for every lane of the workgroup, whole waves of 256 columns.
+inline int64_t lookback_row_words(int w) { return static_cast<int64_t>((w + 255) / 256) * 256; }
 constexpr int kPublishScope = __HIP_MEMORY_SCOPE_WORKGROUP;
 constexpr int kCollectScope = __HIP_MEMORY_SCOPE_AGENT;
 
@@ -425,8 +427,12 @@ band_scan_lookback_kernel(const TI* __restrict__ in, float* __restrict__ out, do
     const Rows<const TI, false> irows(src, w, w, h);
     T* dst = out + p * static_cast<int64_t>(h + 1) * W1;
     const Rows<T, FULL> orows(dst, W1, w + 1, h + 1);
+    // [nb-1][4][NT]: word v of lane t at v * NT + t, so that a wave's load or store of one word
+    // per lane covers 512 consecutive bytes (with the four words of a lane side by side every such
+    // instruction touched 16 cache lines for 512 bytes, and the look-back's requests outnumbered
+    // those of the band itself)
     unsigned long long* sums = reinterpret_cast<unsigned long long*>(aux) +
-                               p * static_cast<int64_t>(nb - 1) * w;      // [nb-1][w]
+                               p * static_cast<int64_t>(nb - 1) * (4 * NT) + tid;
     const int in_off = c0 * static_cast<int>(sizeof(TI));
     const int out_off = (c0 + 1) * static_cast<int>(sizeof(T));
 
@@ -461,16 +467,20 @@ band_scan_lookback_kernel(const TI* __restrict__ in, float* __restrict__ out, do
         for (int r = 0; r < RMAX; ++r)
 #pragma unroll
             for (int v = 0; v < 4; ++v) own[v] += static_cast<double>(x[r][v]);
-        unsigned long long* mine = sums + static_cast<int64_t>(band) * w + c0;
+        unsigned long long* mine = sums + static_cast<int64_t>(band) * (4 * NT);
 #pragma unroll
-        for (int v = 0; v < 4; ++v)
-            if (c0 + v < w)
-                __hip_atomic_store(mine + v, static_cast<unsigned long long>(__double_as_longlong(own[v])),
-                                   __ATOMIC_RELAXED, kPublishScope);
+        for (int v = 0; v < 4; ++v)      // (lanes past the row's end publish the zeros they hold)
+            __hip_atomic_store(mine + v * NT, static_cast<unsigned long long>(__double_as_longlong(own[v])),
+                               __ATOMIC_RELAXED, kPublishScope);
     }
 
     // -- column sums of the bands above, four bands per round trip: the first loads of a group
-    // are all in flight together; a band that was not published yet is then waited for on its own
+    // are all in flight together; a band that was not published yet is then waited for on its own.
+    // (Measured no faster: groups of eight bands, and two groups in flight with the next one's
+    // loads issued before the current one is waited for, whose registers also cost the workgroups
+    // of four waves a wave per SIMD. What the hand-over costs is the wait for the bands above to
+    // have read their rows, not the round trips: with the collection left out the kernel takes
+    // 0.77 to 0.85 of its time.)
     double colacc[4] = {0.0, 0.0, 0.0, 0.0};
     constexpr int GROUP = 4;
     for (int b0 = 0; b0 < band; b0 += GROUP) {
@@ -482,11 +492,10 @@ band_scan_lookback_kernel(const TI* __restrict__ in, float* __restrict__ out, do
 #pragma unroll
             for (int v = 0; v < 4; ++v) bits[u][v] = 0ull;
             if (b0 + u < band && spin_limit > 0) {
-                const unsigned long long* theirs = sums + static_cast<int64_t>(b0 + u) * w + c0;
+                const unsigned long long* theirs = sums + static_cast<int64_t>(b0 + u) * (4 * NT);
 #pragma unroll
                 for (int v = 0; v < 4; ++v)
-                    if (c0 + v < w)
-                        bits[u][v] = __hip_atomic_load(theirs + v, __ATOMIC_RELAXED, kCollectScope);
+                    bits[u][v] = __hip_atomic_load(theirs + v * NT, __ATOMIC_RELAXED, kCollectScope);
             }
         }
 #pragma unroll
@@ -498,16 +507,15 @@ band_scan_lookback_kernel(const TI* __restrict__ in, float* __restrict__ out, do
 #pragma unroll
                 for (int v = 0; v < 4; ++v) have[u] = have[u] && bits[u][v] != kNotPublished;
             }
-            const unsigned long long* theirs = sums + static_cast<int64_t>(b) * w + c0;
+            const unsigned long long* theirs = sums + static_cast<int64_t>(b) * (4 * NT);
             for (int it = 1; it < spin_limit && !have[u]; ++it) {
                 __builtin_amdgcn_s_sleep(8);
                 have[u] = true;
 #pragma unroll
-                for (int v = 0; v < 4; ++v)
-                    if (c0 + v < w) {
-                        bits[u][v] = __hip_atomic_load(theirs + v, __ATOMIC_RELAXED, kCollectScope);
-                        have[u] = have[u] && bits[u][v] != kNotPublished;
-                    }
+                for (int v = 0; v < 4; ++v) {
+                    bits[u][v] = __hip_atomic_load(theirs + v * NT, __ATOMIC_RELAXED, kCollectScope);
+                    have[u] = have[u] && bits[u][v] != kNotPublished;
+                }
             }
             if (have[u]) {
 #pragma unroll
@@ -622,7 +630,7 @@ template <class TI, int WAVES>
 hipError_t launch_lookback(const TI* in, float* out, double* aux, int64_t planes, int h, int w,
                            int nb, int R, bool reverse, bool prepared, hipStream_t stream) {
     if (!prepared) {
-        const int64_t nsums = planes * static_cast<int64_t>(nb - 1) * w;
+        const int64_t nsums = planes * static_cast<int64_t>(nb - 1) * lookback_row_words(w);
         BOXCONV_LAUNCH("fill_marker", fill_marker_kernel, dim3(static_cast<unsigned>((nsums + 255) / 256)),
                        dim3(256), 0, stream, reinterpret_cast<unsigned long long*>(aux), nsums);
         hipError_t e = hipGetLastError();
@@ -727,9 +735,9 @@ IntegralPlan plan_integral(int64_t planes, int h, int w, int64_t want) {
     nb = (h + R - 1) / R;
     pl.nb = nb;
     pl.R = R;
-    pl.aux_doubles = (nb > 1) ? planes * static_cast<int64_t>(nb - 1) * w : 0;
     pl.lookback = single_pass && nb > 1 && nb <= kLookbackBands && R <= kLookbackRows &&
                   planes * nb < (1ll << 31);
+    pl.aux_doubles = (nb > 1) ? planes * static_cast<int64_t>(nb - 1) * (pl.lookback ? lookback_row_words(w) : w) : 0;
     return pl;
 }
 
@@ -740,7 +748,7 @@ hipError_t clip_and_prepare_integral_launch(const ClipArgs<T>& clip, int64_t pla
     const bool fill = single_pass_applies<T>(pl);
     *prepared = fill;
     const int clip_blocks = (clip.n + 255) / 256;
-    const int64_t nsums = fill ? planes * static_cast<int64_t>(pl.nb - 1) * w : 0;
+    const int64_t nsums = fill ? planes * static_cast<int64_t>(pl.nb - 1) * lookback_row_words(w) : 0;
     const int64_t blocks = clip_blocks + (nsums + 255) / 256;
     if (blocks == 0) return hipSuccess;
     BOXCONV_LAUNCH("clip", (clip_and_fill_marker_kernel<T>), dim3(static_cast<unsigned>(blocks)), dim3(256),

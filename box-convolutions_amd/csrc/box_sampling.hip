@@ -33,6 +33,7 @@ Switches read_switches() {
         const char* e = text("BOXCONV_STREAM_CONSEC");
         s.stream_consecutive_partial = e == nullptr || (e[0] != '0' && e[0] != '1');
     }
+    s.stream_narrow_double = flag_unless_zero("BOXCONV_STREAM_F64_NARROW");
     s.interleave_workspace = flag_unless_zero("BOXCONV_M_INTERLEAVE");
     e = text("BOXCONV_STREAM_WGS");
     s.stream_workgroups = e != nullptr ? std::max(1, std::atoi(e)) : 2048;
@@ -102,7 +103,7 @@ hipError_t grad_params_begin(double* acc, int n_boxes, hipStream_t stream) {
 
 StreamPlan plan_grad_output_stream(int64_t planes_f, int h, int w, size_t elem_size) {
     StreamPlan sp{};
-    const RowConfig rc = stream_row_config(std::max(w, 1));
+    const RowConfig rc = stream_row_config(std::max(w, 1), elem_size);
     sp.usable = row_kernels_apply(h, w, elem_size) &&
                 stream_lds_bytes(rc.K, rc.nt, elem_size) <= kMaxDynamicLds;
     int nb = bands_for(std::max<int64_t>(planes_f, 1), h, 32, switches().stream_workgroups);

@@ -281,7 +281,23 @@ inline bool row_kernels_apply(int h, int w, size_t elem_size) {
 // planes written last are the ones most likely still held by the memory-side cache.
 inline bool reverse_grad_input() { return switches().gi_reverse; }
 
-inline RowConfig stream_row_config(int w) {
+// The grad_output pass keeps the most state per column of all row kernels. With 8-byte elements
+// three or four columns per lane need 200 to 580 registers more than a lane has: the kernels ran
+// out of scratch memory, at 8 times the time of their float counterparts instead of twice. Rows of
+// up to 1024 doubles therefore get at most two columns per lane (a lane's state is then what four
+// columns are in floats). Wider rows keep three or four on eight waves: sixteen waves with two
+// columns per lane, the two jobs as two launches, leave a lane 128 registers, spill as well and
+// were measured slower (2048 columns: 1176 against 1092 us).
+inline RowConfig stream_row_config(int w, size_t elem_size) {
+    if (elem_size == 8 && w <= 1024 && switches().stream_narrow_double) {
+        RowConfig c;
+        if (w <= 128)      { c.nt = w <= 64 ? 64 : 128; c.K = 1; }
+        else if (w <= 256) { c.nt = 128; c.K = 2; }
+        else if (w <= 512) { c.nt = 256; c.K = 2; }
+        else               { c.nt = 512; c.K = 2; }
+        c.full = (c.K * c.nt == w);
+        return c;
+    }
     return row_config(w, switches().stream_threads);
 }
 
@@ -325,15 +341,20 @@ void finish_args(SampleArgs<T>& a, int64_t total) {
         else { BOXCONV_DISPATCH_K34(KERNEL, 64, (RC).K, __VA_ARGS__) }               \
     } else if ((RC).nt == 128) {                                                     \
         if ((RC).K == 1) { KERNEL(128, 1, __VA_ARGS__); }                            \
+        else if ((RC).K == 2) { BOXCONV_DISPATCH_K2(KERNEL, 128, __VA_ARGS__) }      \
         else { BOXCONV_DISPATCH_K34(KERNEL, 128, (RC).K, __VA_ARGS__) }              \
     } else if ((RC).nt == 256) {                                                     \
-        BOXCONV_DISPATCH_K34(KERNEL, 256, (RC).K, __VA_ARGS__)                       \
+        if ((RC).K == 2) { BOXCONV_DISPATCH_K2(KERNEL, 256, __VA_ARGS__) }           \
+        else { BOXCONV_DISPATCH_K34(KERNEL, 256, (RC).K, __VA_ARGS__) }              \
     } else if ((RC).nt == 512) {                                                     \
         if ((RC).K == 2) { KERNEL(512, 2, __VA_ARGS__); }                            \
         else { BOXCONV_DISPATCH_K34(KERNEL, 512, (RC).K, __VA_ARGS__) }              \
     } else {                                                                         \
         BOXCONV_DISPATCH_WIDE(KERNEL, (RC).K, __VA_ARGS__)                           \
     }
+// two columns per lane on two or four waves: only the grad_output pass, for 8-byte arithmetic,
+// instantiates these (it redefines the macro around its dispatch)
+#define BOXCONV_DISPATCH_K2(KERNEL, NT, ...) { return hipErrorInvalidValue; }
 // 1024 threads: instantiated for 4-byte arithmetic only (`T` is the launch function's type)
 #define BOXCONV_DISPATCH_WIDE(KERNEL, K, ...)                                        \
     if constexpr (sizeof(T) <= 4) { BOXCONV_DISPATCH_K34(KERNEL, 1024, K, __VA_ARGS__) } \

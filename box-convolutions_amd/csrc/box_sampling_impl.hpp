@@ -1522,7 +1522,7 @@ hipError_t grad_output_stream_launch(const T* integ, const TG* grad_out, BoxPara
     set_workspace_layout(a, d.h, sp.R);
     a.keep_tail = scan ? cached_tail_bytes() / kXcds : 0;
     finish_args(a, planes_f * a.nb);
-    const RowConfig rc = stream_row_config(d.w);
+    const RowConfig rc = stream_row_config(d.w, sizeof(T));
     // The workspace layout was fixed by plan_grad_output_stream for a gfx950 CU's LDS; a device
     // that grants a workgroup less cannot run this kernel (and has no fallback at this point).
     if (stream_lds_bytes(rc.K, rc.nt, sizeof(T)) > device_lds_limit()) return hipErrorInvalidConfiguration;
@@ -1568,15 +1568,30 @@ hipError_t grad_output_stream_launch(const T* integ, const TG* grad_out, BoxPara
             return grad_output_stream_consec_launch<TG>(a, lanes, cnt, exact, grid, stream);
         }
     }
+    // doubles, two columns per lane on four or eight waves: the kernel that does both jobs needs
+    // more registers than a lane has there (512 threads: 50 to 120 of them in scratch memory);
+    // either job alone fits. Measured, 16 x 8 planes of 256 rows: 512 columns 212 -> 186 us,
+    // 1024 columns 468 -> 362 us; on two waves (256 columns) the one kernel is as fast.
+    const bool split_jobs = sizeof(T) == 8 && rc.K == 2 && rc.nt >= 256 && switches().stream_narrow_double;
 #pragma push_macro("BOXCONV_DISPATCH_WIDE")
+#pragma push_macro("BOXCONV_DISPATCH_K2")
 #undef BOXCONV_DISPATCH_WIDE
+#undef BOXCONV_DISPATCH_K2
 #define BOXCONV_DISPATCH_WIDE(KERNEL, K, ...) { return hipErrorInvalidValue; }
+#define BOXCONV_DISPATCH_K2(KERNEL, NT, ...)                                         \
+    if constexpr (sizeof(T) == 8) { KERNEL(NT, 2, __VA_ARGS__); }                    \
+    else { return hipErrorInvalidValue; }
 #define LAUNCH_GS(NT, KK, EX, FU) \
+    if (params && scan && split_jobs) { \
+        BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_kernel<T, TG, NT, KK, EX, FU, true, false>), grid, dim3(NT), lds, stream, a); \
+        BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_kernel<T, TG, NT, KK, EX, FU, false, true>), grid, dim3(NT), lds, stream, a); \
+    } else \
     if (params && scan) BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_kernel<T, TG, NT, KK, EX, FU, true, true>), grid, dim3(NT), lds, stream, a); \
     else if (params)    BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_kernel<T, TG, NT, KK, EX, FU, true, false>), grid, dim3(NT), lds, stream, a); \
     else                BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_kernel<T, TG, NT, KK, EX, FU, false, true>), grid, dim3(NT), lds, stream, a)
     BOXCONV_DISPATCH_SHAPE_EXACT_FULL(LAUNCH_GS, rc, exact)
 #undef LAUNCH_GS
+#pragma pop_macro("BOXCONV_DISPATCH_K2")
 #pragma pop_macro("BOXCONV_DISPATCH_WIDE")
     return hipGetLastError();
 }

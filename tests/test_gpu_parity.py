@@ -369,6 +369,33 @@ def test_grad_output_pass_variants_agree(hip, oracle, switches, h, w, exact):
         assert np.abs(a - b).max() <= 1e-4 * max(np.abs(b).max(), 1e-30) + 1e-5 * max(np.abs(t).max() for t in back_b[1:])
 
 
+@pytest.mark.parametrize("exact", [True, False])
+@pytest.mark.parametrize("h,w", [(37, 130), (40, 256), (34, 300), (70, 512), (21, 700), (36, 1024), (18, 1025)])
+def test_float64_grad_output_pass_shapes_agree(hip, oracle, switches, h, w, exact):
+    """float64 rows of up to 1024 columns run the grad_output pass with at most two columns per
+    lane, and on four or eight waves as two launches (parameter sums, column workspace);
+    BOXCONV_STREAM_F64_NARROW=0 gives them float32's three or four columns per lane and the one
+    launch, which rows of 1025 columns and more keep. Both against the oracle and against each other."""
+    rng = np.random.default_rng(3 * h + w + int(exact))
+    B, C, F = 2, 2, 3
+    x = rng.standard_normal((B, C, h, w))
+    g = rng.standard_normal((B, C * F, h, w)) + 0.25
+    boxes = list(make_boxes(rng, C, F, h, w, "hanging", away_from_integers=0.05))
+    if not exact:
+        boxes[1] = np.maximum(boxes[1], np.ceil(boxes[0]) + 1)
+        boxes[3] = np.maximum(boxes[3], np.ceil(boxes[2]) + 1)
+    boxes = tuple(np.asarray(b, dtype=np.float64) for b in boxes)
+    results = []
+    for variant in (None, "0"):
+        switches("BOXCONV_STREAM_F64_NARROW", variant)
+        cpu, gpu, sc = run_both(hip, oracle, x, boxes, 3.5 * h, 2.25 * w, True, exact, g)
+        assert_parity(cpu, gpu, np.float64, "narrow=%s %dx%d exact=%s" % (variant, h, w, exact), **sc)
+        results.append(gpu)
+    (_, back_a), (_, back_b) = results
+    for a, b in zip(back_a, back_b):
+        assert np.abs(a - b).max() <= 1e-11 * max(np.abs(b).max(), 1e-30) + 1e-12 * max(np.abs(t).max() for t in back_b[1:])
+
+
 @pytest.mark.parametrize("h,w,F", [(64, 20, 3), (64, 40, 5), (96, 200, 3), (128, 256, 2), (256, 512, 3),
                                    (64, 1024, 3), (128, 2500, 2)])
 def test_workspace_layouts_agree(hip, oracle, switches, h, w, F):

@@ -16,7 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_NAME = "libboxconv_hip.so"
 LIB_PATH = os.path.join(_HERE, LIB_NAME)
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _lib = None
 
@@ -50,6 +50,8 @@ for _s in ("f32", "f64"):
 
 _SIGNATURES["boxconv_backward_half_f32"] = (
     _i, [_vp] * 6 + [_i, _f, _f, _i, _i] + [_vp] * 5 + [_i] * 5 + [_vp, _sz, _vp])
+_SIGNATURES["boxconv_training_forward_half_f32"] = (
+    _i, [_vp, _i] + [_vp] * 7 + [_i] * 5 + [_d] * 4 + [_i, _i, _i] + [_vp, _sz, _vp])
 _SIGNATURES["boxconv_integral_image_static_f32"] = (_i, [_vp, _vp, _i64, _i, _i, _vp])
 _SIGNATURES["boxconv_integral_image_int"] = (_i, [_vp, _vp, _i, _i64, _i, _i, _vp])
 _SIGNATURES["boxconv_integral_image_half_f32"] = (_i, [_vp, _i, _vp, _i64, _i, _i, _vp, _sz, _vp])
@@ -116,8 +118,9 @@ def glue():
             module.init(*[ctypes.cast(getattr(lib, name), ctypes.c_void_p).value for name in (
                 "boxconv_training_forward_f32", "boxconv_training_forward_f64",
                 "boxconv_inference_forward_f32", "boxconv_inference_forward_f64", "boxconv_backward_f32",
-                "boxconv_backward_f64", "boxconv_integral_image_workspace_bytes",
-                "boxconv_backward_workspace_bytes", "boxconv_last_error")])
+                "boxconv_backward_f64", "boxconv_training_forward_half_f32", "boxconv_backward_half_f32",
+                "boxconv_integral_image_workspace_bytes", "boxconv_backward_workspace_bytes",
+                "boxconv_last_error")])
             _glue = module
     return _glue or None
 
@@ -248,6 +251,12 @@ _MAX_WIDENING_WIDTH = 2048     # widest row boxconv_integral_image_half_f32 read
 _MAX_STREAM_WIDTH = 4096       # widest row boxconv_backward_half_f32 reads directly
 
 
+def half_rows_read_directly(h, w):
+    """Whether the integral image kernels read float16 / bfloat16 planes of h x w themselves
+    (otherwise the tensor is converted to float32 first)."""
+    return w <= _MAX_WIDENING_WIDTH and (h + 1) * (w + 1) * 4 < 2 ** 31
+
+
 def integral_image(input):
     """``integral_image(Tensor) -> Tensor`` (reference src/integral_image_interface.cpp:8-27).
 
@@ -260,7 +269,7 @@ def integral_image(input):
         return _integral_image_int(input)
     half = input.dtype in (torch.float16, torch.bfloat16)
     h, w = input.shape[-2:]
-    if half and (w > _MAX_WIDENING_WIDTH or (h + 1) * (w + 1) * 4 >= 2 ** 31):
+    if half and not half_rows_read_directly(h, w):
         input, half = input.float(), False
     sfx = "half_f32" if half else _suffix(input, "integral image input")
     lib = load()

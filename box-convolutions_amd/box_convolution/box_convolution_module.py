@@ -220,6 +220,13 @@ class BoxConv2d(torch.nn.Module):
         widened as it is loaded, grad_input rounded once in the store; parameter gradients are
         float32, or the parameters' own half type after ``module.half()``)."""
         params = (self.x_min, self.x_max, self.y_min, self.y_max)
+        h, w = input.shape[-2:]
+        if (input.is_cuda and input.dim() == 4 and self.x_min.is_cuda and self.x_min.dtype == torch.float32
+                and _native.glue() is not None and _native.half_rows_read_directly(h, w)):
+            # the whole call's host side in C++, as for float32 (same native kernels)
+            return _native.training_step(
+                input, *params, self.reparametrization_h, self.reparametrization_w,
+                self.max_input_h, self.max_input_w, self.normalize, self.exact, clip=self.training)
         if torch.is_grad_enabled() and (input.requires_grad or any(p.requires_grad for p in params)):
             clip_to = (self.max_input_h, self.max_input_w) if self.training else None
             return BoxConvolutionFunction.apply(

@@ -255,6 +255,38 @@ int training_forward_impl(const T* input, T* x_min, T* x_max, T* y_min, T* y_max
                       "forward launch");
 }
 
+// The same for a float16 / bfloat16 input and output (TH): float32 bounds, float32 integral image.
+template <class TH>
+int training_forward_half_impl(const TH* input, float* x_min, float* x_max, float* y_min, float* y_max,
+                               float* real, float* integ, TH* output, int batch, int in_planes,
+                               int num_filters, int h, int w, double reparam_h, double reparam_w,
+                               double max_h, double max_w, bool project, int normalize, int exact,
+                               void* workspace, size_t workspace_bytes, void* stream) {
+    const int n = in_planes * num_filters;
+    const int64_t planes = static_cast<int64_t>(batch) * in_planes;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    double* aux = static_cast<double*>(workspace);
+    const boxconv::IntegralPlan plan = boxconv::plan_integral(planes, h, w);
+    bool prepared = false;
+    if (int rc = hip_result(boxconv::clip_and_prepare_integral_launch<float>(
+            boxconv::clip_args<float>(x_min, x_max, y_min, y_max, real, n, reparam_h, reparam_w, max_h,
+                                      max_w, exact != 0, project),
+            planes, w, aux, plan, &prepared, s), "clip launch"))
+        return rc;
+    if (planes == 0) return 0;
+    if (int rc = hip_result(boxconv::integral_image_widening_launch<TH>(input, integ, planes, h, w, aux,
+                                                                        plan, s, prepared),
+                            "integral image launch"))
+        return rc;
+    if (n == 0) return 0;
+    const boxconv::Dims d{in_planes, num_filters, h, w, planes, 0};
+    const boxconv::BoxParams<float> prm{real, real + n, real + 2 * n, real + 3 * n};
+    return hip_result(boxconv::forward_fused_launch<TH>(integ, prm, output, static_cast<const TH*>(nullptr),
+                                                        nullptr, nullptr, false, d, normalize != 0,
+                                                        exact != 0, s),
+                      "forward launch");
+}
+
 template <class TI>
 int integral_image_widening_impl(const TI* in, float* out, int64_t planes, int h, int w,
                                  void* workspace, size_t workspace_bytes, void* stream) {
@@ -570,6 +602,47 @@ int boxconv_training_forward_f64(const double* input, double* x_min, double* x_m
                                          w, reparametrization_h, reparametrization_w, max_input_h,
                                          max_input_w, normalize, exact, workspace, workspace_bytes,
                                          stream);
+}
+
+int boxconv_training_forward_half_f32(const void* input, int io_dtype, float* x_min, float* x_max,
+                                      float* y_min, float* y_max, float* real_parameters,
+                                      float* input_integrated, void* output, int batch, int in_planes,
+                                      int num_filters, int h, int w, double reparametrization_h,
+                                      double reparametrization_w, double max_input_h, double max_input_w,
+                                      int clip, int normalize, int exact, void* workspace,
+                                      size_t workspace_bytes, void* stream) {
+    if (int rc = check_dims(batch, in_planes, num_filters, h, w)) return rc;
+    if (io_dtype != BOXCONV_F16 && io_dtype != BOXCONV_BF16)
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "half training forward: io_dtype %d is neither BOXCONV_F16 nor BOXCONV_BF16",
+                    io_dtype);
+    const int n = in_planes * num_filters;
+    if (n > 0 && (!x_min || !x_max || !y_min || !y_max || !real_parameters))
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "half training forward: null parameter pointer");
+    if (!(reparametrization_h > 0) || !(reparametrization_w > 0))
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "half training forward: reparametrization factors must be positive");
+    const int64_t planes = static_cast<int64_t>(batch) * in_planes;
+    if (planes > 0 && (!input || !input_integrated || (n > 0 && !output)))
+        return fail(BOXCONV_E_INVALID_ARGUMENT, "half training forward: null tensor pointer");
+    if (!boxconv::integral_image_widening_applies(h, w))
+        return fail(BOXCONV_E_TOO_LARGE, "half training forward: half-precision input is read directly for rows "
+                    "of at most %d columns and planes below 2 GiB; convert wider inputs to float first",
+                    boxconv::kMaxWideningWidth);
+    const size_t need = boxconv_integral_image_workspace_bytes(planes, h, w);
+    if (need > 0 && (workspace == nullptr || workspace_bytes < need ||
+                     reinterpret_cast<uintptr_t>(workspace) % 8 != 0))
+        return fail(BOXCONV_E_WORKSPACE, "half training forward: workspace of %zu bytes (8-byte aligned) required, got %zu",
+                    need, workspace_bytes);
+    if (io_dtype == BOXCONV_F16)
+        return training_forward_half_impl(static_cast<const boxconv::f16_t*>(input), x_min, x_max, y_min, y_max,
+                                          real_parameters, input_integrated, static_cast<boxconv::f16_t*>(output),
+                                          batch, in_planes, num_filters, h, w, reparametrization_h,
+                                          reparametrization_w, max_input_h, max_input_w, clip != 0, normalize,
+                                          exact, workspace, workspace_bytes, stream);
+    return training_forward_half_impl(static_cast<const boxconv::bf16_t*>(input), x_min, x_max, y_min, y_max,
+                                      real_parameters, input_integrated, static_cast<boxconv::bf16_t*>(output),
+                                      batch, in_planes, num_filters, h, w, reparametrization_h,
+                                      reparametrization_w, max_input_h, max_input_w, clip != 0, normalize,
+                                      exact, workspace, workspace_bytes, stream);
 }
 
 int boxconv_inference_forward_f32(const float* input, const float* x_min, const float* x_max,

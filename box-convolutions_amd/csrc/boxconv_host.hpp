@@ -52,7 +52,8 @@ struct f16_t;
 struct bf16_t;
 template <class TI>
 hipError_t integral_image_widening_launch(const TI* in, float* out, int64_t planes, int h, int w,
-                                          double* aux, const IntegralPlan& plan, hipStream_t stream);
+                                          double* aux, const IntegralPlan& plan, hipStream_t stream,
+                                          bool workspace_prepared = false);
 bool integral_image_widening_applies(int h, int w);
 
 // Integral image of an integer tensor (dtype: BOXCONV_U8 .. BOXCONV_I64 of include/boxconv.h),

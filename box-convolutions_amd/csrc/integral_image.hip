@@ -827,8 +827,9 @@ hipError_t integral_image_launch(const T* in, T* out, int64_t planes, int h, int
 
 template <class TI>
 hipError_t integral_image_widening_launch(const TI* in, float* out, int64_t planes, int h, int w,
-                                          double* aux, const IntegralPlan& pl, hipStream_t stream) {
-    return integral_image_any<float, TI>(in, out, planes, h, w, aux, pl, false, false, stream);
+                                          double* aux, const IntegralPlan& pl, hipStream_t stream,
+                                          bool workspace_prepared) {
+    return integral_image_any<float, TI>(in, out, planes, h, w, aux, pl, workspace_prepared, false, stream);
 }
 
 bool integral_image_widening_applies(int h, int w) {
@@ -836,9 +837,9 @@ bool integral_image_widening_applies(int h, int w) {
 }
 
 template hipError_t integral_image_widening_launch<f16_t>(const f16_t*, float*, int64_t, int, int,
-                                                          double*, const IntegralPlan&, hipStream_t);
+                                                          double*, const IntegralPlan&, hipStream_t, bool);
 template hipError_t integral_image_widening_launch<bf16_t>(const bf16_t*, float*, int64_t, int, int,
-                                                           double*, const IntegralPlan&, hipStream_t);
+                                                           double*, const IntegralPlan&, hipStream_t, bool);
 template hipError_t integral_image_launch<float>(const float*, float*, int64_t, int, int,
                                                  double*, const IntegralPlan&, bool, bool, hipStream_t);
 template hipError_t integral_image_launch<double>(const double*, double*, int64_t, int, int,

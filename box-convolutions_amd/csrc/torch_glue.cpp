@@ -4,8 +4,9 @@
 //   box_convolution/box_convolution_function.py (BoxConvolutionFunction.forward / .backward, the
 //   counterpart of the reference's box_convolution/box_convolution_function.py:30-65) and the
 //   tensor-level checks and allocations of box_convolution/_native.py,
-// for the common case only: float32 or float64, everything on one GPU; training mode (parameters
-// clipped on the way in) and eval mode (parameters only read). On the layer shapes of the reference's model zoo the kernels of
+// for the common case only: float32 or float64, or float16 / bfloat16 tensors with float32
+// parameters, everything on one GPU; training mode (parameters clipped on the way in) and eval
+// mode (parameters only read). On the layer shapes of the reference's model zoo the kernels of
 // a step take under 100 us, and the Python versions of this glue cost more than that per step
 // (argument checks, seven tensor allocations, two ctypes calls with 22 and 24 arguments, and the
 // autograd engine calling back into Python from its own thread). Here the engine calls straight
@@ -34,6 +35,12 @@ using BackwardFn = int (*)(const T*, const T*, const T*, const T*, const T*, con
 template <class T>
 using InferenceForwardFn = int (*)(const T*, const T*, const T*, const T*, const T*, T*, T*, T*, int, int, int, int,
                                    int, double, double, int, int, void*, size_t, void*);
+using TrainingForwardHalfFn = int (*)(const void*, int, float*, float*, float*, float*, float*, float*, void*, int,
+                                      int, int, int, int, double, double, double, double, int, int, int, void*,
+                                      size_t, void*);
+using BackwardHalfFn = int (*)(const float*, const float*, const float*, const float*, const float*, const void*,
+                               int, float, float, int, int, void*, float*, float*, float*, float*, int, int, int,
+                               int, int, void*, size_t, void*);
 using IntegralWorkspaceFn = size_t (*)(int64_t, int, int);
 using BackwardWorkspaceFn = size_t (*)(int, int, int, int, int, int, int, int);
 using LastErrorFn = const char* (*)();
@@ -45,6 +52,8 @@ struct Abi {
     void* inference_forward_f64 = nullptr;
     void* backward_f32 = nullptr;
     void* backward_f64 = nullptr;
+    TrainingForwardHalfFn training_forward_half = nullptr;
+    BackwardHalfFn backward_half = nullptr;
     IntegralWorkspaceFn integral_workspace_bytes = nullptr;
     BackwardWorkspaceFn backward_workspace_bytes = nullptr;
     LastErrorFn last_error = nullptr;
@@ -97,6 +106,9 @@ at::Tensor workspace(size_t nbytes, const at::Device& device, uint64_t stream, b
 
 void* ptr_or_null(const at::Tensor& t) { return t.defined() ? t.data_ptr() : nullptr; }
 
+bool is_half(at::ScalarType t) { return t == at::kHalf || t == at::kBFloat16; }
+int half_code(at::ScalarType t) { return t == at::kHalf ? 1 : 2; }     // BOXCONV_F16, BOXCONV_BF16
+
 // ---- the autograd node -----------------------------------------------------------------------------
 struct TrainingStep : public torch::autograd::Function<TrainingStep> {
     // Returns the output [B, C*F, h, w]. x_min .. y_max are the stored parameters, clipped in place
@@ -108,12 +120,24 @@ struct TrainingStep : public torch::autograd::Function<TrainingStep> {
                               bool capturing) {
         const at::Tensor in = input.contiguous();
         const int64_t B = in.size(0), C = in.size(1), h = in.size(2), w = in.size(3), F = x_min.size(1);
-        const auto opts = in.options();
+        const bool half = is_half(in.scalar_type());
+        // (half tensors: float32 integral image and bounds; the kernels read and write the half type)
+        const auto opts = half ? in.options().dtype(at::kFloat) : in.options();
         at::Tensor integrated = at::empty({B, C, h + 1, w + 1}, opts);
-        at::Tensor output = at::empty({B, C * F, h, w}, opts);
+        at::Tensor output = at::empty({B, C * F, h, w}, in.options());
         at::Tensor real = at::empty({4, C, F}, opts);
         const size_t nbytes = g_abi.integral_workspace_bytes(B * C, static_cast<int>(h), static_cast<int>(w));
         at::Tensor ws = workspace(nbytes, in.device(), static_cast<uint64_t>(stream), capturing);
+        if (half)
+            check_rc(g_abi.training_forward_half(
+                         in.data_ptr(), half_code(in.scalar_type()), x_min.data_ptr<float>(),
+                         x_max.data_ptr<float>(), y_min.data_ptr<float>(), y_max.data_ptr<float>(),
+                         real.data_ptr<float>(), integrated.data_ptr<float>(), output.data_ptr(),
+                         static_cast<int>(B), static_cast<int>(C), static_cast<int>(F), static_cast<int>(h),
+                         static_cast<int>(w), reparam_h, reparam_w, max_h, max_w, clip ? 1 : 0, normalize ? 1 : 0,
+                         exact ? 1 : 0, ptr_or_null(ws), nbytes, reinterpret_cast<void*>(stream)),
+                     "training_forward_half");
+        else
         AT_DISPATCH_FLOATING_TYPES(in.scalar_type(), "boxconv_module_forward", [&] {
             if (clip)
                 check_rc(training_forward_fn<scalar_t>()(
@@ -158,7 +182,10 @@ struct TrainingStep : public torch::autograd::Function<TrainingStep> {
         TORCH_CHECK(grad_output.size(0) == B && grad_output.size(1) == C * F && grad_output.size(2) == h &&
                         grad_output.size(3) == w,
                     "box_convolution: sizes of grad_output and input_integrated don't match");
-        TORCH_CHECK(grad_output.device() == integrated.device() && grad_output.scalar_type() == integrated.scalar_type(),
+        const bool half = is_half(grad_output.scalar_type());
+        TORCH_CHECK(grad_output.device() == integrated.device() &&
+                        (grad_output.scalar_type() == integrated.scalar_type() ||
+                         (half && integrated.scalar_type() == at::kFloat)),
                     "box_convolution: grad_output and input_integrated differ in device or dtype");
         const bool need_input = ctx->needs_input_grad(0);
         bool need[4];
@@ -166,7 +193,8 @@ struct TrainingStep : public torch::autograd::Function<TrainingStep> {
         for (int k = 0; k < 4; ++k) { need[k] = ctx->needs_input_grad(1 + k); any_param = any_param || need[k]; }
         const auto opts = integrated.options();
         at::Tensor grad_input;
-        if (need_input) grad_input = F > 0 ? at::empty({B, C, h, w}, opts) : at::zeros({B, C, h, w}, opts);
+        const auto io_opts = grad_output.options();         // (the input's own type)
+        if (need_input) grad_input = F > 0 ? at::empty({B, C, h, w}, io_opts) : at::zeros({B, C, h, w}, io_opts);
         at::Tensor grad_params;                               // one allocation for the four
         if (any_param) grad_params = at::empty({4, C, F}, opts);
         const bool want_input = need_input && grad_input.numel() > 0 && F > 0;
@@ -184,6 +212,18 @@ struct TrainingStep : public torch::autograd::Function<TrainingStep> {
             const int normalize = ctx->saved_data["normalize"].toBool() ? 1 : 0;
             const int exact = ctx->saved_data["exact"].toBool() ? 1 : 0;
             const int64_t n = C * F;
+            if (half) {
+                const float* r = real.data_ptr<float>();
+                float* gp = want_params ? grad_params.data_ptr<float>() : nullptr;
+                check_rc(g_abi.backward_half(
+                             integrated.data_ptr<float>(), r, r + n, r + 2 * n, r + 3 * n, grad_output.data_ptr(),
+                             half_code(grad_output.scalar_type()), reparam_h, reparam_w, normalize, exact,
+                             want_input ? grad_input.data_ptr() : nullptr, gp, gp ? gp + n : nullptr,
+                             gp ? gp + 2 * n : nullptr, gp ? gp + 3 * n : nullptr, static_cast<int>(B),
+                             static_cast<int>(C), static_cast<int>(F), static_cast<int>(h), static_cast<int>(w),
+                             ptr_or_null(ws), nbytes, reinterpret_cast<void*>(stream)),
+                         "box_convolution_backward_half");
+            } else
             AT_DISPATCH_FLOATING_TYPES(integrated.scalar_type(), "boxconv_backward", [&] {
                 const scalar_t* r = real.data_ptr<scalar_t>();
                 scalar_t* gp = want_params ? grad_params.data_ptr<scalar_t>() : nullptr;
@@ -218,12 +258,14 @@ at::Tensor training_step(const at::Tensor& input, const at::Tensor& x_min, const
     TORCH_CHECK(input.is_cuda(), "box_convolution: input is on '", input.device(),
                 "'; this build runs on AMD GPUs only (no CPU path)");
     TORCH_CHECK(input.dim() == 4, "BoxConv2d: input must have 4 dimensions");
-    TORCH_CHECK(input.scalar_type() == at::kFloat || input.scalar_type() == at::kDouble,
-                "box_convolution: input must be float32 or float64, got ", input.scalar_type());
+    const bool half = is_half(input.scalar_type());
+    TORCH_CHECK(input.scalar_type() == at::kFloat || input.scalar_type() == at::kDouble || half,
+                "box_convolution: input must be float32, float64, float16 or bfloat16, got ", input.scalar_type());
+    const at::ScalarType param_type = half ? at::kFloat : input.scalar_type();
     const at::Tensor* params[4] = {&x_min, &x_max, &y_min, &y_max};
     for (const at::Tensor* p : params) {
         TORCH_CHECK(p->device() == input.device(), "BoxConv2d: input and parameters are on different devices");
-        TORCH_CHECK(p->scalar_type() == input.scalar_type(), "box_convolution: input and parameters have different dtypes (",
+        TORCH_CHECK(p->scalar_type() == param_type, "box_convolution: input and parameters have different dtypes (",
                     input.scalar_type(), ", ", p->scalar_type(), ")");
         TORCH_CHECK(!clip || p->is_contiguous(), "box_convolution: parameters must be contiguous to be clipped in place");
         TORCH_CHECK(p->dim() == 2, "BoxConv2d: all parameters must have 2 dimensions");
@@ -243,14 +285,17 @@ at::Tensor training_step(const at::Tensor& input, const at::Tensor& x_min, const
 }
 
 void init(uint64_t training_forward_f32, uint64_t training_forward_f64, uint64_t inference_forward_f32,
-          uint64_t inference_forward_f64, uint64_t backward_f32, uint64_t backward_f64, uint64_t integral_workspace_bytes, uint64_t backward_workspace_bytes,
-          uint64_t last_error) {
+          uint64_t inference_forward_f64, uint64_t backward_f32, uint64_t backward_f64,
+          uint64_t training_forward_half, uint64_t backward_half, uint64_t integral_workspace_bytes,
+          uint64_t backward_workspace_bytes, uint64_t last_error) {
     g_abi.training_forward_f32 = reinterpret_cast<void*>(training_forward_f32);
     g_abi.training_forward_f64 = reinterpret_cast<void*>(training_forward_f64);
     g_abi.inference_forward_f32 = reinterpret_cast<void*>(inference_forward_f32);
     g_abi.inference_forward_f64 = reinterpret_cast<void*>(inference_forward_f64);
     g_abi.backward_f32 = reinterpret_cast<void*>(backward_f32);
     g_abi.backward_f64 = reinterpret_cast<void*>(backward_f64);
+    g_abi.training_forward_half = reinterpret_cast<TrainingForwardHalfFn>(training_forward_half);
+    g_abi.backward_half = reinterpret_cast<BackwardHalfFn>(backward_half);
     g_abi.integral_workspace_bytes = reinterpret_cast<IntegralWorkspaceFn>(integral_workspace_bytes);
     g_abi.backward_workspace_bytes = reinterpret_cast<BackwardWorkspaceFn>(backward_workspace_bytes);
     g_abi.last_error = reinterpret_cast<LastErrorFn>(last_error);

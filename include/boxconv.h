@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define BOXCONV_ABI_VERSION 3
+#define BOXCONV_ABI_VERSION 4
 
 #define BOXCONV_E_INVALID_ARGUMENT (-1) /* null pointer, non-positive size, ... */
 #define BOXCONV_E_WORKSPACE        (-2) /* workspace missing or smaller than *_workspace_bytes() */
@@ -202,6 +202,24 @@ int boxconv_inference_forward_f64(const double* input, const double* x_min, cons
                                   int num_filters, int h, int w, double reparametrization_h,
                                   double reparametrization_w, int normalize, int exact, void* workspace,
                                   size_t workspace_bytes, void* stream);
+
+/* ---- training- and eval-mode forward in one call, half-precision tensors -------------------------
+ * The two entry points above for a float16 / bfloat16 input and output (io_dtype: BOXCONV_F16 or
+ * BOXCONV_BF16, both tensors of that type) with float32 parameters: what the reference's
+ * `BoxConv2d.forward` (box_convolution/box_convolution_module.py:208-214) does with a half tensor
+ * on its CUDA path, except that the integral image (input_integrated, float32 out, what
+ * boxconv_backward_half_f32 takes) and all sums are float32 / double, as in
+ * boxconv_integral_image_half_f32 and boxconv_forward_fused_f32, whose results this call returns
+ * bit for bit. clip != 0: training mode (the stored parameters are projected in place first, limits
+ * max_input_h / max_input_w); clip == 0: eval mode (the stored parameters are only read).
+ * Rows of at most 2048 columns (BOXCONV_E_TOO_LARGE otherwise: convert to float first). */
+int boxconv_training_forward_half_f32(const void* input, int io_dtype, float* x_min, float* x_max,
+                                      float* y_min, float* y_max, float* real_parameters,
+                                      float* input_integrated, void* output, int batch, int in_planes,
+                                      int num_filters, int h, int w, double reparametrization_h,
+                                      double reparametrization_w, double max_input_h, double max_input_w,
+                                      int clip, int normalize, int exact, void* workspace,
+                                      size_t workspace_bytes, void* stream);
 
 /* ---- forward, half-precision output and fused tail (inference) ------------------------------
  * The same box sums as boxconv_forward_f32 (reference src/box_convolution_interface.cpp:13-139),

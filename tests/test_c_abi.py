@@ -91,6 +91,19 @@ def test_argument_errors_are_reported_without_launching(lib):
                                           dummy16, 1, 1, 1, 4, 4, f64(0.0), f64(8.0), f64(4.0), f64(4.0),
                                           1, 1, null, 0, null)
     assert rc == -1 and b"positive" in lib.boxconv_last_error()
+    half_args = (dummy16,) * 7
+    rc = lib.boxconv_training_forward_half_f32(dummy16, 0, *half_args, 1, 1, 1, 4, 4, f64(8.0), f64(8.0), f64(4.0),
+                                               f64(4.0), 1, 1, 1, null, 0, null)
+    assert rc == -1 and b"io_dtype" in lib.boxconv_last_error()
+    rc = lib.boxconv_training_forward_half_f32(null, 1, *((null,) * 7), 1, 1, 1, 4, 4, f64(8.0), f64(8.0), f64(4.0),
+                                               f64(4.0), 1, 1, 1, null, 0, null)
+    assert rc == -1 and b"null parameter pointer" in lib.boxconv_last_error()
+    rc = lib.boxconv_training_forward_half_f32(dummy16, 2, *half_args, 1, 1, 1, 4, 4096, f64(8.0), f64(8.0), f64(4.0),
+                                               f64(4.0), 0, 1, 1, null, 0, null)
+    assert rc == -3 and b"2048" in lib.boxconv_last_error()
+    rc = lib.boxconv_training_forward_half_f32(dummy16, 1, *half_args, 2, 16, 8, 512, 1024, f64(8.0), f64(8.0),
+                                               f64(512.0), f64(1024.0), 1, 1, 1, null, 0, null)
+    assert rc == -2 and b"workspace" in lib.boxconv_last_error()
     # several bands and no workspace: refused before anything is launched
     rc = lib.boxconv_training_forward_f32(dummy16, dummy16, dummy16, dummy16, dummy16, dummy16, dummy16,
                                           dummy16, 2, 16, 8, 512, 1024, f64(8.0), f64(8.0), f64(512.0),

@@ -133,6 +133,63 @@ def test_training_step_on_half_precision_input(oracle, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("training", [True, False])
+@pytest.mark.parametrize("shape,needs", [((2, 3, 4, 40, 130), (True, True, True, True, True)),
+                                         ((1, 2, 3, 64, 1024), (True, False, True, False, True)),
+                                         ((2, 2, 2, 33, 2048), (False, True, True, True, True)),
+                                         ((3, 1, 5, 70, 77), (True, False, False, False, False))])
+def test_half_precision_step_through_the_cpp_node(dtype, training, shape, needs):
+    """A float16 / bfloat16 input with float32 parameters goes through the C++ autograd node like
+    a float32 one (one native call for clip, integral image and sampling, one for the backward);
+    BoxConvolutionFunction is the same step in Python with the same kernels. Output, clipped
+    parameters and every requested gradient agree bit for bit; under no_grad there is no graph."""
+    from box_convolution import _native
+    from box_convolution.box_convolution_function import BoxConvolutionFunction
+    if _native.glue() is None:
+        pytest.skip("the C++ glue was not built")
+    B, C, F, h, w = shape
+    modules = [make_module(C, F, h, w, 21) for _ in range(2)]
+    modules[1].load_state_dict(modules[0].state_dict())
+    torch.manual_seed(h + w)
+    x0 = torch.randn(B, C, h, w, device=DEV).to(dtype)
+    g = torch.randn(B, C * F, h, w, device=DEV).to(dtype)
+    names = ("x_min", "x_max", "y_min", "y_max")
+    results = []
+    for which, m in enumerate(modules):
+        with torch.no_grad():
+            m.x_min.mul_(2.0)          # some boxes out of bounds: the clip has work to do (training mode only)
+        for name, need in zip(names, needs[1:]):
+            getattr(m, name).requires_grad_(need)
+        x = x0.clone().requires_grad_(needs[0])
+        m.train(training)
+        if which == 0:
+            out = m(x)                                                      # C++ node
+            assert type(out.grad_fn).__name__ != "BoxConvolutionFunctionBackward"
+        else:
+            out = BoxConvolutionFunction.apply(
+                x, m.x_min, m.x_max, m.y_min, m.y_max, m.reparametrization_h, m.reparametrization_w,
+                m.normalize, m.exact, (m.max_input_h, m.max_input_w) if training else None)
+        assert out.dtype == dtype
+        out.backward(g)
+        results.append((out.detach(), x.grad, [getattr(m, n).grad for n in names],
+                        [getattr(m, n).detach().clone() for n in names]))
+    (out_a, gx_a, gp_a, p_a), (out_b, gx_b, gp_b, p_b) = results
+    assert torch.equal(out_a, out_b)
+    assert (gx_a is None) == (not needs[0])
+    if needs[0]:
+        assert gx_a.dtype == dtype and torch.equal(gx_a, gx_b)
+    for a, b, need in zip(gp_a, gp_b, needs[1:]):
+        assert (a is None) == (not need) and (b is None) == (not need)
+        if need:
+            assert a.dtype == torch.float32 and torch.equal(a, b)
+    for a, b in zip(p_a, p_b):
+        assert torch.equal(a, b)
+    with torch.no_grad():
+        quiet = modules[0](x0)
+    assert quiet.grad_fn is None and torch.equal(quiet, out_a)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_module_converted_to_half_precision(dtype):
     """module.half() / .bfloat16(): the four bounds are stored in the half type; they are clipped
     through a float32 copy, used in float32, and receive gradients of their own type."""

@@ -130,8 +130,13 @@ __global__ void __launch_bounds__(NT) forward_rows_kernel(SampleArgs<T> a, Forwa
                 TO z0, z1;
                 narrow(y0, z0);
                 narrow(y1, z1);
-                store_slot<TO, NT, kCacheStream>(z0, ob0, qo, k);
-                store_slot<TO, NT, kCacheStream>(z1, ob1, qo, k);
+                if (a.stream_out) {                      // (workgroup-uniform)
+                    store_slot<TO, NT, kCacheStream>(z0, ob0, qo, k);
+                    store_slot<TO, NT, kCacheStream>(z1, ob1, qo, k);
+                } else {
+                    store_slot<TO, NT, kCacheDefault>(z0, ob0, qo, k);
+                    store_slot<TO, NT, kCacheDefault>(z1, ob1, qo, k);
+                }
             }
         }
         if (PREFETCH) {
@@ -217,6 +222,16 @@ hipError_t forward_launch_any(const T* integ, BoxParams<T> prm, ForwardTail<TO> 
     // side their rows (a box height apart at most) are fetched together (1024 x 2048 with two
     // filters: 737 -> 703 us). Planes that fit are faster in filter order (512 x 1024: 97 vs 100 us).
     a.band_major = (static_cast<uint64_t>(d.h + 1) * (d.w + 1) * sizeof(T) > (4u << 20)) ? 1 : 0;
+    // The output is written once and not read again by this pass: non-temporal stores keep it out
+    // of the way of the integral rows in the caches (512 x 1024, 16 x 8 planes: 97 against 130 us,
+    // and the grad-input pass that follows 121 against 132). A lane stores one element per
+    // instruction, though, and where rows do not start on 64-byte boundaries such stores reach
+    // memory as partly covered 32-byte sectors that nothing merges any more: 256 x 132, 16 x 64
+    // planes, 61 against 37 us; 256 x 300 51 against 38. Such rows keep the ordinary policy while
+    // the output fits the memory-side cache; beyond that the streaming policy wins even so
+    // (500 x 1000, 512 MB: 128 against 142 us, and the next pass 122 against 138).
+    const uint64_t out_bytes = static_cast<uint64_t>(planes_f) * d.hw() * sizeof(TO);
+    a.stream_out = ((static_cast<uint64_t>(d.w) * sizeof(TO)) % 64 == 0 || out_bytes > (256ull << 20)) ? 1 : 0;
     const dim3 grid(static_cast<unsigned>(a.per_xcd * kXcds));
     const size_t lds = 4 * static_cast<size_t>(d.w + 3) * sizeof(T);
 #define LAUNCH_FWD(NT, KK, EX, FU) \

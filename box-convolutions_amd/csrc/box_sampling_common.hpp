@@ -37,6 +37,7 @@ struct SampleArgs {
     int64_t mpitch;       // elements between rows of M (a multiple of 4)
     int vec_out;          // grad input only: rows of dst are 16-byte aligned
     int band_major;       // forward only: work items ordered (plane, band, filter) instead of (plane, filter, band)
+    int stream_out;       // forward only: the output is stored with the non-temporal policy
     int C, F, h, w;
     int nb, R;            // bands per plane and rows per band
     int64_t plane0;       // global index of the first plane (selects the boxes)

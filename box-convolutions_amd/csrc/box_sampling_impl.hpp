@@ -1556,14 +1556,19 @@ hipError_t grad_output_stream_launch(const T* integ, const TG* grad_out, BoxPara
     // sums: the kernel with four consecutive columns per lane
     if constexpr (std::is_same<T, float>::value) {
         const bool aligned = reinterpret_cast<uintptr_t>(grad_out) % (4 * sizeof(TG)) == 0 && d.w % 4 == 0;
-        // the smallest workgroup (whole waves) whose lanes, four columns each, cover the row. Rows
-        // that would leave more than two fifths of its lanes idle stay with the other kernel
-        // (measured, 16 x 8 planes: 1920 columns 649 -> 490 us, 960: 261 -> 230, 480: 165 -> 137).
+        // the smallest workgroup (whole waves) whose lanes, four columns each, cover the row. Only
+        // a single wave can be left mostly idle (from two waves on, more than half of the lanes
+        // are busy): rows that fill less than three eighths of it stay with the other kernel
+        // (measured, 16 x 4 planes of 256 rows: 100 columns 97 -> 86 us, 128: 91 -> 91, 144:
+        // 110 -> 90, 260: 138 -> 118, 300: 142 -> 121; but 64 columns 72 -> 83). Rows of exactly
+        // 128 columns also stay there: they fill that kernel's two waves at one column per lane
+        // with no bounds to check (10 to 38 x 64 planes of 64 to 256 rows: 70 against 80 us).
         const int lanes = d.w / 4;
         const int cnt = (lanes + 63) / 64 * 64;
         const bool exact_fit = lanes == cnt && (cnt == 64 || cnt == 128 || cnt == 256 || cnt == 512);
         const bool covers = d.w <= 2048 && lanes >= 1 &&
-                            (exact_fit || (switches().stream_consecutive_partial && lanes * 5 >= cnt * 3));
+                            (exact_fit || (switches().stream_consecutive_partial && lanes * 8 >= cnt * 3 &&
+                                           !(rc.full && rc.K == 1)));
         if (switches().stream_consecutive && covers && params && scan && acc_slots > 0 && aligned) {
             return grad_output_stream_consec_launch<TG>(a, lanes, cnt, exact, grid, stream);
         }

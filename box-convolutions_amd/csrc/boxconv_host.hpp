@@ -1,5 +1,6 @@
 // Host-side declarations shared by the translation units of libboxconv_hip.so.
 #pragma once
+#include <cstdlib>
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>

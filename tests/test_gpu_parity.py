@@ -341,9 +341,9 @@ def test_grad_input_filter_sharing_matches_one_set_per_workgroup(hip, switches, 
 @pytest.mark.parametrize("h,w", [(67, 256), (130, 512), (70, 1024), (66, 2048),
                                  # rows that leave lanes of that workgroup idle (whole waves, half a wave, one lane)
                                  (36, 240), (30, 640), (40, 960), (64, 1000), (18, 1280), (22, 1800), (34, 1920),
-                                 (20, 2044), (50, 160), (33, 44)])
+                                 (20, 2044), (50, 160), (33, 44), (36, 100), (40, 96), (34, 92), (30, 272), (31, 132)])
 def test_grad_output_pass_variants_agree(hip, oracle, switches, h, w, exact):
-    """Rows of a multiple of four columns that fill at least three fifths of a workgroup at four
+    """Rows of a multiple of four columns that fill at least three eighths of a workgroup at four
     columns per lane run the grad_output pass with consecutive columns per lane (the lanes past
     the row's end idle along); BOXCONV_STREAM_CONSEC=0 sends them to the kernel with wave-strided
     columns, as every other width. Both against the oracle, and against each other to the last

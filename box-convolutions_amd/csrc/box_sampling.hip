@@ -28,6 +28,7 @@ Switches read_switches() {
     e = text("BOXCONV_INTEGRAL_LOOKBACK");
     s.lookback = e == nullptr || std::atoi(e) != 0;
     s.lookback_any_shape = e != nullptr && std::atoi(e) == 2;
+    s.plane_integral = flag_unless_zero("BOXCONV_INTEGRAL_PLANE");
     s.stream_consecutive = flag_unless_zero("BOXCONV_STREAM_CONSEC");
     {
         const char* e = text("BOXCONV_STREAM_CONSEC");

@@ -33,6 +33,7 @@ struct IntegralPlan {
     int R;                 // rows per band
     int64_t aux_doubles;   // scratch for the column sums of all bands but the last
     bool lookback;         // geometry fits the single-pass kernel (bands of <= 32 rows, one tile wide)
+    bool plane_per_workgroup;  // planes of at most 192 rows and 256 columns: one workgroup scans a whole plane (float output)
 };
 // `want`: number of workgroups to aim for.
 IntegralPlan plan_integral(int64_t planes, int h, int w, int64_t want = 1024);
@@ -187,6 +188,7 @@ struct Switches {
     bool gi_split_filters;    // BOXCONV_GI_SPLIT_FILTERS=0 clears it: no filter sharing in small grad-input launches
     bool lookback;            // BOXCONV_INTEGRAL_LOOKBACK=0 clears it: no single-pass integral image
     bool lookback_any_shape;  // BOXCONV_INTEGRAL_LOOKBACK=2: single pass for every shape it covers
+    bool plane_integral;      // BOXCONV_INTEGRAL_PLANE=0 clears it: no plane-per-workgroup integral image
     bool stream_consecutive;  // BOXCONV_STREAM_CONSEC=0 clears it: no consecutive-column variant of the grad_output pass at all
     bool stream_consecutive_partial;  // BOXCONV_STREAM_CONSEC=1 clears it: that variant only for rows that fill its workgroup exactly
     bool stream_narrow_double;  // BOXCONV_STREAM_F64_NARROW=0 clears it: float64 rows of up to 1024 columns with three or four columns per lane like float32

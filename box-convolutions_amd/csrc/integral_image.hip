@@ -15,7 +15,9 @@
 // columns use band_scan_rows_kernel for launch 3, which adds up the bands above itself (no launch
 // 2). For float rows that fill a workgroup exactly and planes of at most 16 bands of 32 rows, one
 // kernel does everything in a single pass over the input (band_scan_lookback_kernel): workgroups
-// hand their column sums to the ones below them, with a bounded wait.
+// hand their column sums to the ones below them, with a bounded wait. Planes of at most 192 rows
+// and 256 columns take plane_scan_kernel: the bands of a plane are the waves of one workgroup,
+// which hand their sums over through LDS.
 //
 // Arithmetic. All sums are carried in double and rounded once on store, so every stored value
 // is the correctly rounded exact sum (the CPU reference carries row sums in double as well but
@@ -575,6 +577,107 @@ band_scan_lookback_kernel(const TI* __restrict__ in, float* __restrict__ out, do
     }
 }
 
+// ---- single pass, a whole plane per workgroup ---------------------------------------------------
+// Planes of at most 256 columns and 192 rows: wave b of the workgroup owns band b of the plane at
+// full width (a row is one wave, four columns per lane), so the bands of a plane meet in one
+// workgroup and hand their column sums over through LDS with one barrier: one launch, the input
+// read once, nothing in global memory besides input and output, no waiting between workgroups.
+// The arithmetic is that of band_scan_lookback_kernel with one wave per row: the band's rows in
+// registers, double column sums added in band order, rows scanned out of the registers.
+constexpr int kPlaneWaves = 8;        // bands per plane at most
+constexpr int kPlaneRows = 24;        // rows per band at most (registers: 4 x 24 floats per lane without spilling)
+constexpr int kPlaneMaxRows = kPlaneWaves * kPlaneRows, kPlaneMaxCols = 256;
+
+template <class TI, int RMAX, bool VEC>
+__global__ void __launch_bounds__(kPlaneWaves * 64)
+plane_scan_kernel(const TI* __restrict__ in, float* __restrict__ out, int h, int w, int R, int64_t planes,
+                  int reverse) {
+    using T = float;
+    constexpr int RB = 4;
+    __shared__ double sums[kPlaneWaves][4][64];
+
+    int64_t p = blockIdx.x;
+    if (reverse) p = planes - 1 - p;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int band = __builtin_amdgcn_readfirstlane(tid >> 6);     // one wave per band
+    const int r0 = band * R;
+    const int r1 = min(h, r0 + R);                                  // (every wave of the launch has rows)
+    const int64_t W1 = static_cast<int64_t>(w) + 1;
+    const int c0 = 4 * lane;
+
+    const TI* src = in + p * static_cast<int64_t>(h) * w;
+    const Rows<const TI, false> irows(src, w, w, h);
+    T* dst = out + p * static_cast<int64_t>(h + 1) * W1;
+    const Rows<T, VEC> orows(dst, W1, w + 1, h + 1);
+    const int in_off = c0 * static_cast<int>(sizeof(TI));
+    const int out_off = (c0 + 1) * static_cast<int>(sizeof(T));
+    const bool lane_in = c0 < w;
+    const unsigned lane_col = lane_in ? static_cast<unsigned>(c0) : 0u;
+
+    // the whole band into registers, all loads in flight together (clamped addresses, values of
+    // rows and lanes that do not exist dropped afterwards)
+    T x[RMAX][4];
+#pragma unroll
+    for (int r = 0; r < RMAX; ++r) {
+        const int row = r0 + r;
+        const bool exists = r < R && row < r1;
+        if (VEC) {
+            load_quad(src + static_cast<int64_t>(min(row, h - 1)) * w + lane_col, x[r]);
+            if (!(exists && lane_in)) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) x[r][v] = T(0);
+            }
+        } else {
+            buffer_load_run_as<kCacheStream, TI>(x[r], irows.row(min(row, h - 1), exists), in_off);
+        }
+    }
+
+    if (band == 0)
+        for (int c = lane; c <= w; c += 64) dst[c] = T(0);
+
+    {
+        double own[4] = {0.0, 0.0, 0.0, 0.0};
+#pragma unroll
+        for (int r = 0; r < RMAX; ++r)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) own[v] += static_cast<double>(x[r][v]);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) sums[band][v][lane] = own[v];
+    }
+    __syncthreads();
+    double colacc[4] = {0.0, 0.0, 0.0, 0.0};
+    for (int b = 0; b < band; ++b)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) colacc[v] += sums[b][v][lane];
+
+#pragma unroll
+    for (int bi = 0; bi < RMAX / RB; ++bi) {
+        if (bi * RB >= R) break;
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            const int row = r0 + bi * RB + rb;
+            double run = 0.0, pre[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                colacc[v] += static_cast<double>(x[bi * RB + rb][v]);
+                run += colacc[v];
+                pre[v] = run;
+            }
+            const double left = wave_inclusive_scan(run) - run;
+            T res[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) res[v] = static_cast<T>(left + pre[v]);
+            const RowRef orow = orows.row(min(row + 1, h), row < r1);
+            // (VEC: the rows are addressed by offset into one descriptor for the plane, without a
+            // bounds check of their own, so a lane past the row's end must not store)
+            if (!VEC || lane_in)
+                buffer_store_run<kCacheDefault, VEC>(res, orow, out_off, (w + 1) * static_cast<int>(sizeof(T)));
+            if (lane == 0 && row < r1) dst[static_cast<int64_t>(row + 1) * W1] = T(0);
+        }
+    }
+}
+
 template <class T>
 bool aligned_for_vec4(const T* p, int w) {
     return (w % 4 == 0) && (reinterpret_cast<uintptr_t>(p) % (4 * sizeof(T)) == 0);
@@ -676,9 +779,44 @@ struct LookbackByWidth<float, TI> {
     }
 };
 
+template <class TI>
+hipError_t launch_plane_scan(const TI* in, float* out, int64_t planes, int h, int w, int nb, int R,
+                             bool reverse, hipStream_t stream) {
+    const dim3 grid(static_cast<unsigned>(planes)), block(nb * 64);
+    const int rev = reverse ? 1 : 0;
+    const bool vec = aligned_for_vec4(in, w);
+#define LAUNCH_PLANE(RMAX)                                                                                \
+    if (vec) BOXCONV_LAUNCH("band_scan", (plane_scan_kernel<TI, RMAX, true>), grid, block, 0, stream, in, out, \
+                            h, w, R, planes, rev);                                                        \
+    else     BOXCONV_LAUNCH("band_scan", (plane_scan_kernel<TI, RMAX, false>), grid, block, 0, stream, in, out, \
+                            h, w, R, planes, rev)
+    if (R <= 8)       { LAUNCH_PLANE(8); }
+    else if (R <= 16) { LAUNCH_PLANE(16); }
+    else              { LAUNCH_PLANE(kPlaneRows); }
+#undef LAUNCH_PLANE
+    return hipGetLastError();
+}
+template <class T, class TI>
+struct PlaneScan {
+    static hipError_t run(const TI*, T*, int64_t, int, int, int, int, bool, hipStream_t) {
+        return hipErrorInvalidValue;       // float output only
+    }
+};
+template <class TI>
+struct PlaneScan<float, TI> {
+    static hipError_t run(const TI* in, float* out, int64_t planes, int h, int w, int nb, int R,
+                          bool reverse, hipStream_t stream) {
+        return launch_plane_scan<TI>(in, out, planes, h, w, nb, R, reverse, stream);
+    }
+};
+
 template <class T>
 bool single_pass_applies(const IntegralPlan& pl) {
     return pl.lookback && std::is_same<T, float>::value && lookback_enabled();
+}
+template <class T>
+bool plane_pass_applies(const IntegralPlan& pl) {
+    return pl.plane_per_workgroup && std::is_same<T, float>::value;
 }
 
 // Rows this narrow are scanned by band_scan_rows_kernel, which sums the band column sums itself;
@@ -692,6 +830,22 @@ inline bool scan_by_rows(int h, int w, size_t elem) {
 
 IntegralPlan plan_integral(int64_t planes, int h, int w, int64_t want) {
     IntegralPlan pl;
+    pl.plane_per_workgroup = false;
+    // Small planes: a workgroup per plane, a wave per band, bands of 8 to 24 rows (whole row
+    // batches) so that up to eight waves share the plane. (Types the kernel is not built for take
+    // the two passes with the same bands.)
+    // (BOXCONV_INTEGRAL_LOOKBACK=2 asks for the look-back kernel wherever it applies, here too)
+    if (switches().plane_integral && !lookback_any_shape() && h <= kPlaneMaxRows && w <= kPlaneMaxCols &&
+        planes < (1ll << 31)) {
+        int R = ((h + kPlaneWaves - 1) / kPlaneWaves + 3) / 4 * 4;
+        R = std::max(R, 8);
+        pl.R = R;
+        pl.nb = (h + R - 1) / R;
+        pl.aux_doubles = pl.nb > 1 ? planes * static_cast<int64_t>(pl.nb - 1) * w : 0;
+        pl.lookback = false;
+        pl.plane_per_workgroup = true;
+        return pl;
+    }
     // Enough workgroups to cover 256 CUs several times over, but bands no shorter than 32 rows
     // (the per-band column-sum vector is 8 B per column, i.e. 2/R of the input bytes) and no
     // taller than 256 (size of the per-row carry array in LDS).
@@ -784,6 +938,8 @@ hipError_t integral_image_any(const TI* in, T* out, int64_t planes, int h, int w
     const int nb = pl.nb, R = pl.R;
     const bool by_rows = scan_by_rows(h, w, sizeof(T));
     if (!by_rows && !std::is_same<T, TI>::value) return hipErrorInvalidValue;
+    if (plane_pass_applies<T>(pl))
+        return PlaneScan<T, TI>::run(in, out, planes, h, w, nb, R, reverse_order, stream);
     if (single_pass_applies<T>(pl))
         return LookbackByWidth<T, TI>::run(in, out, aux, planes, h, w, nb, R, reverse_order,
                                            workspace_prepared, stream);

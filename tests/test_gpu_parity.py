@@ -84,6 +84,30 @@ def test_integral_image_single_pass_waits_are_bounded(hip, switches, planes, h, 
     assert torch.allclose(three, usual, rtol=2e-7, atol=0) and torch.allclose(hip.integral_image(x), usual, rtol=2e-7, atol=0)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("planes,h,w", [(5, 1, 1), (3, 5, 7), (6, 28, 28), (2, 64, 128), (40, 64, 128), (3, 8, 256),
+                                        (2, 9, 255), (4, 57, 100), (3, 128, 256), (2, 129, 33), (7, 135, 240),
+                                        (2, 192, 256), (3, 191, 254), (2, 170, 3), (1, 100, 253)])
+def test_integral_image_plane_per_workgroup(hip, switches, planes, h, w, dtype):
+    """Planes of at most 192 rows and 256 columns are scanned by one workgroup each (a wave per
+    band of 8 to 24 rows, the bands' column sums handed over through LDS);
+    BOXCONV_INTEGRAL_PLANE=0 sends them through the two launches with the same bands, which give
+    the same bits. Both against float64 cumulative sums."""
+    x = torch.from_numpy(np.random.default_rng(planes + 7 * h + 1000 * w).random((planes, h, w), dtype=np.float32)
+                         * 4 - 1).cuda().to(dtype)
+    exact = torch.zeros(planes, h + 1, w + 1, dtype=torch.float64, device="cuda")
+    exact[:, 1:, 1:] = x.double().cumsum(1).cumsum(2)
+    got = hip.integral_image(x)
+    assert got.dtype == torch.float32 and got.shape == exact.shape
+    ideal = exact.float()
+    assert torch.all((got - ideal).abs() <= torch.from_numpy(np.spacing(np.abs(ideal.cpu().numpy()))).cuda())
+    assert (got != ideal).float().mean().item() < 1e-4
+    switches("BOXCONV_INTEGRAL_PLANE", "0")
+    two_launches = hip.integral_image(x)
+    switches("BOXCONV_INTEGRAL_PLANE", None)
+    assert torch.equal(got, two_launches)
+
+
 INT_TYPES = [(np.uint8, torch.uint8), (np.int8, torch.int8), (np.int16, torch.int16),
              (np.int32, torch.int32), (np.int64, torch.int64)]
 

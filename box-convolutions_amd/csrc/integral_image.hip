@@ -811,12 +811,12 @@ struct PlaneScan<float, TI> {
 };
 
 template <class T>
-bool single_pass_applies(const IntegralPlan& pl) {
-    return pl.lookback && std::is_same<T, float>::value && lookback_enabled();
-}
-template <class T>
 bool plane_pass_applies(const IntegralPlan& pl) {
     return pl.plane_per_workgroup && std::is_same<T, float>::value;
+}
+template <class T>
+bool single_pass_applies(const IntegralPlan& pl) {
+    return pl.lookback && std::is_same<T, float>::value && lookback_enabled() && !plane_pass_applies<T>(pl);
 }
 
 // Rows this narrow are scanned by band_scan_rows_kernel, which sums the band column sums itself;
@@ -830,22 +830,14 @@ inline bool scan_by_rows(int h, int w, size_t elem) {
 
 IntegralPlan plan_integral(int64_t planes, int h, int w, int64_t want) {
     IntegralPlan pl;
-    pl.plane_per_workgroup = false;
-    // Small planes: a workgroup per plane, a wave per band, bands of 8 to 24 rows (whole row
-    // batches) so that up to eight waves share the plane. (Types the kernel is not built for take
-    // the two passes with the same bands.)
+    // Small planes (float output): a workgroup per plane, a wave per band, bands of 8 to 24 rows
+    // (whole row batches) so that up to eight waves share the plane. The rest of the plan is what
+    // the types that kernel is not built for take, and what the workspace is sized for.
     // (BOXCONV_INTEGRAL_LOOKBACK=2 asks for the look-back kernel wherever it applies, here too)
-    if (switches().plane_integral && !lookback_any_shape() && h <= kPlaneMaxRows && w <= kPlaneMaxCols &&
-        planes < (1ll << 31)) {
-        int R = ((h + kPlaneWaves - 1) / kPlaneWaves + 3) / 4 * 4;
-        R = std::max(R, 8);
-        pl.R = R;
-        pl.nb = (h + R - 1) / R;
-        pl.aux_doubles = pl.nb > 1 ? planes * static_cast<int64_t>(pl.nb - 1) * w : 0;
-        pl.lookback = false;
-        pl.plane_per_workgroup = true;
-        return pl;
-    }
+    pl.plane_per_workgroup = switches().plane_integral && !lookback_any_shape() && h <= kPlaneMaxRows &&
+                             w <= kPlaneMaxCols && planes < (1ll << 31);
+    pl.plane_R = std::max(((h + kPlaneWaves - 1) / kPlaneWaves + 3) / 4 * 4, 8);
+    pl.plane_nb = (h + pl.plane_R - 1) / pl.plane_R;
     // Enough workgroups to cover 256 CUs several times over, but bands no shorter than 32 rows
     // (the per-band column-sum vector is 8 B per column, i.e. 2/R of the input bytes) and no
     // taller than 256 (size of the per-row carry array in LDS).
@@ -939,7 +931,7 @@ hipError_t integral_image_any(const TI* in, T* out, int64_t planes, int h, int w
     const bool by_rows = scan_by_rows(h, w, sizeof(T));
     if (!by_rows && !std::is_same<T, TI>::value) return hipErrorInvalidValue;
     if (plane_pass_applies<T>(pl))
-        return PlaneScan<T, TI>::run(in, out, planes, h, w, nb, R, reverse_order, stream);
+        return PlaneScan<T, TI>::run(in, out, planes, h, w, pl.plane_nb, pl.plane_R, reverse_order, stream);
     if (single_pass_applies<T>(pl))
         return LookbackByWidth<T, TI>::run(in, out, aux, planes, h, w, nb, R, reverse_order,
                                            workspace_prepared, stream);

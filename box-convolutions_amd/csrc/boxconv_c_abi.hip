@@ -237,17 +237,31 @@ int training_forward_impl(const T* input, T* x_min, T* x_max, T* y_min, T* y_max
     hipStream_t s = static_cast<hipStream_t>(stream);
     double* aux = static_cast<double*>(workspace);
     const boxconv::IntegralPlan plan = boxconv::plan_integral(planes, h, w);
-    bool prepared = false;
-    if (int rc = hip_result(boxconv::clip_and_prepare_integral_launch<T>(
-            boxconv::clip_args<T>(x_min, x_max, y_min, y_max, real, n, reparam_h, reparam_w, max_h,
-                                  max_w, exact != 0, project),
-            planes, w, aux, plan, &prepared, s), "clip launch"))
-        return rc;
-    if (planes == 0) return 0;
-    if (int rc = hip_result(boxconv::integral_image_launch<T>(input, integ, planes, h, w, aux, plan,
-                                                              prepared, false, s),
-                            "integral image launch"))
-        return rc;
+    bool fused = false;
+    if constexpr (std::is_same<T, float>::value) {
+        // small planes: the clip job rides on the integral image's own launch
+        if (boxconv::clip_rides_on_integral(plan, planes)) {
+            fused = true;
+            if (int rc = hip_result(boxconv::clip_and_plane_integral_launch<float>(
+                    boxconv::clip_args<float>(x_min, x_max, y_min, y_max, real, n, reparam_h, reparam_w,
+                                              max_h, max_w, exact != 0, project),
+                    input, integ, planes, h, w, plan, s), "clip and integral image launch"))
+                return rc;
+        }
+    }
+    if (!fused) {
+        bool prepared = false;
+        if (int rc = hip_result(boxconv::clip_and_prepare_integral_launch<T>(
+                boxconv::clip_args<T>(x_min, x_max, y_min, y_max, real, n, reparam_h, reparam_w, max_h,
+                                      max_w, exact != 0, project),
+                planes, w, aux, plan, &prepared, s), "clip launch"))
+            return rc;
+        if (planes == 0) return 0;
+        if (int rc = hip_result(boxconv::integral_image_launch<T>(input, integ, planes, h, w, aux, plan,
+                                                                  prepared, false, s),
+                                "integral image launch"))
+            return rc;
+    }
     if (n == 0) return 0;
     const boxconv::Dims d{in_planes, num_filters, h, w, planes, 0};
     const boxconv::BoxParams<T> prm{real, real + n, real + 2 * n, real + 3 * n};
@@ -267,17 +281,24 @@ int training_forward_half_impl(const TH* input, float* x_min, float* x_max, floa
     hipStream_t s = static_cast<hipStream_t>(stream);
     double* aux = static_cast<double*>(workspace);
     const boxconv::IntegralPlan plan = boxconv::plan_integral(planes, h, w);
-    bool prepared = false;
-    if (int rc = hip_result(boxconv::clip_and_prepare_integral_launch<float>(
-            boxconv::clip_args<float>(x_min, x_max, y_min, y_max, real, n, reparam_h, reparam_w, max_h,
-                                      max_w, exact != 0, project),
-            planes, w, aux, plan, &prepared, s), "clip launch"))
-        return rc;
-    if (planes == 0) return 0;
-    if (int rc = hip_result(boxconv::integral_image_widening_launch<TH>(input, integ, planes, h, w, aux,
-                                                                        plan, s, prepared),
-                            "integral image launch"))
-        return rc;
+    const boxconv::ClipArgs<float> clip = boxconv::clip_args<float>(
+        x_min, x_max, y_min, y_max, real, n, reparam_h, reparam_w, max_h, max_w, exact != 0, project);
+    if (boxconv::clip_rides_on_integral(plan, planes)) {
+        if (int rc = hip_result(boxconv::clip_and_plane_integral_launch<TH>(clip, input, integ, planes, h, w,
+                                                                            plan, s),
+                                "clip and integral image launch"))
+            return rc;
+    } else {
+        bool prepared = false;
+        if (int rc = hip_result(boxconv::clip_and_prepare_integral_launch<float>(clip, planes, w, aux, plan,
+                                                                                &prepared, s), "clip launch"))
+            return rc;
+        if (planes == 0) return 0;
+        if (int rc = hip_result(boxconv::integral_image_widening_launch<TH>(input, integ, planes, h, w, aux,
+                                                                            plan, s, prepared),
+                                "integral image launch"))
+            return rc;
+    }
     if (n == 0) return 0;
     const boxconv::Dims d{in_planes, num_filters, h, w, planes, 0};
     const boxconv::BoxParams<float> prm{real, real + n, real + 2 * n, real + 3 * n};

@@ -173,6 +173,14 @@ hipError_t clip_and_prepare_integral_launch(const ClipArgs<T>& clip, int64_t pla
                                             double* aux, const IntegralPlan& plan, bool* prepared,
                                             hipStream_t stream);
 
+// Small planes with float output (clip_rides_on_integral): the clip job in the launch of the
+// integral image itself, which needs no preparation there. TI: float, f16_t or bf16_t.
+bool clip_rides_on_integral(const IntegralPlan& plan, int64_t planes);
+template <class TI>
+hipError_t clip_and_plane_integral_launch(const ClipArgs<float>& clip, const TI* in, float* out,
+                                          int64_t planes, int h, int w, const IntegralPlan& plan,
+                                          hipStream_t stream);
+
 // real: null, or [4][n] receiving the clipped bounds times their reparametrization factor.
 template <class T>
 hipError_t clip_launch(T* xmin, T* xmax, T* ymin, T* ymax, T* real, int n, double reparam_h,

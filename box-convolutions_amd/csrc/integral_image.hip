@@ -591,12 +591,19 @@ constexpr int kPlaneMaxRows = kPlaneWaves * kPlaneRows, kPlaneMaxCols = 256;
 template <class TI, int RMAX, bool VEC>
 __global__ void __launch_bounds__(kPlaneWaves * 64)
 plane_scan_kernel(const TI* __restrict__ in, float* __restrict__ out, int h, int w, int R, int64_t planes,
-                  int reverse) {
+                  int reverse, ClipArgs<float> clip, int clip_blocks) {
     using T = float;
     constexpr int RB = 4;
     __shared__ double sums[kPlaneWaves][4][64];
 
-    int64_t p = blockIdx.x;
+    // a clip job on the side (its first clip_blocks workgroups): what a training-mode forward does
+    // before the integral image, in the same launch
+    if (static_cast<int>(blockIdx.x) < clip_blocks) {
+        const int i = blockIdx.x * blockDim.x + threadIdx.x;
+        if (i < clip.n) clip_box(clip, i);
+        return;
+    }
+    int64_t p = blockIdx.x - clip_blocks;
     if (reverse) p = planes - 1 - p;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -781,15 +788,17 @@ struct LookbackByWidth<float, TI> {
 
 template <class TI>
 hipError_t launch_plane_scan(const TI* in, float* out, int64_t planes, int h, int w, int nb, int R,
-                             bool reverse, hipStream_t stream) {
-    const dim3 grid(static_cast<unsigned>(planes)), block(nb * 64);
+                             bool reverse, hipStream_t stream, const ClipArgs<float>* clip_job = nullptr) {
+    const ClipArgs<float> clip = clip_job != nullptr ? *clip_job : ClipArgs<float>{};
+    const int clip_blocks = (clip.n + nb * 64 - 1) / (nb * 64);
+    const dim3 grid(static_cast<unsigned>(planes + clip_blocks)), block(nb * 64);
     const int rev = reverse ? 1 : 0;
     const bool vec = aligned_for_vec4(in, w);
 #define LAUNCH_PLANE(RMAX)                                                                                \
     if (vec) BOXCONV_LAUNCH("band_scan", (plane_scan_kernel<TI, RMAX, true>), grid, block, 0, stream, in, out, \
-                            h, w, R, planes, rev);                                                        \
+                            h, w, R, planes, rev, clip, clip_blocks);                                     \
     else     BOXCONV_LAUNCH("band_scan", (plane_scan_kernel<TI, RMAX, false>), grid, block, 0, stream, in, out, \
-                            h, w, R, planes, rev)
+                            h, w, R, planes, rev, clip, clip_blocks)
     if (R <= 8)       { LAUNCH_PLANE(8); }
     else if (R <= 16) { LAUNCH_PLANE(16); }
     else              { LAUNCH_PLANE(kPlaneRows); }
@@ -886,6 +895,24 @@ IntegralPlan plan_integral(int64_t planes, int h, int w, int64_t want) {
     pl.aux_doubles = (nb > 1) ? planes * static_cast<int64_t>(nb - 1) * (pl.lookback ? lookback_row_words(w) : w) : 0;
     return pl;
 }
+
+bool clip_rides_on_integral(const IntegralPlan& pl, int64_t planes) {
+    return pl.plane_per_workgroup && planes > 0 && planes + (1 << 20) < (1ll << 31);
+}
+
+template <class TI>
+hipError_t clip_and_plane_integral_launch(const ClipArgs<float>& clip, const TI* in, float* out,
+                                          int64_t planes, int h, int w, const IntegralPlan& pl,
+                                          hipStream_t stream) {
+    if (!clip_rides_on_integral(pl, planes)) return hipErrorInvalidValue;
+    return launch_plane_scan<TI>(in, out, planes, h, w, pl.plane_nb, pl.plane_R, false, stream, &clip);
+}
+template hipError_t clip_and_plane_integral_launch<float>(const ClipArgs<float>&, const float*, float*, int64_t,
+                                                          int, int, const IntegralPlan&, hipStream_t);
+template hipError_t clip_and_plane_integral_launch<f16_t>(const ClipArgs<float>&, const f16_t*, float*, int64_t,
+                                                          int, int, const IntegralPlan&, hipStream_t);
+template hipError_t clip_and_plane_integral_launch<bf16_t>(const ClipArgs<float>&, const bf16_t*, float*, int64_t,
+                                                           int, int, const IntegralPlan&, hipStream_t);
 
 template <class T>
 hipError_t clip_and_prepare_integral_launch(const ClipArgs<T>& clip, int64_t planes, int w,

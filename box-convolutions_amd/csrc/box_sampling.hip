@@ -112,7 +112,7 @@ StreamPlan plan_grad_output_stream(int64_t planes_f, int h, int w, size_t elem_s
     R += R & 1;                                        // rows are handled in pairs
     sp.R = std::max(R, 2);
     sp.nb = (h + sp.R - 1) / sp.R;
-    sp.parts = rc.nt == 1024 ? 2 : 1;
+    sp.parts = (rc.nt == 1024 || stream_double_wide_split(w, elem_size)) ? 2 : 1;
     return sp;
 }
 

@@ -286,9 +286,14 @@ inline bool reverse_grad_input() { return switches().gi_reverse; }
 // three or four columns per lane need 200 to 580 registers more than a lane has: the kernels ran
 // out of scratch memory, at 8 times the time of their float counterparts instead of twice. Rows of
 // up to 1024 doubles therefore get at most two columns per lane (a lane's state is then what four
-// columns are in floats). Wider rows keep three or four on eight waves: sixteen waves with two
-// columns per lane, the two jobs as two launches, leave a lane 128 registers, spill as well and
-// were measured slower (2048 columns: 1176 against 1092 us).
+// columns are in floats).
+// Rows of 1025 to 2048 doubles: the two jobs of the grad_output pass as two launches, the
+// parameter sums by two workgroups of 512 threads per band that own half of the columns each
+// (two columns per lane), the column workspace by one workgroup with three or four columns per
+// lane; neither spills.
+inline bool stream_double_wide_split(int w, size_t elem_size) {
+    return elem_size == 8 && w > 1024 && w <= 2048 && switches().stream_narrow_double;
+}
 inline RowConfig stream_row_config(int w, size_t elem_size) {
     if (elem_size == 8 && w <= 1024 && switches().stream_narrow_double) {
         RowConfig c;

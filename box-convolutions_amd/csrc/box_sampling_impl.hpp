@@ -1552,6 +1552,24 @@ hipError_t grad_output_stream_launch(const T* integ, const TG* grad_out, BoxPara
             return hipErrorInvalidValue;
         }
     }
+    if constexpr (sizeof(T) == 8) {
+        if (stream_double_wide_split(d.w, sizeof(T))) {
+            SampleArgs<T> ap = a;
+            if (params && acc_slots == 0) return hipErrorInvalidValue;   // (the atomic mode has no slot per part)
+            finish_args(ap, planes_f * a.nb * 2);
+            const dim3 grid_p(static_cast<unsigned>(ap.per_xcd * kXcds));
+#define LAUNCH_GD(KK, EX, FU) \
+            if (params) BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_kernel<T, TG, 512, 2, EX, false, true, false, 2>), grid_p, dim3(512), lds, stream, ap); \
+            if (scan)   BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_kernel<T, TG, 512, KK, EX, FU, false, true>), grid, dim3(512), lds, stream, a)
+#define LAUNCH_GD_K(EX, FU) if (rc.K == 3) { LAUNCH_GD(3, EX, FU); } else { LAUNCH_GD(4, EX, FU); }
+            if (rc.nt != 512 || rc.K < 3) return hipErrorInvalidValue;
+            if (exact) { if (rc.full) { LAUNCH_GD_K(true, true) } else { LAUNCH_GD_K(true, false) } }
+            else       { if (rc.full) { LAUNCH_GD_K(false, true) } else { LAUNCH_GD_K(false, false) } }
+#undef LAUNCH_GD_K
+#undef LAUNCH_GD
+            return hipGetLastError();
+        }
+    }
     // float rows of a multiple of four columns, both products wanted, a slot per workgroup for the
     // sums: the kernel with four consecutive columns per lane
     if constexpr (std::is_same<T, float>::value) {

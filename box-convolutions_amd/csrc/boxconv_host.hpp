@@ -200,7 +200,7 @@ struct Switches {
     bool plane_integral;      // BOXCONV_INTEGRAL_PLANE=0 clears it: no plane-per-workgroup integral image
     bool stream_consecutive;  // BOXCONV_STREAM_CONSEC=0 clears it: no consecutive-column variant of the grad_output pass at all
     bool stream_consecutive_partial;  // BOXCONV_STREAM_CONSEC=1 clears it: that variant only for rows that fill its workgroup exactly
-    bool stream_narrow_double;  // BOXCONV_STREAM_F64_NARROW=0 clears it: float64 rows of up to 1024 columns with three or four columns per lane like float32
+    bool stream_narrow_double;  // BOXCONV_STREAM_F64_NARROW=0 clears it: float64 rows with three or four columns per lane and one launch like float32
     bool interleave_workspace;  // BOXCONV_M_INTERLEAVE=0 clears it: rows of the column workspace in their natural order
     int stream_workgroups;    // BOXCONV_STREAM_WGS: workgroups the grad_output pass aims for when it cuts planes into bands (2048)
     int spin_limit;           // BOXCONV_INTEGRAL_SPIN: polls of a hand-over word before re-summing (64)

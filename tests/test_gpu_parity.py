@@ -394,12 +394,14 @@ def test_grad_output_pass_variants_agree(hip, oracle, switches, h, w, exact):
 
 
 @pytest.mark.parametrize("exact", [True, False])
-@pytest.mark.parametrize("h,w", [(37, 130), (40, 256), (34, 300), (70, 512), (21, 700), (36, 1024), (18, 1025)])
+@pytest.mark.parametrize("h,w", [(37, 130), (40, 256), (34, 300), (70, 512), (21, 700), (36, 1024), (18, 1025),
+                                 (12, 1100), (16, 1536), (10, 1538), (14, 2047), (12, 2048)])
 def test_float64_grad_output_pass_shapes_agree(hip, oracle, switches, h, w, exact):
     """float64 rows of up to 1024 columns run the grad_output pass with at most two columns per
-    lane, and on four or eight waves as two launches (parameter sums, column workspace);
-    BOXCONV_STREAM_F64_NARROW=0 gives them float32's three or four columns per lane and the one
-    launch, which rows of 1025 columns and more keep. Both against the oracle and against each other."""
+    lane, and on four or eight waves as two launches (parameter sums, column workspace); rows of
+    1025 to 2048 columns as two launches as well, the parameter sums by two workgroups per band
+    with two columns per lane. BOXCONV_STREAM_F64_NARROW=0 gives all of them float32's three or
+    four columns per lane and the one launch. Both against the oracle and against each other."""
     rng = np.random.default_rng(3 * h + w + int(exact))
     B, C, F = 2, 2, 3
     x = rng.standard_normal((B, C, h, w))

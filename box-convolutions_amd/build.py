@@ -34,7 +34,7 @@ SOURCES = [(s, s.replace(".hip", ".o"), []) for s in
             "boxconv_c_abi.hip")]
 for _tag, _t, _tg in (("f32", "float", "float"), ("f64", "double", "double"),
                       ("f16", "float", "f16_t"), ("bf16", "float", "bf16_t")):
-    for _part in (1, 2) + ((3,) if _t == "float" else ()):
+    for _part in (1, 2) + ((3, 4) if _t == "float" else ()):
         SOURCES.append(_inst(_tag, _t, _tg, _part, _t == _tg))
 HEADERS = ["boxconv_device.hpp", "boxconv_host.hpp", "box_sampling_common.hpp", "box_sampling_impl.hpp",
            os.path.join("..", "..", "include", "boxconv.h")]

@@ -930,8 +930,11 @@ __device__ __forceinline__ void load4_dword_aligned(const float* p, float (&v)[4
 // share a CU, where at two per SIMD two, three or two of its eight wave slots would stay empty.
 // Measured at three waves: 480 x 640 170 -> 149 us; rows of 960 and 1000 columns, four waves with
 // idle lanes, got slower with three per SIMD like the full rows: 230 -> 235 us.)
-template <class TG, int NT, bool EXACT, bool FULL>
-__global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, (NT == 192 || NT == 320 || NT == 384) ? 3 : 2)))
+// SCAN = false: the parameter sums only (the input needs no gradient, as in a network's first
+// layer): no suffix sums, no column workspace, half the registers; four waves per SIMD then (no
+// column workspace competes for the L2).
+template <class TG, int NT, bool EXACT, bool FULL, bool SCAN = true>
+__global__ void __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(2, !SCAN ? 4 : (NT == 192 || NT == 320 || NT == 384) ? 3 : 2)))
 grad_output_stream_consec_kernel(SampleArgs<float> a) {
     using T = float;
     constexpr int K = 4;
@@ -1009,7 +1012,7 @@ grad_output_stream_consec_kernel(SampleArgs<float> a) {
         grow[0][e] = RowPair<T>{T(0), T(0)};
         grow[1][e] = RowPair<T>{T(0), T(0)};
     }
-    if (band == 0)
+    if (SCAN && band == 0)
         for (int c = tid; c < mpitch; c += NT) mrows[c] = T(0);
 
     auto tail_weight = [&](int j, int ylo, int yhi, T fylo, T fyhi) {
@@ -1163,7 +1166,7 @@ grad_output_stream_consec_kernel(SampleArgs<float> a) {
             for (int n = 0; n < 5; ++n) total[n] += static_cast<double>(sum[n]);
         }
 
-        if (OWN_W) {
+        if (SCAN && OWN_W) {
             // rare: the mirrored split cuts the box at other whole pixels; weights and tails of
             // the column workspace from that split
             RowPair<T> R[K + 1], L[K + 1];
@@ -1189,9 +1192,9 @@ grad_output_stream_consec_kernel(SampleArgs<float> a) {
 
         // A[c] = (sum of all W + tail) - (W of the columns before c): exclusive prefix inside the
         // lane, the lanes to the left by a wave scan, the other waves through LDS
-        T ex0[K], ex1[K];
-        T base0, base1;
-        {
+        T ex0[K] = {}, ex1[K] = {};
+        T base0 = T(0), base1 = T(0);
+        if (SCAN) {
             T run0 = T(0), run1 = T(0);
 #pragma unroll
             for (int k = 0; k < K; ++k) {
@@ -1211,7 +1214,7 @@ grad_output_stream_consec_kernel(SampleArgs<float> a) {
         }
         if (MERGED && PREFETCH) BOXCONV_PUBLISH_CONSEC(FLIP ^ 1, i + 2, m0, m1, t1, n0, n1, b2, n2, n3, tn0, tn1)
         __syncthreads();                             // wave totals (and the next pair's rows) visible
-        {
+        if (SCAN) {
 #pragma unroll
             for (int wv = 0; wv < WAVES; ++wv) {
                 const WaveSums ws = wsum[FLIP][wv];
@@ -1270,7 +1273,7 @@ grad_output_stream_consec_kernel(SampleArgs<float> a) {
             row_pair(i, std::false_type{}, Flip0{}, OWN_W_TAG{});            \
         }                                                                    \
     }
-    if (own_w) BOXCONV_ALL_PAIRS(std::true_type)
+    if (SCAN && own_w) BOXCONV_ALL_PAIRS(std::true_type)
     else BOXCONV_ALL_PAIRS(std::false_type)
 #undef BOXCONV_ALL_PAIRS
 #undef BOXCONV_PUBLISH_CONSEC
@@ -1471,24 +1474,25 @@ hipError_t grad_input_launch(const T* gint, int band_rows, BoxParams<T> prm, TO*
 // policy (the memory-side cache holds 256 MB; the grad-input kernel reads that part first).
 inline int64_t cached_tail_bytes() { return switches().keep_tail_bytes; }
 
-// The launches of grad_output_stream_consec_kernel (`lanes` busy lanes of a workgroup of `cnt`).
-// Its instantiations are a translation unit of their own (BOXCONV_INST_PART 3): some hundred
-// kernels that would otherwise double the compile time of the unit with the other variant.
-template <class TG>
+// The launches of grad_output_stream_consec_kernel (`lanes` busy lanes of a workgroup of `cnt`;
+// SCAN = false: parameter sums only). Its instantiations are translation units of their own
+// (BOXCONV_INST_PART 3 and 4): some hundred kernels that would otherwise double the compile time
+// of the unit with the other variant.
+template <class TG, bool SCAN>
 hipError_t grad_output_stream_consec_launch(const SampleArgs<float>& a, int lanes, int cnt, bool exact,
                                             dim3 grid, hipStream_t stream);
-#if defined(BOXCONV_INST_PART) && BOXCONV_INST_PART == 3
-template <class TG>
+#if defined(BOXCONV_INST_PART) && (BOXCONV_INST_PART == 3 || BOXCONV_INST_PART == 4)
+template <class TG, bool SCAN>
 hipError_t grad_output_stream_consec_launch(const SampleArgs<float>& a, int lanes, int cnt, bool exact,
                                             dim3 grid, hipStream_t stream) {
     const size_t lds = 0;                              // the kernel's LDS is statically sized
 #define LAUNCH_GC(NT) \
     if (lanes == NT) { \
-        if (exact) BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, true, true>), grid, dim3(NT), lds, stream, a); \
-        else       BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, false, true>), grid, dim3(NT), lds, stream, a); \
+        if (exact) BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, true, true, SCAN>), grid, dim3(NT), lds, stream, a); \
+        else       BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, false, true, SCAN>), grid, dim3(NT), lds, stream, a); \
     } else { \
-        if (exact) BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, true, false>), grid, dim3(NT), lds, stream, a); \
-        else       BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, false, false>), grid, dim3(NT), lds, stream, a); \
+        if (exact) BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, true, false, SCAN>), grid, dim3(NT), lds, stream, a); \
+        else       BOXCONV_LAUNCH("grad_output_stream", (grad_output_stream_consec_kernel<TG, NT, false, false, SCAN>), grid, dim3(NT), lds, stream, a); \
     }
     switch (cnt) {
         case 64: LAUNCH_GC(64) break;
@@ -1570,8 +1574,8 @@ hipError_t grad_output_stream_launch(const T* integ, const TG* grad_out, BoxPara
             return hipGetLastError();
         }
     }
-    // float rows of a multiple of four columns, both products wanted, a slot per workgroup for the
-    // sums: the kernel with four consecutive columns per lane
+    // float rows of a multiple of four columns, the parameter sums wanted (with or without the column
+    // workspace), a slot per workgroup for the sums: the kernel with four consecutive columns per lane
     if constexpr (std::is_same<T, float>::value) {
         const bool aligned = reinterpret_cast<uintptr_t>(grad_out) % (4 * sizeof(TG)) == 0 && d.w % 4 == 0;
         // the smallest workgroup (whole waves) whose lanes, four columns each, cover the row. Only
@@ -1587,8 +1591,9 @@ hipError_t grad_output_stream_launch(const T* integ, const TG* grad_out, BoxPara
         const bool covers = d.w <= 2048 && lanes >= 1 &&
                             (exact_fit || (switches().stream_consecutive_partial && lanes * 8 >= cnt * 3 &&
                                            !(rc.full && rc.K == 1)));
-        if (switches().stream_consecutive && covers && params && scan && acc_slots > 0 && aligned) {
-            return grad_output_stream_consec_launch<TG>(a, lanes, cnt, exact, grid, stream);
+        if (switches().stream_consecutive && covers && params && acc_slots > 0 && aligned) {
+            if (scan) return grad_output_stream_consec_launch<TG, true>(a, lanes, cnt, exact, grid, stream);
+            return grad_output_stream_consec_launch<TG, false>(a, lanes, cnt, exact, grid, stream);
         }
     }
     // doubles, two columns per lane on four or eight waves: the kernel that does both jobs needs

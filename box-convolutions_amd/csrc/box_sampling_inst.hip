@@ -3,7 +3,8 @@
 // element type of grad_output / grad_input, BOXCONV_INST_PART the half of the templates
 //   1: the streaming pass over grad_output
 //   2: the gradient w.r.t. the input, and (where T == TG) the gather and finalize launches.
-//   3: (T = float) the streaming pass's variant with consecutive columns per lane.
+//   3: (T = float) the streaming pass's variant with consecutive columns per lane;
+//   4: the same variant for the parameter sums alone.
 
 #include "box_sampling_impl.hpp"
 
@@ -14,8 +15,11 @@ template hipError_t grad_output_stream_launch<BOXCONV_INST_T, BOXCONV_INST_TG>(
     const BOXCONV_INST_T*, const BOXCONV_INST_TG*, BoxParams<BOXCONV_INST_T>, double*, int, BOXCONV_INST_T*,
     const StreamPlan&, Dims, bool, hipStream_t);
 #elif BOXCONV_INST_PART == 3
-template hipError_t grad_output_stream_consec_launch<BOXCONV_INST_TG>(const SampleArgs<float>&, int, int, bool, dim3,
-                                                                      hipStream_t);
+template hipError_t grad_output_stream_consec_launch<BOXCONV_INST_TG, true>(const SampleArgs<float>&, int, int, bool,
+                                                                            dim3, hipStream_t);
+#elif BOXCONV_INST_PART == 4
+template hipError_t grad_output_stream_consec_launch<BOXCONV_INST_TG, false>(const SampleArgs<float>&, int, int, bool,
+                                                                             dim3, hipStream_t);
 #else
 template hipError_t grad_input_launch<BOXCONV_INST_T, BOXCONV_INST_TG>(
     const BOXCONV_INST_T*, int, BoxParams<BOXCONV_INST_T>, BOXCONV_INST_TG*, Dims, bool, bool, hipStream_t,

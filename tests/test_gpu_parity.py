@@ -394,6 +394,30 @@ def test_grad_output_pass_variants_agree(hip, oracle, switches, h, w, exact):
 
 
 @pytest.mark.parametrize("exact", [True, False])
+@pytest.mark.parametrize("h,w", [(67, 256), (30, 640), (70, 1024), (22, 1800), (20, 2044), (36, 100), (33, 44), (25, 2048)])
+def test_parameter_gradients_alone(hip, oracle, h, w, exact):
+    """When the input needs no gradient (a network's first layer) the grad_output pass forms the
+    parameter sums only: on rows that take the kernel with consecutive columns per lane, that
+    kernel without its column workspace. The sums are formed the same way with or without it, so
+    the four gradients equal those of the full backward bit for bit; and they meet the oracle."""
+    rng = np.random.default_rng(11 * h + w + int(exact))
+    B, C, F = 2, 2, 3
+    x = rng.standard_normal((B, C, h, w)).astype(np.float32)
+    g = (rng.standard_normal((B, C * F, h, w)) + 0.25).astype(np.float32)
+    boxes = list(make_boxes(rng, C, F, h, w, "hanging", away_from_integers=0.05))
+    if not exact:
+        boxes[1] = np.maximum(boxes[1], np.ceil(boxes[0]) + 1).astype(np.float32)
+        boxes[3] = np.maximum(boxes[3], np.ceil(boxes[2]) + 1).astype(np.float32)
+    needs = (False, True, True, True, True)
+    cpu, gpu, sc = run_both(hip, oracle, x, tuple(boxes), 3.5 * h, 2.25 * w, True, exact, g, needs)
+    assert gpu[1][0] is None
+    assert_parity(cpu, gpu, np.float32, "parameters only %dx%d exact=%s" % (h, w, exact), **sc)
+    _, full, _ = run_both(hip, oracle, x, tuple(boxes), 3.5 * h, 2.25 * w, True, exact, g)
+    for a, b in zip(gpu[1][1:], full[1][1:]):
+        assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("exact", [True, False])
 @pytest.mark.parametrize("h,w", [(37, 130), (40, 256), (34, 300), (70, 512), (21, 700), (36, 1024), (18, 1025),
                                  (12, 1100), (16, 1536), (10, 1538), (14, 2047), (12, 2048)])
 def test_float64_grad_output_pass_shapes_agree(hip, oracle, switches, h, w, exact):

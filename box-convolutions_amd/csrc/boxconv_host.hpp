@@ -34,7 +34,6 @@ struct IntegralPlan {
     int64_t aux_doubles;   // scratch for the column sums of all bands but the last
     bool lookback;         // geometry fits the single-pass kernel (bands of <= 32 rows, one tile wide)
     bool plane_per_workgroup;  // planes of at most 192 rows and 256 columns: one workgroup scans a whole plane (float output)
-    int plane_nb, plane_R;     // that kernel's bands per plane (its waves) and rows per band
 };
 // `want`: number of workgroups to aim for.
 IntegralPlan plan_integral(int64_t planes, int h, int w, int64_t want = 1024);

@@ -685,6 +685,113 @@ plane_scan_kernel(const TI* __restrict__ in, float* __restrict__ out, int h, int
     }
 }
 
+// Inclusive prefix sum within segments of L consecutive lanes (L = 16 or 32): the first steps of
+// wave_inclusive_scan. All lanes must be active.
+template <int L>
+__device__ __forceinline__ double segment_inclusive_scan(double x) {
+    static_assert(L == 16 || L == 32, "segments of one or two DPP rows");
+    x += dpp_move<0x111, 0xf>(x, x);
+    x += dpp_move<0x112, 0xf>(x, x);
+    x += dpp_move<0x114, 0xf>(x, x);
+    x += dpp_move<0x118, 0xf>(x, x);
+    if (L == 32) x += dpp_move<0x142, 0xa>(0.0, x);   // lane 15 of rows 0,2 into rows 1,3
+    return x;
+}
+
+// The same for planes of at most 128 (L = 32) or 64 (L = 16) columns, which would leave half or
+// three quarters of every wave idle: a wave takes 64 / L bands side by side, L lanes each (band
+// v of the plane: wave v / (64/L), lanes (v % (64/L)) * L ..), every lane walking down its own
+// band's rows. Rows of a multiple of four columns from a 16-byte aligned address only.
+template <class TI, int RMAX, int L>
+__global__ void __launch_bounds__(kPlaneWaves * 64)
+plane_scan_packed_kernel(const TI* __restrict__ in, float* __restrict__ out, int h, int w, int R, int64_t planes,
+                         int reverse, ClipArgs<float> clip, int clip_blocks) {
+    using T = float;
+    constexpr int RB = 4, S = 64 / L;
+    __shared__ double sums[kPlaneWaves * S * 4 * L];      // [band][4][L]
+
+    if (static_cast<int>(blockIdx.x) < clip_blocks) {
+        const int i = blockIdx.x * blockDim.x + threadIdx.x;
+        if (i < clip.n) clip_box(clip, i);
+        return;
+    }
+    int64_t p = blockIdx.x - clip_blocks;
+    if (reverse) p = planes - 1 - p;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int l = lane & (L - 1);
+    const int band = (tid >> 6) * S + lane / L;             // per lane; bands past the plane hold no rows
+    const int r0 = band * R;
+    const int r1 = min(h, r0 + R);
+    const int64_t W1 = static_cast<int64_t>(w) + 1;
+    const int c0 = 4 * l;
+    const bool lane_in = c0 < w;
+
+    const TI* src = in + p * static_cast<int64_t>(h) * w;
+    T* dst = out + p * static_cast<int64_t>(h + 1) * W1;
+    const Rows<T, true> orows(dst, W1, w + 1, h + 1);
+    const RowRef oplane = orows.row(0);                      // the plane as one buffer; rows by offset
+    const unsigned lane_col = lane_in ? static_cast<unsigned>(c0) : 0u;
+
+    T x[RMAX][4];
+#pragma unroll
+    for (int r = 0; r < RMAX; ++r) {
+        const int row = r0 + r;
+        const bool exists = r < R && row < r1 && lane_in;
+        load_quad(src + static_cast<int64_t>(min(row, h - 1)) * w + lane_col, x[r]);
+        if (!exists) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) x[r][v] = T(0);
+        }
+    }
+
+    if (tid < 64)
+        for (int c = tid; c <= w; c += 64) dst[c] = T(0);
+
+    {
+        double own[4] = {0.0, 0.0, 0.0, 0.0};
+#pragma unroll
+        for (int r = 0; r < RMAX; ++r)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) own[v] += static_cast<double>(x[r][v]);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) sums[(band * 4 + v) * L + l] = own[v];
+    }
+    __syncthreads();
+    double colacc[4] = {0.0, 0.0, 0.0, 0.0};
+    const int wave_last = ((tid >> 6) + 1) * S - 1;         // the wave's last band (wave-uniform)
+    for (int b = 0; b < wave_last; ++b)
+        if (b < band) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) colacc[v] += sums[(b * 4 + v) * L + l];
+        }
+
+#pragma unroll
+    for (int bi = 0; bi < RMAX / RB; ++bi) {
+        if (bi * RB >= R) break;
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            const int row = r0 + bi * RB + rb;
+            double run = 0.0, pre[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                colacc[v] += static_cast<double>(x[bi * RB + rb][v]);
+                run += colacc[v];
+                pre[v] = run;
+            }
+            const double left = segment_inclusive_scan<L>(run) - run;
+            T res[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) res[v] = static_cast<T>(left + pre[v]);
+            if (row < r1) {
+                const int off = static_cast<int>((static_cast<int64_t>(row + 1) * W1 + c0 + 1) * sizeof(T));
+                if (lane_in) buffer_store_run<kCacheDefault, true>(res, oplane, off, 0);
+                if (l == 0) dst[static_cast<int64_t>(row + 1) * W1] = T(0);
+            }
+        }
+    }
+}
+
 template <class T>
 bool aligned_for_vec4(const T* p, int w) {
     return (w % 4 == 0) && (reinterpret_cast<uintptr_t>(p) % (4 * sizeof(T)) == 0);
@@ -786,16 +893,33 @@ struct LookbackByWidth<float, TI> {
     }
 };
 
+// Bands of the plane-per-workgroup kernels: `slots` bands fit a workgroup (eight waves, times the
+// bands a wave takes side by side); rows per band: whole row batches, at least 8, so that all
+// rows fit those bands.
+inline int plane_band_rows(int h, int slots) {
+    return std::max(((h + slots - 1) / slots + 3) / 4 * 4, 8);
+}
+
 template <class TI>
-hipError_t launch_plane_scan(const TI* in, float* out, int64_t planes, int h, int w, int nb, int R,
-                             bool reverse, hipStream_t stream, const ClipArgs<float>* clip_job = nullptr) {
+hipError_t launch_plane_scan(const TI* in, float* out, int64_t planes, int h, int w, bool reverse,
+                             hipStream_t stream, const ClipArgs<float>* clip_job = nullptr) {
     const ClipArgs<float> clip = clip_job != nullptr ? *clip_job : ClipArgs<float>{};
-    const int clip_blocks = (clip.n + nb * 64 - 1) / (nb * 64);
-    const dim3 grid(static_cast<unsigned>(planes + clip_blocks)), block(nb * 64);
     const int rev = reverse ? 1 : 0;
     const bool vec = aligned_for_vec4(in, w);
+    // lanes per row: rows of at most 128 / 64 columns share a wave with one / three more bands
+    const int L = (vec && w <= 64) ? 16 : (vec && w <= 128) ? 32 : 64;
+    const int S = 64 / L;
+    const int R = plane_band_rows(h, kPlaneWaves * S);
+    const int nb = (h + R - 1) / R;
+    const int waves = (nb + S - 1) / S;
+    const int clip_blocks = (clip.n + waves * 64 - 1) / (waves * 64);
+    const dim3 grid(static_cast<unsigned>(planes + clip_blocks)), block(waves * 64);
 #define LAUNCH_PLANE(RMAX)                                                                                \
-    if (vec) BOXCONV_LAUNCH("band_scan", (plane_scan_kernel<TI, RMAX, true>), grid, block, 0, stream, in, out, \
+    if (L == 16)  BOXCONV_LAUNCH("band_scan", (plane_scan_packed_kernel<TI, RMAX, 16>), grid, block, 0, stream, \
+                                 in, out, h, w, R, planes, rev, clip, clip_blocks);                       \
+    else if (L == 32) BOXCONV_LAUNCH("band_scan", (plane_scan_packed_kernel<TI, RMAX, 32>), grid, block, 0, stream, \
+                                 in, out, h, w, R, planes, rev, clip, clip_blocks);                       \
+    else if (vec) BOXCONV_LAUNCH("band_scan", (plane_scan_kernel<TI, RMAX, true>), grid, block, 0, stream, in, out, \
                             h, w, R, planes, rev, clip, clip_blocks);                                     \
     else     BOXCONV_LAUNCH("band_scan", (plane_scan_kernel<TI, RMAX, false>), grid, block, 0, stream, in, out, \
                             h, w, R, planes, rev, clip, clip_blocks)
@@ -807,15 +931,15 @@ hipError_t launch_plane_scan(const TI* in, float* out, int64_t planes, int h, in
 }
 template <class T, class TI>
 struct PlaneScan {
-    static hipError_t run(const TI*, T*, int64_t, int, int, int, int, bool, hipStream_t) {
+    static hipError_t run(const TI*, T*, int64_t, int, int, bool, hipStream_t) {
         return hipErrorInvalidValue;       // float output only
     }
 };
 template <class TI>
 struct PlaneScan<float, TI> {
-    static hipError_t run(const TI* in, float* out, int64_t planes, int h, int w, int nb, int R,
-                          bool reverse, hipStream_t stream) {
-        return launch_plane_scan<TI>(in, out, planes, h, w, nb, R, reverse, stream);
+    static hipError_t run(const TI* in, float* out, int64_t planes, int h, int w, bool reverse,
+                          hipStream_t stream) {
+        return launch_plane_scan<TI>(in, out, planes, h, w, reverse, stream);
     }
 };
 
@@ -845,8 +969,6 @@ IntegralPlan plan_integral(int64_t planes, int h, int w, int64_t want) {
     // (BOXCONV_INTEGRAL_LOOKBACK=2 asks for the look-back kernel wherever it applies, here too)
     pl.plane_per_workgroup = switches().plane_integral && !lookback_any_shape() && h <= kPlaneMaxRows &&
                              w <= kPlaneMaxCols && planes < (1ll << 31);
-    pl.plane_R = std::max(((h + kPlaneWaves - 1) / kPlaneWaves + 3) / 4 * 4, 8);
-    pl.plane_nb = (h + pl.plane_R - 1) / pl.plane_R;
     // Enough workgroups to cover 256 CUs several times over, but bands no shorter than 32 rows
     // (the per-band column-sum vector is 8 B per column, i.e. 2/R of the input bytes) and no
     // taller than 256 (size of the per-row carry array in LDS).
@@ -905,7 +1027,7 @@ hipError_t clip_and_plane_integral_launch(const ClipArgs<float>& clip, const TI*
                                           int64_t planes, int h, int w, const IntegralPlan& pl,
                                           hipStream_t stream) {
     if (!clip_rides_on_integral(pl, planes)) return hipErrorInvalidValue;
-    return launch_plane_scan<TI>(in, out, planes, h, w, pl.plane_nb, pl.plane_R, false, stream, &clip);
+    return launch_plane_scan<TI>(in, out, planes, h, w, false, stream, &clip);
 }
 template hipError_t clip_and_plane_integral_launch<float>(const ClipArgs<float>&, const float*, float*, int64_t,
                                                           int, int, const IntegralPlan&, hipStream_t);
@@ -958,7 +1080,7 @@ hipError_t integral_image_any(const TI* in, T* out, int64_t planes, int h, int w
     const bool by_rows = scan_by_rows(h, w, sizeof(T));
     if (!by_rows && !std::is_same<T, TI>::value) return hipErrorInvalidValue;
     if (plane_pass_applies<T>(pl))
-        return PlaneScan<T, TI>::run(in, out, planes, h, w, pl.plane_nb, pl.plane_R, reverse_order, stream);
+        return PlaneScan<T, TI>::run(in, out, planes, h, w, reverse_order, stream);
     if (single_pass_applies<T>(pl))
         return LookbackByWidth<T, TI>::run(in, out, aux, planes, h, w, nb, R, reverse_order,
                                            workspace_prepared, stream);

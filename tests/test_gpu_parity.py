@@ -108,6 +108,19 @@ def test_integral_image_plane_per_workgroup(hip, switches, planes, h, w, dtype):
     assert torch.allclose(got, two_launches, rtol=2e-7, atol=0)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("planes,h,w", [(3, 28, 28), (5, 64, 128), (2, 100, 64), (4, 33, 256), (3, 64, 1024), (2, 40, 2048)])
+def test_integral_image_of_a_misaligned_tensor(hip, planes, h, w, dtype):
+    """A contiguous tensor whose first element is not 16-byte aligned (a view into a larger
+    buffer) takes the kernels' element-wise loads instead of the 16-byte ones, and small planes
+    other bands; the sums are the same."""
+    for shift in (1, 3):
+        flat = torch.randn(planes * h * w + shift, device="cuda").to(dtype)
+        x = flat[shift:].view(planes, h, w)
+        assert x.is_contiguous() and x.data_ptr() % 16 != 0
+        assert torch.allclose(hip.integral_image(x), hip.integral_image(x.clone()), rtol=2e-7, atol=0)
+
+
 INT_TYPES = [(np.uint8, torch.uint8), (np.int8, torch.int8), (np.int16, torch.int16),
              (np.int32, torch.int32), (np.int64, torch.int64)]
 
